@@ -1,0 +1,187 @@
+"""Pins the flash-attention part of the CPU oracle: reference golden vectors, torch's CPU
+scaled_dot_product_attention + autograd, scipy logsumexp, finite differences, blob bytes."""
+import os
+import struct
+
+import numpy as np
+import pytest
+import torch
+from scipy.special import logsumexp
+
+import oracle
+
+
+def load_golden(golden_dir):
+    return {n: np.load(os.path.join(golden_dir, f"fa_{n}.npy")) for n in
+            ("q", "k", "v", "dout", "out", "dq", "dk", "dv")}
+
+
+def ulp_diff_f16(a, b):
+    """distance in fp16 units-in-the-last-place (monotone integer mapping of the bits)"""
+    def key(x):
+        u = x.view(np.uint16).astype(np.int32)
+        return np.where(u & 0x8000, -(u & 0x7FFF), u)
+    return np.abs(key(a) - key(b))
+
+
+def test_golden_inputs_are_the_documented_closed_form(golden_dir):
+    # generate_flash_attn_ground_truth.py:23-25: arange(n, fp16)/30000, /40000, /50000
+    g = load_golden(golden_dir)
+    n = 128 * 3 * 32
+    ar = torch.arange(n, dtype=torch.float16)
+    for name, div in (("q", 30000), ("k", 40000), ("v", 50000)):
+        want = (ar / div).numpy().reshape(1, 128, 3, 32)
+        assert np.array_equal(g[name], want), name
+    assert np.all(g["dout"] == np.float16(1 / 32))
+
+
+def test_forward_against_reference_golden_vectors(golden_dir):
+    g = load_golden(golden_dir)
+    o, lse, _ = oracle.flash_fwd(g["q"], g["k"], g["v"], 0.5, window=(-1, 0))
+    d = ulp_diff_f16(o, g["out"])
+    # the reference test demands bit equality of its own kernel (flash_attn_fwd_test.cc:137-147);
+    # summation order inside the CUDA kernel is not reproducible on a CPU, so allow one fp16 ulp
+    assert d.max() <= 1, d.max()
+    assert (d == 0).mean() > 0.97
+    assert np.all(np.isfinite(lse))
+
+
+def test_backward_against_reference_golden_vectors(golden_dir):
+    g = load_golden(golden_dir)
+    o, lse, _ = oracle.flash_fwd(g["q"], g["k"], g["v"], 0.5, window=(-1, 0))
+    dq, dk, dv, _ = oracle.flash_bwd(g["dout"], g["q"], g["k"], g["v"], g["out"], lse, 0.5, window=(-1, 0))
+    for name, got in (("dq", dq), ("dk", dk), ("dv", dv)):
+        want = g[name].astype(np.float32)
+        err = np.abs(got.astype(np.float32) - want)
+        # <= 2 fp16 ulp of the value with an absolute floor for the exact zeros in dq's first row
+        tol = 2 * 2.0 ** -10 * np.abs(want) + 2e-6
+        assert np.all(err <= tol), (name, float((err / tol).max()))
+    # the first query row attends to one key only, so dS = P*(dP - D) = 0 there exactly
+    assert np.all(g["dq"][0, 0] == 0) and np.all(dq[0, 0] == 0)
+
+
+def torch_sdpa(q, k, v, scale, causal):
+    tq, tk, tv = (torch.tensor(t.astype(np.float32)).permute(0, 2, 1, 3).requires_grad_() for t in (q, k, v))
+    sq, sk = q.shape[1], k.shape[1]
+    mask = None
+    if causal:  # bottom-right aligned, col <= row + sk - sq (lib/mask.h:171-172)
+        i = torch.arange(sq)[:, None]
+        j = torch.arange(sk)[None, :]
+        mask = j <= i + sk - sq
+    out = torch.nn.functional.scaled_dot_product_attention(tq, tk, tv, attn_mask=mask, scale=scale)
+    return out, (tq, tk, tv)
+
+
+@pytest.mark.parametrize("causal,sq,sk", [(False, 40, 72), (True, 64, 64), (True, 33, 80)])
+def test_forward_matches_torch_sdpa_and_logsumexp(causal, sq, sk):
+    rng = np.random.default_rng(8)
+    b, h, d = 2, 3, 32
+    q = rng.standard_normal((b, sq, h, d)).astype(np.float16)
+    k = rng.standard_normal((b, sk, h, d)).astype(np.float16)
+    v = rng.standard_normal((b, sk, h, d)).astype(np.float16)
+    scale = 1 / np.sqrt(d)
+    window = (-1, 0) if causal else (-1, -1)
+    o, lse, o32 = oracle.flash_fwd(q, k, v, scale, window, round_p=False)
+    want, _ = torch_sdpa(q, k, v, scale, causal)
+    want = want.detach().permute(0, 2, 1, 3).numpy()
+    np.testing.assert_allclose(o32, want, atol=2e-5, rtol=1e-4)
+    # LSE: natural log of the sum over kept keys of exp(scale * q.k) (softmax.h:172)
+    s = np.einsum("bihd,bjhd->bhij", q.astype(np.float64), k.astype(np.float64)) * scale
+    if causal:
+        i = np.arange(sq)[:, None]
+        j = np.arange(sk)[None, :]
+        s = np.where(j <= i + sk - sq, s, -np.inf)
+    np.testing.assert_allclose(lse, logsumexp(s, axis=-1), atol=1e-4, rtol=1e-5)
+    # reconstruct O from LSE: o_i = sum_j exp(s_ij - lse_i) v_j
+    p = np.exp(s - lse[..., None].astype(np.float64))
+    rec = np.einsum("bhij,bjhd->bihd", p, v.astype(np.float64))
+    np.testing.assert_allclose(o32, rec, atol=1e-4)
+    # rounding P to fp16 (the reference's arithmetic) stays within 2e-2 of plain float attention
+    o_r, _, _ = oracle.flash_fwd(q, k, v, scale, window, round_p=True)
+    assert np.abs(o_r.astype(np.float32) - want).max() < 2e-2
+
+
+def test_fully_masked_rows_give_zero_and_inf():
+    # causal with sq > sk: rows i < sq - sk keep no key -> O = 0, LSE = +inf
+    # (flash_fwd_kernel.h:70-104, softmax.h:171-172)
+    rng = np.random.default_rng(9)
+    q = rng.standard_normal((1, 8, 1, 32)).astype(np.float16)
+    k = rng.standard_normal((1, 5, 1, 32)).astype(np.float16)
+    o, lse, _ = oracle.flash_fwd(q, k, k, 0.3, (-1, 0))
+    assert np.all(o[0, :3] == 0) and np.all(np.isposinf(lse[0, 0, :3]))
+    assert np.all(np.isfinite(lse[0, 0, 3:]))
+    # row 3 keeps exactly key 0 -> O = v_0
+    assert np.array_equal(o[0, 3, 0], k[0, 0, 0])
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_backward_matches_torch_autograd(causal):
+    rng = np.random.default_rng(10)
+    b, h, d, sq, sk = 1, 2, 32, 48, 64
+    q = rng.standard_normal((b, sq, h, d)).astype(np.float32)
+    k = rng.standard_normal((b, sk, h, d)).astype(np.float32)
+    v = rng.standard_normal((b, sk, h, d)).astype(np.float32)
+    do = rng.standard_normal((b, sq, h, d)).astype(np.float32)
+    scale = 0.2
+    window = (-1, 0) if causal else (-1, -1)
+    o, lse, _ = oracle.flash_fwd(q, k, v, scale, window, round_p=False)
+    dq, dk, dv, D = oracle.flash_bwd(do, q, k, v, o, lse, scale, window, round_p=False)
+    out, (tq, tk, tv) = torch_sdpa(q, k, v, scale, causal)
+    out.backward(torch.tensor(do).permute(0, 2, 1, 3))
+    for got, t in ((dq, tq), (dk, tk), (dv, tv)):
+        np.testing.assert_allclose(got, t.grad.permute(0, 2, 1, 3).numpy(), atol=3e-5, rtol=1e-4)
+    np.testing.assert_allclose(D, np.einsum("bihd,bihd->bhi", do, o), atol=1e-5)
+
+
+def test_backward_finite_difference():
+    rng = np.random.default_rng(11)
+    q = rng.standard_normal((1, 6, 1, 32)).astype(np.float32)
+    k = rng.standard_normal((1, 7, 1, 32)).astype(np.float32)
+    v = rng.standard_normal((1, 7, 1, 32)).astype(np.float32)
+    do = rng.standard_normal((1, 6, 1, 32)).astype(np.float32)
+    scale = 0.25
+
+    def loss(qq, kk, vv):  # float64 loss through plain numpy
+        s = np.einsum("bihd,bjhd->bhij", qq, kk) * scale
+        i = np.arange(6)[:, None]; j = np.arange(7)[None, :]
+        s = np.where(j <= i + 1, s, -np.inf)
+        p = np.exp(s - logsumexp(s, axis=-1, keepdims=True))
+        return float((np.einsum("bhij,bjhd->bihd", p, vv) * do).sum())
+
+    o, lse, _ = oracle.flash_fwd(q, k, v, scale, (-1, 0), round_p=False)
+    dq, dk, dv, _ = oracle.flash_bwd(do, q, k, v, o, lse, scale, (-1, 0), round_p=False)
+    q64, k64, v64 = (t.astype(np.float64) for t in (q, k, v))
+    eps = 1e-5
+    for arr, grad, which in ((q64, dq, 0), (k64, dk, 1), (v64, dv, 2)):
+        for idx in [(0, 0, 0, 0), (0, 3, 0, 5), (0, 5, 0, 31)]:
+            hi = [q64.copy(), k64.copy(), v64.copy()]; lo = [q64.copy(), k64.copy(), v64.copy()]
+            hi[which][idx] += eps; lo[which][idx] -= eps
+            fd = (loss(*hi) - loss(*lo)) / (2 * eps)
+            assert abs(fd - grad[idx]) < 1e-4, (which, idx, fd, grad[idx])
+
+
+def test_bf16_storage_path():
+    rng = np.random.default_rng(12)
+    b, s, h, d = 1, 64, 2, 64
+    q32, k32, v32 = (rng.standard_normal((b, s, h, d)).astype(np.float32) for _ in range(3))
+    q, k, v = (oracle.to_bf16_bits(t) for t in (q32, k32, v32))
+    o, lse, o32 = oracle.flash_fwd(q, k, v, 0.125)
+    want, _ = torch_sdpa(oracle.from_bf16_bits(q), oracle.from_bf16_bits(k), oracle.from_bf16_bits(v), 0.125, False)
+    want = want.detach().permute(0, 2, 1, 3).numpy()
+    assert np.abs(oracle.from_bf16_bits(o) - want).max() < 2e-2
+
+
+def test_extra_args_blob_known_answer():
+    # runtime/test/test_files/flash_attn_fwd.mlir:9 extra_args, packed as
+    # OpAccessor::GetAttrAsVoidPtr does (op_accessor.cc:212-242): i64 -> 8 B, f32 -> 4 B
+    fields = [12288] * 4 + [96] * 4 + [32] * 4 + [1, 3, 3, 32, 32, 0.5, 128, 128, 128, 128, 0.0, -1, 0]
+    want = b"".join(struct.pack("<f", f) if isinstance(f, float) else struct.pack("<q", f) for f in fields)
+    assert len(want) == 192
+    a = oracle.fa_args(1, 128, 128, 3, 3, 32, 0.5, window=(-1, 0))
+    blob = oracle.fa_pack_args(a)
+    assert blob.tobytes() == want
+    back = oracle.fa_unpack_args(blob)
+    assert (back.seqlen_q, back.window_size_left, back.window_size_right, back.softmax_scale) == (128, -1, 0, 0.5)
+    # BASELINE config 4 strides
+    c4 = oracle.fa_args(4, 2048, 2048, 32, 32, 128, 1 / np.sqrt(128), window=(-1, 0))
+    assert (c4.q_batch_stride, c4.q_row_stride, c4.q_head_stride) == (8388608, 4096, 128)
