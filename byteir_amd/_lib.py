@@ -1,0 +1,88 @@
+"""ctypes loaders for the in-tree shared libraries.  Loading fails loudly: there is no
+fallback path of any kind."""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_DIR = os.path.join(_HERE, "lib")
+
+F32, F16, BF16 = 0, 1, 2
+REDUCE_SUM, REDUCE_MAX = 0, 1
+
+
+class LibraryMissing(RuntimeError):
+    pass
+
+
+def lib_path(name):
+    return os.path.join(LIB_DIR, name)
+
+
+def _load(name, mode=ctypes.DEFAULT_MODE):
+    path = lib_path(name)
+    if not os.path.exists(path):
+        raise LibraryMissing(
+            f"{path} is not built; run `python -c 'import __graft_entry__ as g; g.build()'` "
+            "(hipcc --offload-arch=gfx950). There is no fallback implementation.")
+    return ctypes.CDLL(path, mode=mode)
+
+
+_kernels = None
+
+
+def kernels():
+    """libbrt_rocm_kernels.so with argtypes set from include/brt_rocm_kernels.h."""
+    global _kernels
+    if _kernels is None:
+        L = _load("libbrt_rocm_kernels.so", ctypes.RTLD_GLOBAL)
+        vp, sz, i32 = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int
+        pvp = ctypes.POINTER(ctypes.c_void_p)
+        L.brt_rocm_version.restype = ctypes.c_char_p
+        L.brt_rocm_error_string.argtypes = [i32]
+        L.brt_rocm_error_string.restype = ctypes.c_char_p
+        L.brt_rocm_device_count.argtypes = [ctypes.POINTER(i32)]
+        L.brt_rocm_set_device.argtypes = [i32]
+        L.brt_rocm_malloc.argtypes = [pvp, sz]
+        L.brt_rocm_free.argtypes = [vp]
+        L.brt_rocm_host_malloc.argtypes = [pvp, sz]
+        L.brt_rocm_host_free.argtypes = [vp]
+        for n in ("h2d", "d2h", "d2d"):
+            getattr(L, f"brt_rocm_memcpy_{n}").argtypes = [vp, vp, sz, vp]
+        L.brt_rocm_memset.argtypes = [vp, i32, sz, vp]
+        L.brt_rocm_stream_create.argtypes = [pvp]
+        L.brt_rocm_stream_destroy.argtypes = [vp]
+        L.brt_rocm_stream_synchronize.argtypes = [vp]
+        L.brt_rocm_event_create.argtypes = [pvp]
+        L.brt_rocm_event_destroy.argtypes = [vp]
+        L.brt_rocm_event_record.argtypes = [vp, vp]
+        L.brt_rocm_event_synchronize.argtypes = [vp]
+        L.brt_rocm_event_elapsed_ms.argtypes = [ctypes.POINTER(ctypes.c_float), vp, vp]
+        L.brt_rocm_reduce_workspace_bytes.argtypes = [i32, sz, sz, sz]
+        L.brt_rocm_reduce_workspace_bytes.restype = sz
+        L.brt_rocm_reduce.argtypes = [i32, i32, vp, vp, sz, sz, sz, vp, sz, vp]
+        L.brt_rocm_softmax.argtypes = [i32, vp, vp, sz, sz, vp]
+        _kernels = L
+    return _kernels
+
+
+def check(err, what=""):
+    if err != 0:
+        msg = kernels().brt_rocm_error_string(err).decode()
+        raise RuntimeError(f"{what}: HIP error {err} ({msg})")
+
+
+_flash = None
+
+
+def flash_attn():
+    """libflash_attn.so: VERSION + run_flash_attn_{fwd,bwd}[_bf16] (include/flash_api.h)."""
+    global _flash
+    if _flash is None:
+        L = _load("libflash_attn.so", ctypes.RTLD_GLOBAL)
+        vp = ctypes.c_void_p
+        for n in ("run_flash_attn_fwd", "run_flash_attn_bwd", "run_flash_attn_fwd_bf16", "run_flash_attn_bwd_bf16"):
+            f = getattr(L, n)
+            f.argtypes = [ctypes.POINTER(vp), vp, vp]
+            f.restype = None
+        _flash = L
+    return _flash

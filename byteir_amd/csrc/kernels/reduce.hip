@@ -1,0 +1,329 @@
+// Reduction kernels of the ROCm provider: out[a, c] = fold_b in[a, b, c] over a dense
+// row-major [A, B, C] view, for gfx950 (wave64).
+//
+// Two kernels cover every shape:
+//   * reduce_row_kernel  (C == 1): G lanes cooperate on one row segment with 128-bit loads,
+//     several loads in flight per lane, then a wave shuffle tree (and one LDS hop when a
+//     whole 256-thread block shares a row).
+//   * reduce_col_kernel  (C > 1): each lane owns a 128-bit group of adjacent columns, a wave
+//     spans 1 KiB of contiguous columns, the waves of a block interleave rows; partial
+//     results meet in LDS.
+// When one pass cannot fill the chip (few outputs, long fold axis) the fold axis is split in
+// S segments whose float partials go to the caller's workspace, and the same kernels run a
+// second, tiny pass over [A, S, C].  The split depends only on (dtype, A, B, C), so the
+// workspace can be sized when an execution plan is built.
+//
+// Semantics follow the reference's operators
+// (runtime/lib/backends/cuda/providers/default/reduction/kernels/reduction_helper.h:18-36,158-179):
+// sum starts from 0, max from -inf and returns NaN when either operand is NaN; f16 folds in
+// float (reduce_impl.h:64-69).
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+#include "brt_rocm_kernels.h"
+
+namespace {
+
+constexpr int kBlock = 256;            // threads per workgroup (4 waves)
+constexpr uint64_t kFillThreads = 256ull * 1024;  // threads wanted in flight chip-wide
+
+template <int OP> struct Fold;
+template <> struct Fold<BRT_ROCM_REDUCE_SUM> {
+  static __device__ __forceinline__ float init() { return 0.f; }
+  static __device__ __forceinline__ float apply(float l, float r) { return l + r; }
+};
+template <> struct Fold<BRT_ROCM_REDUCE_MAX> {
+  static __device__ __forceinline__ float init() { return -INFINITY; }
+  static __device__ __forceinline__ float apply(float l, float r) {
+    return (l != l || l > r) ? l : r;  // NaN on either side wins
+  }
+};
+
+// ---- typed loads into float -----------------------------------------------------------
+template <typename T, int VEC> struct Loader;
+template <> struct Loader<float, 4> {
+  static __device__ __forceinline__ void load(const float *p, float (&v)[4]) {
+    const float4 t = *reinterpret_cast<const float4 *>(p);
+    v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+  }
+};
+template <> struct Loader<float, 1> {
+  static __device__ __forceinline__ void load(const float *p, float (&v)[1]) { v[0] = *p; }
+};
+template <> struct Loader<__half, 8> {
+  static __device__ __forceinline__ void load(const __half *p, float (&v)[8]) {
+    const uint4 t = *reinterpret_cast<const uint4 *>(p);
+    const __half2 *h = reinterpret_cast<const __half2 *>(&t);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float2 f = __half22float2(h[i]);
+      v[2 * i] = f.x; v[2 * i + 1] = f.y;
+    }
+  }
+};
+template <> struct Loader<__half, 1> {
+  static __device__ __forceinline__ void load(const __half *p, float (&v)[1]) { v[0] = __half2float(*p); }
+};
+
+template <typename TO> __device__ __forceinline__ TO to_out(float v);
+template <> __device__ __forceinline__ float to_out<float>(float v) { return v; }
+template <> __device__ __forceinline__ __half to_out<__half>(float v) { return __float2half_rn(v); }
+
+template <int OP> __device__ __forceinline__ float wave_fold(float r, int width) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1)
+    if (off < width) r = Fold<OP>::apply(r, __shfl_xor(r, off, 64));
+  return r;
+}
+
+// ---- rows: C == 1 -----------------------------------------------------------------------
+// unit = a * S + s; G lanes fold in[a, s*seg_len : min(B, (s+1)*seg_len)] into out[unit].
+template <typename T, typename TO, int OP, int VEC, int G>
+__global__ void __launch_bounds__(kBlock)
+reduce_row_kernel(const T *__restrict__ in, TO *__restrict__ out, uint64_t units, uint64_t B,
+                  uint32_t S, uint64_t seg_len) {
+  constexpr int GPB = kBlock / G;
+  constexpr int U = 4;
+  const int lane = threadIdx.x % G;
+  uint64_t unit = (uint64_t)blockIdx.x * GPB + threadIdx.x / G;
+  const bool valid = unit < units;
+  if (!valid) unit = units - 1;  // surplus groups redo the last unit so shuffles stay whole
+  const uint64_t a = unit / S, s = unit % S;
+  const uint64_t begin = s * seg_len;
+  uint64_t end = begin + seg_len;
+  if (end > B) end = B;
+  const T *row = in + a * B;
+
+  float acc[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) acc[u] = Fold<OP>::init();
+  const uint64_t step = (uint64_t)G * VEC;
+  uint64_t i = begin + (uint64_t)lane * VEC;
+  for (; i + (U - 1) * step < end; i += U * step) {
+    float v[U][VEC];
+#pragma unroll
+    for (int u = 0; u < U; ++u) Loader<T, VEC>::load(row + i + u * step, v[u]);
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int k = 0; k < VEC; ++k) acc[u] = Fold<OP>::apply(acc[u], v[u][k]);
+  }
+  for (; i < end; i += step) {
+    float v[VEC];
+    Loader<T, VEC>::load(row + i, v);
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) acc[0] = Fold<OP>::apply(acc[0], v[k]);
+  }
+  float r = Fold<OP>::apply(Fold<OP>::apply(acc[0], acc[1]), Fold<OP>::apply(acc[2], acc[3]));
+  if constexpr (G <= 64) {
+    r = wave_fold<OP>(r, G);
+  } else {
+    static_assert(G == kBlock, "a unit is shared by lanes of one wave or by the whole block");
+    __shared__ float part[kBlock / 64];
+    r = wave_fold<OP>(r, 64);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = r;
+    __syncthreads();
+    r = Fold<OP>::apply(Fold<OP>::apply(part[0], part[1]), Fold<OP>::apply(part[2], part[3]));
+  }
+  if (valid && lane == 0) out[unit] = to_out<TO>(r);
+}
+
+// ---- columns: C > 1 ---------------------------------------------------------------------
+// block = (column tile, segment s, a); lane (tx, ty) folds rows ty, ty+TY, ... of its segment
+// for VEC adjacent columns; out[(a*S + s)*C + c].
+template <typename T, typename TO, int OP, int VEC, int TX>
+__global__ void __launch_bounds__(kBlock)
+reduce_col_kernel(const T *__restrict__ in, TO *__restrict__ out, uint64_t B, uint64_t C,
+                  uint32_t S, uint64_t seg_rows, uint32_t col_tiles) {
+  constexpr int TY = kBlock / TX;
+  constexpr int U = 8;
+  __shared__ float part[TY][TX * VEC + 1];
+  const int tx = threadIdx.x % TX, ty = threadIdx.x / TX;
+  uint64_t bid = blockIdx.x;
+  const uint32_t tile = bid % col_tiles; bid /= col_tiles;
+  const uint32_t s = bid % S;
+  const uint64_t a = bid / S;
+  const uint64_t c = ((uint64_t)tile * TX + tx) * VEC;
+  const bool col_ok = c < C;
+  const uint64_t r0 = (uint64_t)s * seg_rows;
+  uint64_t r1 = r0 + seg_rows;
+  if (r1 > B) r1 = B;
+
+  float acc[VEC];
+#pragma unroll
+  for (int k = 0; k < VEC; ++k) acc[k] = Fold<OP>::init();
+  if (col_ok) {
+    const T *p = in + a * B * C + c;
+    uint64_t r = r0 + ty;
+    for (; r + (uint64_t)(U - 1) * TY < r1; r += (uint64_t)U * TY) {
+      float v[U][VEC];
+#pragma unroll
+      for (int u = 0; u < U; ++u) Loader<T, VEC>::load(p + (r + (uint64_t)u * TY) * C, v[u]);
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) acc[k] = Fold<OP>::apply(acc[k], v[u][k]);
+    }
+    for (; r < r1; r += TY) {
+      float v[VEC];
+      Loader<T, VEC>::load(p + r * C, v);
+#pragma unroll
+      for (int k = 0; k < VEC; ++k) acc[k] = Fold<OP>::apply(acc[k], v[k]);
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < VEC; ++k) part[ty][tx * VEC + k] = acc[k];
+  __syncthreads();
+  // TX*VEC columns remain, TY partials each: lane j folds column j (coalesced store)
+  for (int j = threadIdx.x; j < TX * VEC; j += kBlock) {
+    float r = part[0][j];
+#pragma unroll 4
+    for (int y = 1; y < TY; ++y) r = Fold<OP>::apply(r, part[y][j]);
+    const uint64_t cj = (uint64_t)tile * TX * VEC + j;
+    if (cj < C) out[(a * S + s) * C + cj] = to_out<TO>(r);
+  }
+}
+
+// ---- host-side planning -------------------------------------------------------------------
+struct Plan {
+  int kind;       // 0 copy, 1 row, 2 col
+  int vec;        // elements per load when pointers are 16-byte aligned
+  int g;          // row: lanes per unit; col: TX
+  uint32_t S;     // segments of the fold axis
+  uint64_t seg;   // row: elements per segment; col: rows per segment
+  uint32_t col_tiles;
+};
+
+inline uint64_t ceil_div(uint64_t a, uint64_t b) { return (a + b - 1) / b; }
+inline uint64_t round_up(uint64_t a, uint64_t b) { return ceil_div(a, b) * b; }
+
+Plan make_plan(int dtype, uint64_t A, uint64_t B, uint64_t C, bool allow_split) {
+  Plan p{};
+  if (!(A && B && C)) { p.kind = 0; p.S = 1; return p; }
+  const int vec_full = dtype == BRT_ROCM_F32 ? 4 : 8;
+  if (C == 1) {
+    p.kind = 1;
+    p.vec = (B % vec_full == 0) ? vec_full : 1;
+    const uint64_t nvec = ceil_div(B, p.vec);
+    p.g = nvec >= 2048 ? 256 : nvec >= 96 ? 64 : nvec >= 24 ? 16 : 4;
+    uint64_t S = 1;
+    if (allow_split && A * p.g < kFillThreads) {
+      const uint64_t want = ceil_div(kFillThreads, A * p.g);
+      const uint64_t room = nvec / ((uint64_t)p.g * 8);  // keep >= 8 loads per lane per segment
+      S = want < room ? want : room;
+      if (S < 1) S = 1;
+      if (S > 1024) S = 1024;
+    }
+    p.seg = round_up(ceil_div(B, S), (uint64_t)p.g * vec_full);
+    p.S = (uint32_t)ceil_div(B, p.seg);
+    return p;
+  }
+  p.kind = 2;
+  p.vec = (C % vec_full == 0) ? vec_full : 1;
+  const uint64_t ncolv = ceil_div(C, p.vec);
+  p.g = ncolv > 32 ? 64 : ncolv > 8 ? 32 : 8;
+  const int ty = kBlock / p.g;
+  p.col_tiles = (uint32_t)ceil_div(ncolv, p.g);
+  const uint64_t blocks0 = A * p.col_tiles;
+  uint64_t S = 1;
+  if (allow_split && blocks0 < 1024 && B > (uint64_t)ty * 8) {
+    const uint64_t want = ceil_div(2048, blocks0);
+    const uint64_t room = ceil_div(B, (uint64_t)ty * 8);
+    S = want < room ? want : room;
+    if (S > 1024) S = 1024;
+  }
+  p.seg = round_up(ceil_div(B, S), ty);
+  p.S = (uint32_t)ceil_div(B, p.seg);
+  return p;
+}
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+template <typename T, typename TO, int OP>
+hipError_t launch(const Plan &p, const T *in, TO *out, uint64_t A, uint64_t B, uint64_t C,
+                  hipStream_t stream) {
+  constexpr int VF = sizeof(T) == 4 ? 4 : 8;
+  const bool vec = p.vec > 1 && aligned16(in);
+  if (p.kind == 1) {
+    const uint64_t units = A * p.S;
+    const uint64_t blocks = ceil_div(units, kBlock / p.g);
+    if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
+    const dim3 grid((unsigned)blocks), block(kBlock);
+#define ROW(G)                                                                                   \
+  if (vec) reduce_row_kernel<T, TO, OP, VF, G><<<grid, block, 0, stream>>>(in, out, units, B, p.S, p.seg); \
+  else reduce_row_kernel<T, TO, OP, 1, G><<<grid, block, 0, stream>>>(in, out, units, B, p.S, p.seg)
+    switch (p.g) {
+    case 4: ROW(4); break;
+    case 16: ROW(16); break;
+    case 64: ROW(64); break;
+    default: ROW(256); break;
+    }
+#undef ROW
+    return hipGetLastError();
+  }
+  const uint64_t blocks = A * p.S * p.col_tiles;
+  if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
+  const dim3 grid((unsigned)blocks), block(kBlock);
+#define COL(TX)                                                                                  \
+  if (vec) reduce_col_kernel<T, TO, OP, VF, TX><<<grid, block, 0, stream>>>(in, out, B, C, p.S, p.seg, p.col_tiles); \
+  else reduce_col_kernel<T, TO, OP, 1, TX><<<grid, block, 0, stream>>>(in, out, B, C, p.S, p.seg, p.col_tiles)
+  switch (p.g) {
+  case 8: COL(8); break;
+  case 32: COL(32); break;
+  default: COL(64); break;
+  }
+#undef COL
+  return hipGetLastError();
+}
+
+template <typename T, int OP>
+hipError_t run(const T *in, T *out, uint64_t A, uint64_t B, uint64_t C, void *ws, size_t ws_bytes,
+               int dtype, hipStream_t stream) {
+  const Plan p = make_plan(dtype, A, B, C, true);
+  if (p.S == 1) return launch<T, T, OP>(p, in, out, A, B, C, stream);
+  const size_t need = sizeof(float) * A * p.S * C;
+  if (ws == nullptr || ws_bytes < need) return hipErrorInvalidValue;
+  float *part = static_cast<float *>(ws);
+  hipError_t e = launch<T, float, OP>(p, in, part, A, B, C, stream);
+  if (e != hipSuccess) return e;
+  const Plan p2 = make_plan(BRT_ROCM_F32, A, p.S, C, false);
+  return launch<float, T, OP>(p2, part, out, A, p.S, C, stream);
+}
+
+}  // namespace
+
+extern "C" size_t brt_rocm_reduce_workspace_bytes(int dtype, size_t A, size_t B, size_t C) {
+  if (dtype != BRT_ROCM_F32 && dtype != BRT_ROCM_F16) return 0;
+  const Plan p = make_plan(dtype, A, B, C, true);
+  return p.S > 1 ? sizeof(float) * A * p.S * C : 0;
+}
+
+extern "C" int brt_rocm_reduce(int op, int dtype, const void *input, void *output, size_t A,
+                               size_t B, size_t C, void *workspace, size_t workspace_bytes,
+                               void *stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  if ((op != BRT_ROCM_REDUCE_SUM && op != BRT_ROCM_REDUCE_MAX) ||
+      (dtype != BRT_ROCM_F32 && dtype != BRT_ROCM_F16))
+    return hipErrorInvalidValue;
+  const size_t es = dtype == BRT_ROCM_F32 ? 4 : 2;
+  if (!(A && B && C)) {  // nothing to fold: copy C elements (reduce_impl.h:71-74)
+    if (C == 0) return hipSuccess;
+    if (!input || !output) return hipErrorInvalidValue;
+    return hipMemcpyAsync(output, input, C * es, hipMemcpyDeviceToDevice, stream);
+  }
+  if (!input || !output) return hipErrorInvalidValue;
+  if (dtype == BRT_ROCM_F32) {
+    const float *in = static_cast<const float *>(input);
+    float *out = static_cast<float *>(output);
+    return op == BRT_ROCM_REDUCE_SUM
+               ? run<float, BRT_ROCM_REDUCE_SUM>(in, out, A, B, C, workspace, workspace_bytes, dtype, stream)
+               : run<float, BRT_ROCM_REDUCE_MAX>(in, out, A, B, C, workspace, workspace_bytes, dtype, stream);
+  }
+  const __half *in = static_cast<const __half *>(input);
+  __half *out = static_cast<__half *>(output);
+  return op == BRT_ROCM_REDUCE_SUM
+             ? run<__half, BRT_ROCM_REDUCE_SUM>(in, out, A, B, C, workspace, workspace_bytes, dtype, stream)
+             : run<__half, BRT_ROCM_REDUCE_MAX>(in, out, A, B, C, workspace, workspace_bytes, dtype, stream);
+}

@@ -1,0 +1,150 @@
+"""Direct calls into the kernel C ABI with torch tensors as device memory.
+
+torch is used for allocation and streams only; every computation below is a hand-written
+HIP kernel reached through libbrt_rocm_kernels.so / libflash_attn.so.  Shapes follow the
+reference's op kernels: reductions take the canonical [A, B, C] view computed by
+`canonicalize_reduce` (ReduceImpl, runtime/lib/backends/cuda/providers/default/reduction/reduce_impl.h:28-59).
+"""
+import ctypes
+import struct
+
+import torch
+
+from . import _lib
+
+_DT = {torch.float32: _lib.F32, torch.float16: _lib.F16, torch.bfloat16: _lib.BF16}
+
+
+def _stream(stream=None):
+    s = stream if stream is not None else torch.cuda.current_stream()
+    return ctypes.c_void_p(s.cuda_stream)
+
+
+def _dev(t):
+    if not t.is_cuda:
+        raise ValueError("device tensor required: the ROCm provider has no host path")
+    if not t.is_contiguous():
+        raise ValueError("dense row-major tensor required")
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def deduce_output_shape(shape, dims):
+    """reduction::DeduceOutputShape, runtime/lib/core/common/utils/math_helper.cc:145-159."""
+    for d in dims:
+        if not 0 <= d < len(shape):
+            raise ValueError("invalid dimension")
+    return [s for i, s in enumerate(shape) if i not in dims]
+
+
+def canonicalize_reduce(in_shape, out_shape, dims):
+    """ReduceImpl's constructor: -> (A, B, C); raises ValueError where the reference throws."""
+    if list(out_shape) != deduce_output_shape(in_shape, dims):
+        raise ValueError("output shape does not match the deduced shape")
+    live = sorted(d for d in dims if in_shape[d] != 1)
+    if not live:
+        n = 1
+        for s in in_shape:
+            n *= s
+        return 0, 0, n
+    if any(b - a != 1 for a, b in zip(live, live[1:])):
+        raise ValueError("Only consecutive dimensions reduction is supported")
+    A = B = C = 1
+    for s in in_shape[:live[0]]:
+        A *= s
+    for d in live:
+        B *= in_shape[d]
+    for s in in_shape[live[-1] + 1:]:
+        C *= s
+    return A, B, C
+
+
+def reduce_workspace_bytes(dtype, A, B, C):
+    return _lib.kernels().brt_rocm_reduce_workspace_bytes(_DT[dtype], A, B, C)
+
+
+def reduce_abc(op, x, out, A, B, C, workspace=None, stream=None):
+    """Enqueue out[a,c] = fold_b x[a,b,c]; `workspace` is a uint8 device tensor of at least
+    reduce_workspace_bytes(...) bytes (allocated here when omitted)."""
+    K = _lib.kernels()
+    need = K.brt_rocm_reduce_workspace_bytes(_DT[x.dtype], A, B, C)
+    if need and workspace is None:
+        workspace = torch.empty(need, dtype=torch.uint8, device=x.device)
+    ws_ptr = ctypes.c_void_p(workspace.data_ptr()) if workspace is not None else None
+    ws_len = workspace.numel() * workspace.element_size() if workspace is not None else 0
+    _lib.check(K.brt_rocm_reduce(op, _DT[x.dtype], _dev(x), _dev(out), A, B, C, ws_ptr, ws_len,
+                                 _stream(stream)), "brt_rocm_reduce")
+    return out
+
+
+def reduce(op, x, dims, stream=None):
+    """ReduceSumOp / ReduceMaxOp over `dims` of a dense tensor (op: _lib.REDUCE_SUM / REDUCE_MAX)."""
+    out_shape = deduce_output_shape(list(x.shape), list(dims))
+    A, B, C = canonicalize_reduce(list(x.shape), out_shape, list(dims))
+    out = torch.empty(out_shape, dtype=x.dtype, device=x.device)
+    return reduce_abc(op, x, out, A, B, C, stream=stream)
+
+
+def softmax(x, out=None, stream=None):
+    """byteir.softmax over the last axis."""
+    if out is None:
+        out = torch.empty_like(x)
+    cols = x.shape[-1]
+    rows = x.numel() // cols if cols else 0
+    _lib.check(_lib.kernels().brt_rocm_softmax(_DT[x.dtype], _dev(x), _dev(out), rows, cols,
+                                               _stream(stream)), "brt_rocm_softmax")
+    return out
+
+
+# ---- flash attention through the custom-library ABI ---------------------------------------
+def round_up(x, m):
+    return (x + m - 1) // m * m
+
+
+def pack_flash_args(q, k, v, o, scale, window, p_dropout=0.0):
+    """The 192-byte extra_args blob for [b, s, h, d] tensors: 17 i64, f32, 4 i64, f32, 2 i64,
+    unpadded (OpAccessor::GetAttrAsVoidPtr, runtime/lib/core/framework/op_accessor.cc:212-242;
+    field order compiler/lib/Conversion/HloToByreTensor/HloToByreCustom.cpp:149-176)."""
+    b, sq, h, d = q.shape
+    sk, h_k = k.shape[1], k.shape[2]
+    ints1 = [q.stride(0), k.stride(0), v.stride(0), o.stride(0),
+             q.stride(1), k.stride(1), v.stride(1), o.stride(1),
+             q.stride(2), k.stride(2), v.stride(2), o.stride(2),
+             b, h, h_k, d, round_up(d, 32)]
+    ints2 = [sq, sk, round_up(sq, 128), round_up(sk, 128)]
+    return (struct.pack("<17q", *ints1) + struct.pack("<f", scale) + struct.pack("<4q", *ints2)
+            + struct.pack("<f", p_dropout) + struct.pack("<2q", *window))
+
+
+def _call_custom(fn, tensors, blob, stream):
+    arr = (ctypes.c_void_p * len(tensors))(*[t.data_ptr() if t is not None else None for t in tensors])
+    buf = ctypes.create_string_buffer(blob, len(blob))
+    fn(arr, ctypes.cast(buf, ctypes.c_void_p), _stream(stream))
+
+
+def flash_attn_fwd(q, k, v, scale, window=(-1, -1), stream=None):
+    """run_flash_attn_fwd: tensors {q, k, v, rng_state, o, softmax_lse, softmax_P}
+    (external_libs/runtime/flash_attn/lib/flash_api.cu:586-654). -> (o, lse[b,h,sq] f32)."""
+    L = _lib.flash_attn()
+    b, sq, h, d = q.shape
+    o = torch.empty_like(q)
+    lse = torch.empty((b, h, sq), dtype=torch.float32, device=q.device)
+    rng = torch.zeros(2, dtype=torch.int64, device=q.device)
+    fn = L.run_flash_attn_fwd if q.dtype == torch.float16 else L.run_flash_attn_fwd_bf16
+    _call_custom(fn, [q, k, v, rng, o, lse, None], pack_flash_args(q, k, v, o, scale, window), stream)
+    return o, lse
+
+
+def flash_attn_bwd(dout, q, k, v, o, lse, scale, window=(-1, -1), stream=None):
+    """run_flash_attn_bwd: tensors {dout, q, k, v, out, softmax_lse, rng_state, dq, dk, dv,
+    d_softmax, dq_accum} (flash_api.cu:656-725). -> (dq, dk, dv)."""
+    L = _lib.flash_attn()
+    b, sq, h, d = q.shape
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    sq_r, d_r = round_up(sq, 128), round_up(d, 32)
+    dsm = torch.empty((b, h, sq_r), dtype=torch.float32, device=q.device)
+    dq_accum = torch.empty((b, sq_r, h, d_r), dtype=torch.float32, device=q.device)
+    rng = torch.zeros(2, dtype=torch.int64, device=q.device)
+    fn = L.run_flash_attn_bwd if q.dtype == torch.float16 else L.run_flash_attn_bwd_bf16
+    _call_custom(fn, [dout, q, k, v, o, lse, rng, dq, dk, dv, dsm, dq_accum],
+                 pack_flash_args(q, k, v, o, scale, window), stream)
+    return dq, dk, dv

@@ -1,0 +1,95 @@
+/*
+ * brt_rocm_kernels.h -- C ABI of libbrt_rocm_kernels.so, the device layer of the ROCm
+ * execution provider: plain pointers and sizes, no C++ or framework types.
+ *
+ * Host code (the provider's op kernels, written in C++, or any FFI) reaches HIP only
+ * through these entry points.  Every function returns a hipError_t value as int
+ * (0 == success) unless stated otherwise; kernels are enqueued on `stream`
+ * (a hipStream_t passed as void*, NULL = the default stream) and never synchronise.
+ *
+ * Citations name the interface of the reference (bytedance/byteir, paths relative to its
+ * checkout) that each entry point stands in for.
+ */
+#ifndef BRT_ROCM_KERNELS_H_
+#define BRT_ROCM_KERNELS_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* element types (the subset of brt::DTypeEnum, runtime/include/brt/core/framework/dtype.h,
+ * that the op kernels on this path accept) */
+enum { BRT_ROCM_F32 = 0, BRT_ROCM_F16 = 1, BRT_ROCM_BF16 = 2 };
+/* fold operators: kernel::reduction::SumOp / MaxOp,
+ * runtime/lib/backends/cuda/providers/default/reduction/kernels/reduction_helper.h:18-36,140-179 */
+enum { BRT_ROCM_REDUCE_SUM = 0, BRT_ROCM_REDUCE_MAX = 1 };
+
+/* library identification; returns a static string */
+const char *brt_rocm_version(void);
+/* hipGetErrorString for the int codes returned below */
+const char *brt_rocm_error_string(int err);
+
+/* ---- device plumbing ------------------------------------------------------------- */
+/* Stand-ins for the CUDA runtime calls made by the reference's device layer:
+ * allocator  runtime/lib/backends/cuda/device/cuda_allocator.cc:36-86 (cudaMalloc/cudaFree,
+ *            cudaMallocHost/cudaFreeHost),
+ * work queue runtime/lib/backends/cuda/device/cuda_work_queue.cc:139-177 (stream create /
+ *            destroy / synchronize),
+ * device API runtime/lib/backends/cuda/device/cuda_device_api.cc:29-55 (memcpy H2D/D2H/D2D,
+ *            memset, set device). */
+int brt_rocm_device_count(int *count);
+int brt_rocm_set_device(int device_id);
+int brt_rocm_malloc(void **ptr, size_t bytes);
+int brt_rocm_free(void *ptr);
+int brt_rocm_host_malloc(void **ptr, size_t bytes); /* pinned host memory */
+int brt_rocm_host_free(void *ptr);
+/* copies are asynchronous on `stream`; with pageable host memory HIP stages them */
+int brt_rocm_memcpy_h2d(void *dst, const void *src, size_t bytes, void *stream);
+int brt_rocm_memcpy_d2h(void *dst, const void *src, size_t bytes, void *stream);
+int brt_rocm_memcpy_d2d(void *dst, const void *src, size_t bytes, void *stream);
+int brt_rocm_memset(void *dst, int value, size_t bytes, void *stream);
+int brt_rocm_stream_create(void **stream);
+int brt_rocm_stream_destroy(void *stream);
+int brt_rocm_stream_synchronize(void *stream);
+int brt_rocm_device_synchronize(void);
+/* events, for timing a launch on the stream it runs on */
+int brt_rocm_event_create(void **event);
+int brt_rocm_event_destroy(void *event);
+int brt_rocm_event_record(void *event, void *stream);
+int brt_rocm_event_synchronize(void *event);
+int brt_rocm_event_elapsed_ms(float *ms, void *start, void *stop);
+
+/* ---- reductions ------------------------------------------------------------------ */
+/* out[a, c] = fold_b in[a, b, c] for a dense row-major tensor viewed as [A, B, C];
+ * f16 is folded in float.  Stands in for
+ *   kernel::call_reduce<T, Op>(input, output, A, B, C, workspace, stream)
+ * (runtime/lib/backends/cuda/providers/default/reduction/kernels/reduction.h:13-15,
+ *  reduction.cu:415-426), and
+ *   kernel::get_reduce_workspace_in_bytes<T>(A, B, C)          (reduction.h:17-18,
+ *  reduction.cu:428-434).
+ * A == 0 or B == 0 means "nothing to fold": C elements are copied device to device, as
+ * ReduceImpl::Execute does (reduce_impl.h:61-75).
+ * The workspace holds float partials of the split first pass; its size depends only on
+ * (dtype, A, B, C), so it can be queried once when an execution plan is built.  A NULL or
+ * too small workspace is an error (hipErrorInvalidValue) when the size is non-zero.
+ * dtype: BRT_ROCM_F32 or BRT_ROCM_F16.  Max propagates NaN from either operand. */
+size_t brt_rocm_reduce_workspace_bytes(int dtype, size_t A, size_t B, size_t C);
+int brt_rocm_reduce(int op, int dtype, const void *input, void *output, size_t A, size_t B,
+                    size_t C, void *workspace, size_t workspace_bytes, void *stream);
+
+/* ---- fused row softmax ----------------------------------------------------------- */
+/* y[r, :] = exp(x[r, :] - max_j x[r, j]) / sum_j exp(...) over the last axis of a dense
+ * [rows, cols] tensor; float internals for every storage type, one rounding at the store.
+ * The reference runtime has no softmax kernel; the arithmetic contract is the compiler's
+ * linalg_ext.softmax lowering (compiler/lib/Conversion/ToLinalg/LinalgExtToLinalg.cpp:286-410).
+ * dtype: BRT_ROCM_F32, BRT_ROCM_F16 or BRT_ROCM_BF16.  In-place (output == input) is allowed. */
+int brt_rocm_softmax(int dtype, const void *input, void *output, size_t rows, size_t cols,
+                     void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BRT_ROCM_KERNELS_H_ */
