@@ -1,0 +1,76 @@
+"""Builds the in-tree shared libraries with hipcc for gfx950 (no GPU needed to compile).
+
+    python -m byteir_amd.build            # build everything
+    python -m byteir_amd.build kernels    # one target
+
+Targets:
+  kernels -> lib/libbrt_rocm_kernels.so   reductions, softmax, device plumbing (C ABI)
+  flash   -> lib/libflash_attn.so         flash-attention custom library (C ABI)
+  brt     -> lib/libbrt.so                BRT-shaped C++ host runtime (g++, no HIP headers)
+"""
+import os
+import subprocess
+import sys
+import time
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+CSRC = os.path.join(HERE, "csrc")
+LIB = os.path.join(HERE, "lib")
+INC = os.path.join(ROOT, "include")
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+# -packed-fp32-ops is switched off on purpose: the compiler must not form v_pk_*_f32.
+HIP_FLAGS = ["-O3", "-std=c++17", "--offload-arch=gfx950", "-fPIC", "-shared",
+             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+             "-Wno-unused-command-line-argument", f"-I{INC}"]
+CXX_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", f"-I{INC}"]
+
+
+def _glob(sub, exts):
+    d = os.path.join(CSRC, sub)
+    return sorted(os.path.join(d, f) for f in os.listdir(d) if f.endswith(exts))
+
+
+def _run(cmd, verbose):
+    t = time.time()
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(l for l in r.stdout.splitlines() if "packed-fp32-ops" not in l)
+    if r.returncode != 0:
+        raise RuntimeError("build failed: " + " ".join(cmd) + "\n" + out)
+    if verbose:
+        print(f"[build] {os.path.basename(cmd[cmd.index('-o') + 1])} in {time.time() - t:.1f}s")
+        if out.strip():
+            print(out)
+
+
+def build_kernels(verbose=False):
+    os.makedirs(LIB, exist_ok=True)
+    _run([HIPCC] + HIP_FLAGS + ["-o", os.path.join(LIB, "libbrt_rocm_kernels.so")] + _glob("kernels", (".hip",)), verbose)
+
+
+def build_flash(verbose=False):
+    os.makedirs(LIB, exist_ok=True)
+    _run([HIPCC] + HIP_FLAGS + [f"-I{os.path.join(CSRC, 'flash_attn')}", "-o", os.path.join(LIB, "libflash_attn.so")]
+         + _glob("flash_attn", (".hip",)), verbose)
+
+
+def build_brt(verbose=False):
+    os.makedirs(LIB, exist_ok=True)
+    srcs = _glob("brt", (".cc",))
+    if not srcs:
+        return
+    _run(["g++"] + CXX_FLAGS + [f"-I{os.path.join(CSRC, 'brt')}", "-o", os.path.join(LIB, "libbrt.so")] + srcs
+         + [f"-L{LIB}", "-lbrt_rocm_kernels", "-ldl", "-Wl,-rpath,$ORIGIN"], verbose)
+
+
+TARGETS = {"kernels": build_kernels, "flash": build_flash, "brt": build_brt}
+
+
+def build_all(verbose=False, targets=None):
+    for name in targets or ("kernels", "flash", "brt"):
+        TARGETS[name](verbose)
+
+
+if __name__ == "__main__":
+    build_all(verbose=True, targets=sys.argv[1:] or None)

@@ -1,0 +1,161 @@
+// C entry points of libflash_attn.so (see include/flash_api.h): blob parsing, validation,
+// kernel dispatch.  Counterpart of the reference's run_flash_attn_fwd / run_flash_attn_bwd
+// (external_libs/runtime/flash_attn/lib/flash_api.cu:586-725) and run_mha / run_mha_bwd
+// (:228-432) for the ROCm provider.
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+
+#include "flash_api.h"
+#include "flash_common.h"
+
+namespace fa {
+hipError_t launch_fwd(Params &p, int dtype, hipStream_t stream);
+hipError_t launch_bwd(Params &p, int dtype, hipStream_t stream);
+}  // namespace fa
+
+namespace {
+
+thread_local char g_err[256] = "";
+
+int fail(const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return -1;
+}
+
+struct Blob {
+  int64_t q_bs, k_bs, v_bs, o_bs, q_rs, k_rs, v_rs, o_rs, q_hs, k_hs, v_hs, o_hs;
+  int64_t b, h, h_k, d, d_rounded;
+  float softmax_scale;
+  int64_t seqlen_q, seqlen_k, seqlen_q_rounded, seqlen_k_rounded;
+  float p_dropout;
+  int64_t window_size_left, window_size_right;
+};
+
+// The blob is unpadded: every i64 after the first float is 4-byte misaligned.
+Blob parse(const void *extra_args) {
+  const unsigned char *s = static_cast<const unsigned char *>(extra_args);
+  size_t pos = 0;
+  auto i64 = [&]() { int64_t v; memcpy(&v, s + pos, 8); pos += 8; return v; };
+  auto f32 = [&]() { float v; memcpy(&v, s + pos, 4); pos += 4; return v; };
+  Blob a;
+  a.q_bs = i64(); a.k_bs = i64(); a.v_bs = i64(); a.o_bs = i64();
+  a.q_rs = i64(); a.k_rs = i64(); a.v_rs = i64(); a.o_rs = i64();
+  a.q_hs = i64(); a.k_hs = i64(); a.v_hs = i64(); a.o_hs = i64();
+  a.b = i64(); a.h = i64(); a.h_k = i64(); a.d = i64(); a.d_rounded = i64();
+  a.softmax_scale = f32();
+  a.seqlen_q = i64(); a.seqlen_k = i64(); a.seqlen_q_rounded = i64(); a.seqlen_k_rounded = i64();
+  a.p_dropout = f32();
+  // the reference reads the windows through uint32_t and passes them on as int
+  // (flash_api.cu:621-624,652-653); -1 survives the round trip
+  a.window_size_left = (int32_t)(uint32_t)i64();
+  a.window_size_right = (int32_t)(uint32_t)i64();
+  return a;
+}
+
+bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+int fill(const Blob &a, fa::Params &p) {
+  if (a.b < 0 || a.h <= 0 || a.h_k <= 0 || a.seqlen_q < 0 || a.seqlen_k < 0)
+    return fail("negative or zero dimension (b=%ld h=%ld h_k=%ld sq=%ld sk=%ld)", (long)a.b,
+                (long)a.h, (long)a.h_k, (long)a.seqlen_q, (long)a.seqlen_k);
+  if (a.d != 32 && a.d != 64 && a.d != 128)
+    return fail("head_dim %ld is not supported (32, 64 or 128)", (long)a.d);
+  if (a.h % a.h_k != 0) return fail("h (%ld) must be a multiple of h_k (%ld)", (long)a.h, (long)a.h_k);
+  if (a.p_dropout != 0.f) return fail("p_dropout %g is not supported (0 only)", a.p_dropout);
+  const int64_t strides[] = {a.q_bs, a.k_bs, a.v_bs, a.o_bs, a.q_rs, a.k_rs,
+                             a.v_rs, a.o_rs, a.q_hs, a.k_hs, a.v_hs, a.o_hs};
+  for (int64_t s : strides)
+    if (s % 8 != 0) return fail("stride %ld is not a multiple of 8 elements (16-byte rows needed)", (long)s);
+  if (a.seqlen_q > (1 << 30) || a.seqlen_k > (1 << 30) || a.b * a.h > (1 << 24))
+    return fail("problem too large for 32-bit tile indices");
+  p.q_bs = a.q_bs; p.k_bs = a.k_bs; p.v_bs = a.v_bs; p.o_bs = a.o_bs;
+  p.q_rs = a.q_rs; p.k_rs = a.k_rs; p.v_rs = a.v_rs; p.o_rs = a.o_rs;
+  p.q_hs = a.q_hs; p.k_hs = a.k_hs; p.v_hs = a.v_hs; p.o_hs = a.o_hs;
+  p.b = (int)a.b; p.h = (int)a.h; p.h_k = (int)a.h_k; p.d = (int)a.d;
+  p.sq = (int)a.seqlen_q; p.sk = (int)a.seqlen_k;
+  p.sq_rounded = (int)a.seqlen_q_rounded;
+  p.scale = a.softmax_scale;
+  p.scale_log2 = (float)(a.softmax_scale * M_LOG2E);  // flash_api.cu:289
+  // run_mha turns a one-sided window into seqlen_k on the open side (flash_api.cu:300-309);
+  // "unbounded" (< 0) is the same thing
+  p.wl = a.window_size_left < 0 ? -1 : (int)a.window_size_left;
+  p.wr = a.window_size_right < 0 ? -1 : (int)a.window_size_right;
+  return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *VERSION = "2.5.3";
+
+const char *flash_attn_last_error(void) { return g_err; }
+
+int flash_attn_fwd_checked(void **tensors, const void *extra_args, int dtype, void *stream) {
+  if (!tensors || !extra_args) return fail("null argument");
+  if (dtype != 1 && dtype != 2) return fail("dtype %d is not supported (1 = fp16, 2 = bf16)", dtype);
+  const Blob a = parse(extra_args);
+  fa::Params p{};
+  if (int r = fill(a, p)) return r;
+  // tensors: q, k, v, rng_state, o, softmax_lse, softmax_P
+  p.q = tensors[0]; p.k = tensors[1]; p.v = tensors[2];
+  p.o_w = tensors[4];
+  p.lse = static_cast<float *>(tensors[5]);
+  if (p.b == 0 || p.sq == 0) return 0;
+  if (!p.q || !p.o_w || !p.lse || (p.sk > 0 && (!p.k || !p.v))) return fail("null tensor pointer");
+  if (!aligned16(p.q) || !aligned16(p.k) || !aligned16(p.v) || !aligned16(p.o_w))
+    return fail("q, k, v and o must be 16-byte aligned");
+  return fa::launch_fwd(p, dtype, static_cast<hipStream_t>(stream));
+}
+
+int flash_attn_bwd_checked(void **tensors, const void *extra_args, int dtype, void *stream) {
+  if (!tensors || !extra_args) return fail("null argument");
+  if (dtype != 1 && dtype != 2) return fail("dtype %d is not supported (1 = fp16, 2 = bf16)", dtype);
+  const Blob a = parse(extra_args);
+  fa::Params p{};
+  if (int r = fill(a, p)) return r;
+  if (a.h != a.h_k) return fail("backward needs h == h_k (got %ld, %ld)", (long)a.h, (long)a.h_k);
+  if (a.seqlen_q_rounded < a.seqlen_q) return fail("seqlen_q_rounded < seqlen_q");
+  // tensors: dout, q, k, v, out, softmax_lse, rng_state, dq, dk, dv, d_softmax, dq_accum
+  p.dout = tensors[0]; p.q = tensors[1]; p.k = tensors[2]; p.v = tensors[3]; p.o = tensors[4];
+  p.lse = static_cast<float *>(tensors[5]);
+  p.dq = tensors[7]; p.dk = tensors[8]; p.dv = tensors[9];
+  p.dsoftmax = static_cast<float *>(tensors[10]);
+  if (p.b == 0) return 0;
+  const void *need[] = {p.dout, p.q, p.k, p.v, p.o, p.dq, p.dk, p.dv};
+  for (const void *t : need) {
+    if (!t) return fail("null tensor pointer");
+    if (!aligned16(t)) return fail("tensors must be 16-byte aligned");
+  }
+  if (!p.lse || !p.dsoftmax) return fail("null tensor pointer");
+  return fa::launch_bwd(p, dtype, static_cast<hipStream_t>(stream));
+}
+
+static void die(const char *who, int r) {
+  if (r < 0) fprintf(stderr, "libflash_attn: %s: unsupported arguments: %s\n", who, g_err);
+  else fprintf(stderr, "libflash_attn: %s: %s\n", who, hipGetErrorString(static_cast<hipError_t>(r)));
+  abort();
+}
+
+void run_flash_attn_fwd(void **tensors, void *extra_args, void *stream) {
+  if (int r = flash_attn_fwd_checked(tensors, extra_args, 1, stream)) die("run_flash_attn_fwd", r);
+}
+void run_flash_attn_bwd(void **tensors, void *extra_args, void *stream) {
+  if (int r = flash_attn_bwd_checked(tensors, extra_args, 1, stream)) die("run_flash_attn_bwd", r);
+}
+void run_flash_attn_fwd_bf16(void **tensors, void *extra_args, void *stream) {
+  if (int r = flash_attn_fwd_checked(tensors, extra_args, 2, stream)) die("run_flash_attn_fwd_bf16", r);
+}
+void run_flash_attn_bwd_bf16(void **tensors, void *extra_args, void *stream) {
+  if (int r = flash_attn_bwd_checked(tensors, extra_args, 2, stream)) die("run_flash_attn_bwd_bf16", r);
+}
+
+}  // extern "C"

@@ -1,0 +1,129 @@
+// Shared building blocks of the gfx950 flash-attention kernels: element traits, MFMA
+// wrappers, LDS helpers and the kernel parameter block.
+//
+// Register layouts used throughout (wave64, lane l, r = l % 32, g = l / 32):
+//   v_mfma_f32_32x32x16_{f16,bf16}:  A[32 x 16]: lane holds A[r][8g .. 8g+7]
+//                                     B[16 x 32]: lane holds B[8g .. 8g+7][r]
+//                                     C[32 x 32]: lane holds C[8*(i/4) + 4g + i%4][r], i = 0..15
+// so a C tile keeps one matrix *column* per lane.  All score tiles are therefore computed
+// with the query index on the column axis where per-query statistics (running max, sum, LSE,
+// D) must be lane-local, and a C tile feeds the next MFMA as its B operand without moving
+// between lanes: B slot (g, j) of 16-row window w is C register 8w + j, i.e. matrix row
+// 16w + 8*(j/4) + 4g + j%4.  The other operand is fetched with the same row permutation.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+namespace fa {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef short short4v __attribute__((ext_vector_type(4)));
+typedef short short8v __attribute__((ext_vector_type(8)));
+typedef float float16v __attribute__((ext_vector_type(16)));
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+template <typename T> struct Traits;
+template <> struct Traits<_Float16> {
+  using vec8 = half8;
+  static __device__ __forceinline__ float16v mfma(vec8 a, vec8 b, float16v c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+};
+template <> struct Traits<__bf16> {
+  using vec8 = bf16x8;
+  static __device__ __forceinline__ float16v mfma(vec8 a, vec8 b, float16v c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+};
+
+// 8 floats -> 8 storage elements, round to nearest even
+template <typename T>
+__device__ __forceinline__ typename Traits<T>::vec8 pack8(const float *f) {
+  typename Traits<T>::vec8 v;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) v[j] = (T)f[j];
+  return v;
+}
+
+__device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float log2_fast(float x) { return __builtin_amdgcn_logf(x); }
+
+// value of the partner lane (l ^ 32)
+__device__ __forceinline__ float partner32(float v) {
+  const unsigned u = __builtin_bit_cast(unsigned, v);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  // lanes < 32 receive (own, partner); lanes >= 32 receive (partner, own)
+  const unsigned other = (threadIdx.x & 32) ? r[0] : r[1];
+  return __builtin_bit_cast(float, other);
+}
+
+// 128-bit LDS read of 8 consecutive elements
+template <typename T>
+__device__ __forceinline__ typename Traits<T>::vec8 lds_read8(const T *p) {
+  return *reinterpret_cast<const typename Traits<T>::vec8 *>(p);
+}
+
+// Transposing LDS read (ds_read_b64_tr_b16).  Within each group of 16 lanes, lane i passes
+// the address of 4 consecutive elements: lanes 4r..4r+3 together name row r (16 elements) of
+// a 4 x 16 block; lane i receives column i of that block (4 elements, rows 0..3).
+template <typename T> __device__ __forceinline__ short4v lds_read_tr4(const T *p) {
+  return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+      (__attribute__((address_space(3))) short4v *)(p));
+}
+
+// An MFMA A (or B) operand taken "down the rows" of a row-major LDS tile: the lane ends up
+// with tile[row0 + perm(g, j)][col0 + r], j = 0..7, where perm(g, j) = 8*(j/4) + 4g + j%4 is
+// the row order a C tile presents to the next MFMA.  `stride` in elements.
+template <typename T>
+__device__ __forceinline__ typename Traits<T>::vec8 lds_read_operand_tr(const T *tile, int stride,
+                                                                         int row0, int col0) {
+  const int lane = threadIdx.x & 63;
+  const int i16 = lane & 15, b16 = lane >> 4;
+  const int gg = b16 >> 1;
+  const T *p = tile + (row0 + gg * 4 + (i16 >> 2)) * stride + col0 + (b16 & 1) * 16 + (i16 & 3) * 4;
+  const short4v lo = lds_read_tr4(p);
+  const short4v hi = lds_read_tr4(p + 8 * stride);
+  short8v v;
+  v.s0 = lo.s0; v.s1 = lo.s1; v.s2 = lo.s2; v.s3 = lo.s3;
+  v.s4 = hi.s0; v.s5 = hi.s1; v.s6 = hi.s2; v.s7 = hi.s3;
+  return __builtin_bit_cast(typename Traits<T>::vec8, v);
+}
+
+// LDS row strides (elements).  Rows read with plain 128-bit loads (32 rows x 16 B at a time)
+// want a stride of 4*odd banks; rows read with the transposing load (4 rows x 64 B per
+// half-wave) want a stride of 16 (mod 64) banks.
+template <int D> struct Pad {
+  static constexpr int kPlain = D + 8;
+  static constexpr int kTr = D == 32 ? 32 : D + 32;
+};
+
+struct Params {
+  const void *q, *k, *v, *o, *dout;  // o is written by forward, read by backward
+  void *o_w;                          // forward output
+  float *lse;                         // [b, h, sq]
+  void *dq, *dk, *dv;
+  float *dsoftmax;                    // [b, h, sq_rounded]
+  int64_t q_bs, k_bs, v_bs, o_bs;     // batch strides (elements)
+  int64_t q_rs, k_rs, v_rs, o_rs;     // row strides
+  int64_t q_hs, k_hs, v_hs, o_hs;     // head strides
+  int b, h, h_k, d;
+  int sq, sk, sq_rounded;
+  float scale, scale_log2;
+  int wl, wr;                         // window sizes after normalisation; < 0 = unbounded
+  int n_mblocks, n_nblocks;
+  int xcd_remap;                      // 1: blocks of one (batch, head) share an XCD
+};
+
+// Kept key range [lo, hi) for query row `q` (reference: lib/mask.h:160-200).
+__device__ __forceinline__ void row_limits(const Params &p, int q, int &lo, int &hi) {
+  lo = 0; hi = p.sk;
+  const int off = p.sk - p.sq;
+  if (p.wr >= 0) hi = min(p.sk, q + 1 + off + p.wr);
+  if (p.wl >= 0) lo = max(0, q + off - p.wl);
+}
+
+}  // namespace fa

@@ -1,0 +1,66 @@
+/*
+ * flash_api.h -- C ABI of libflash_attn.so, the MI355X drop-in for the flash-attention
+ * custom library that ByRE's `custom` op kernel dlopen()s.
+ *
+ * The caller is CustomOpKernel::RunImpl (reference:
+ * runtime/lib/backends/cuda/providers/default/custom/custom.cc:69-86):
+ *     run_func_(tensor_args, extra_args, stream);
+ * where tensor_args[i] is the device pointer of operand i, extra_args is a malloc'ed,
+ * unpadded blob built from the op's `extra_args` array attribute (i64 -> 8 bytes,
+ * f32 -> 4 bytes; runtime/lib/core/framework/op_accessor.cc:212-242) and stream is the work
+ * queue's compute stream.  The custom op also requires a data symbol named VERSION
+ * (custom.cc:50-53).
+ *
+ * These declarations replace external_libs/runtime/flash_attn/include/flash_api.h:75-82 of
+ * the reference.  Streams are hipStream_t passed as void*.
+ *
+ * extra_args layout (192 bytes; compiler/lib/Conversion/HloToByreTensor/HloToByreCustom.cpp:149-176,
+ * parsed at external_libs/runtime/flash_attn/lib/flash_api.cu:586-624):
+ *   i64 q,k,v,o batch_stride; i64 q,k,v,o row_stride; i64 q,k,v,o head_stride  (elements)
+ *   i64 b, h, h_k, d, d_rounded; f32 softmax_scale;
+ *   i64 seqlen_q, seqlen_k, seqlen_q_rounded, seqlen_k_rounded; f32 p_dropout;
+ *   i64 window_size_left, window_size_right      (causal = (-1, 0), full = (-1, -1))
+ * Tensors are [batch, seqlen, heads, head_dim] with a contiguous head_dim; softmax_lse is
+ * [batch, heads, seqlen_q] float.
+ *
+ * Supported here: head_dim 32, 64 or 128, p_dropout == 0, any seqlen, h % h_k == 0
+ * (backward: h == h_k).  Anything else is reported on stderr and the process aborts, since
+ * the ABI has no error channel; the *_checked variants return an error code instead.
+ */
+#ifndef BYTEIR_AMD_FLASH_API_H_
+#define BYTEIR_AMD_FLASH_API_H_
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Must be a pointer variable, as in the reference (flash_api.cu:7-9). */
+extern const char *VERSION;
+
+/* tensors: {q, k, v, rng_state, o, softmax_lse, softmax_P}  (flash_api.cu:626-654).
+ * fp16 storage.  rng_state and softmax_P are accepted and never touched (p_dropout == 0). */
+void run_flash_attn_fwd(void **tensors, void *extra_args, void *stream);
+
+/* tensors: {dout, q, k, v, out, softmax_lse, rng_state, dq, dk, dv, d_softmax, dq_accum}
+ * (flash_api.cu:696-725).  fp16 storage.  d_softmax is [b, h, seqlen_q_rounded] float scratch
+ * that receives rowsum(dout * out); dq_accum is accepted and left untouched (dQ is
+ * accumulated without atomics by a pass that is parallel over query blocks). */
+void run_flash_attn_bwd(void **tensors, void *extra_args, void *stream);
+
+/* The same two entry points for bfloat16 storage.  The reference library is fp16 only
+ * (params.is_bf16 = 0, flash_api.cu:295,421) and its blob carries no dtype field, so the
+ * element type is selected by the op's `api_name` attribute. */
+void run_flash_attn_fwd_bf16(void **tensors, void *extra_args, void *stream);
+void run_flash_attn_bwd_bf16(void **tensors, void *extra_args, void *stream);
+
+/* Error-returning forms of the four calls above: 0 on success, a positive hipError_t when a
+ * launch failed, -1 when the arguments are unsupported (reason copied to a thread-local
+ * buffer readable through flash_attn_last_error()).  dtype: 1 = fp16, 2 = bf16. */
+int flash_attn_fwd_checked(void **tensors, const void *extra_args, int dtype, void *stream);
+int flash_attn_bwd_checked(void **tensors, const void *extra_args, int dtype, void *stream);
+const char *flash_attn_last_error(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BYTEIR_AMD_FLASH_API_H_ */
