@@ -49,6 +49,7 @@ def kernels():
         for n in ("h2d", "d2h", "d2d"):
             getattr(L, f"brt_rocm_memcpy_{n}").argtypes = [vp, vp, sz, vp]
         L.brt_rocm_memset.argtypes = [vp, i32, sz, vp]
+        L.brt_rocm_copy_kernel.argtypes = [vp, vp, sz, vp]
         L.brt_rocm_stream_create.argtypes = [pvp]
         L.brt_rocm_stream_destroy.argtypes = [vp]
         L.brt_rocm_stream_synchronize.argtypes = [vp]
@@ -86,3 +87,62 @@ def flash_attn():
             f.restype = None
         _flash = L
     return _flash
+
+
+ALLOC_FN = ctypes.CFUNCTYPE(ctypes.c_void_p, ctypes.c_size_t)
+FREE_FN = ctypes.CFUNCTYPE(None, ctypes.c_void_p)
+OP_LISTENER = ctypes.CFUNCTYPE(None, ctypes.c_void_p, ctypes.c_char_p, ctypes.c_int, ctypes.c_int)
+
+_brt = None
+
+
+def brt():
+    """libbrt.so with argtypes set from include/brt_c_api.h."""
+    global _brt
+    if _brt is None:
+        kernels()  # libbrt.so links against the kernel library
+        L = _load("libbrt.so", ctypes.RTLD_GLOBAL)
+        vp, sz, i32, cp = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_char_p
+        L.brt_last_error.restype = cp
+        L.brt_session_create.argtypes = [i32, ALLOC_FN, FREE_FN]
+        L.brt_session_create.restype = vp
+        L.brt_session_destroy.argtypes = [vp]
+        L.brt_session_destroy.restype = None
+        L.brt_session_load.argtypes = [vp, cp]
+        L.brt_session_load_text.argtypes = [vp, cp]
+        L.brt_register_kernels_from_dynlib.argtypes = [cp]
+        L.brt_session_has_kernel.argtypes = [vp, cp]
+        L.brt_session_arg_num.argtypes = [vp]
+        L.brt_session_arg_num.restype = sz
+        L.brt_session_arg_offset.argtypes = [vp, cp]
+        L.brt_session_arg_name.argtypes = [vp, sz]
+        L.brt_session_arg_name.restype = cp
+        L.brt_session_arg_kind.argtypes = [vp, sz]
+        L.brt_session_arg_rank.argtypes = [vp, sz]
+        L.brt_session_arg_rank.restype = sz
+        L.brt_session_arg_shape.argtypes = [vp, sz, ctypes.POINTER(ctypes.c_int64)]
+        L.brt_session_arg_shape.restype = None
+        L.brt_session_arg_dtype.argtypes = [vp, sz]
+        L.brt_session_arg_dtype.restype = cp
+        L.brt_session_arg_space.argtypes = [vp, sz]
+        L.brt_session_arg_space.restype = cp
+        L.brt_session_op_num.argtypes = [vp]
+        L.brt_session_op_num.restype = sz
+        L.brt_session_op_key.argtypes = [vp, sz]
+        L.brt_session_op_key.restype = cp
+        L.brt_session_op_attr_blob.argtypes = [vp, sz, cp, vp, sz]
+        L.brt_session_op_attr_blob.restype = ctypes.c_long
+        L.brt_request_create.argtypes = [vp, vp, i32]
+        L.brt_request_create.restype = vp
+        L.brt_request_destroy.argtypes = [vp]
+        L.brt_request_destroy.restype = None
+        L.brt_request_bind_arg.argtypes = [vp, sz, vp]
+        L.brt_request_get_arg.argtypes = [vp, sz]
+        L.brt_request_get_arg.restype = vp
+        L.brt_request_finish_io_binding.argtypes = [vp]
+        L.brt_request_sync.argtypes = [vp]
+        L.brt_session_run.argtypes = [vp, vp]
+        L.brt_request_add_op_listener.argtypes = [vp, OP_LISTENER, vp]
+        L.brt_request_add_op_listener.restype = None
+        _brt = L
+    return _brt

@@ -1,0 +1,399 @@
+// brt.h -- a compact, MLIR-free host runtime with the shape of ByteIR's BRT, sized to the
+// op-kernel hot path: a ByRE text reader, the kernel registry, execution providers, op kernels
+// with per-frame workspaces, allocators, work queues, sessions and request contexts.
+//
+// Names and call protocol follow the reference so that provider code reads the same
+// (paths relative to the reference checkout, runtime/include/brt/core/...):
+//   common::Status                       common/status.h:29-181
+//   IAllocator                           framework/allocator.h:49-62
+//   WorkQueue                            context/work_queue.h:48-89
+//   OpKernelInfo / OpAccessor            framework/op_kernel_info.h:53-68, op_accessor.h:36-97
+//   OpKernel                             framework/op_kernel.h:69-178
+//   KernelRegistry + static registration framework/kernel_registry.h:28-94
+//   ExecutionProvider                    framework/execution_provider.h:41-115
+//   ExecutionContext / ExecutionFrame    context/execution_context.h:36-50, execution_frame.h
+//   Session / RequestContext             session/session.h:50-146, request_context.h:44-92
+// This host code includes no HIP header: devices are reached through the C ABI of
+// libbrt_rocm_kernels.so (include/brt_rocm_kernels.h).
+#pragma once
+
+#include <cstdint>
+#include <functional>
+#include <map>
+#include <memory>
+#include <stdexcept>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+namespace brt {
+
+// ---- status and errors ------------------------------------------------------------------
+namespace common {
+class Status {
+public:
+  Status() = default;  // OK
+  static Status OK() { return Status(); }
+  static Status Fail(const std::string &msg) { Status s; s.ok_ = false; s.msg_ = msg; return s; }
+  bool IsOK() const { return ok_; }
+  const std::string &ErrorMessage() const { return msg_; }
+
+private:
+  bool ok_ = true;
+  std::string msg_;
+};
+}  // namespace common
+
+class BrtException : public std::runtime_error {
+public:
+  using std::runtime_error::runtime_error;
+};
+[[noreturn]] void Throw(const char *file, int line, const std::string &msg);
+#define BRT_THROW(msg) ::brt::Throw(__FILE__, __LINE__, (msg))
+#define BRT_ENFORCE(cond, ...)                                                         \
+  do {                                                                                 \
+    if (!(cond)) ::brt::Throw(__FILE__, __LINE__, std::string(#cond " was false. ") + std::string(__VA_ARGS__)); \
+  } while (0)
+
+// ---- element types -----------------------------------------------------------------------
+enum class DTypeEnum { Invalid = 0, Float32, Float16, BFloat16, Float64, Int8, Int16, Int32, Int64, UInt8, Bool };
+size_t GetDTypeByte(DTypeEnum t);
+const char *GetDTypeName(DTypeEnum t);
+using Shape = std::vector<int64_t>;
+int64_t LinearizedShape(const Shape &shape);
+
+namespace reduction {
+// dims dropped from src_shape; throws on an out-of-range dimension
+Shape DeduceOutputShape(const Shape &src_shape, const std::vector<int64_t> &dimensions);
+}
+
+// ---- ByRE IR (text) ------------------------------------------------------------------------
+namespace ir {
+
+struct MemRefType {
+  Shape shape;
+  DTypeEnum dtype = DTypeEnum::Invalid;
+  std::string space;  // memory-space string, selects the allocator ("cuda", "cpu", ...)
+  size_t Bytes() const { return (size_t)LinearizedShape(shape) * GetDTypeByte(dtype); }
+};
+
+struct Scalar {  // one element of an array attribute
+  bool is_float = false;
+  int64_t i = 0;
+  double f = 0.0;
+};
+
+struct Attr {
+  enum Kind { Unit, Int, Float, String, Bool, Array, DenseInt, DenseFloat } kind = Unit;
+  int64_t i = 0;
+  double f = 0.0;
+  bool b = false;
+  std::string s;
+  std::vector<Scalar> elems;  // Array / DenseInt / DenseFloat
+};
+
+enum ArgType { kInput = 1, kOutput = 2, kWeight = 4 };  // byre.argtype bits
+
+struct Value {
+  std::string name;   // SSA name including '%'
+  MemRefType type;
+  int arg_index = -1;      // position in the entry function signature, or -1
+  int alias_of = -1;       // value id this one aliases (byre.alias), or -1
+  int64_t alias_offset = 0;  // in elements of the aliased value's type
+  bool is_alloc = false;   // produced by memref.alloc
+};
+
+struct Op {
+  std::string name;             // "byre.compute", "byre.custom", ...
+  std::string key;              // callee symbol == kernel registry key
+  std::vector<int> operands;    // value ids
+  std::map<std::string, Attr> attrs;
+  int line = 0;
+};
+
+struct EntryArg {
+  int value = -1;
+  std::string argname;  // byre.argname
+  int argtype = 0;      // byre.argtype
+};
+
+// Parsed module: one entry function (the reference also assumes one, ir.cc:222).
+class ByREHandle {
+public:
+  common::Status LoadFromFile(const std::string &path);
+  common::Status LoadFromText(const std::string &text);
+
+  std::string entry_name;
+  std::vector<Value> values;
+  std::vector<EntryArg> args;
+  std::vector<Op> ops;  // compute/custom ops in program order (alias/alloc are folded into values)
+  std::map<std::string, Attr> func_attrs;
+};
+
+}  // namespace ir
+
+// ---- allocators ----------------------------------------------------------------------------
+constexpr size_t kAllocAlignment = 256;
+
+class IAllocator {
+public:
+  explicit IAllocator(std::string key) : key_(std::move(key)) {}
+  virtual ~IAllocator() = default;
+  virtual void *Alloc(size_t size) = 0;
+  virtual void Free(void *p) = 0;
+  const std::string &Key() const { return key_; }  // matched against the memref memory space
+
+private:
+  std::string key_;
+};
+
+// ---- work queues -----------------------------------------------------------------------------
+class WorkQueue {
+public:
+  explicit WorkQueue(std::string name) : name_(std::move(name)) {}
+  virtual ~WorkQueue() = default;
+  const std::string &name() const { return name_; }
+  virtual common::Status Sync() = 0;
+  // device queues expose the stream kernels are enqueued on (void* == hipStream_t)
+  virtual void *GetComputeStream() { return nullptr; }
+
+private:
+  std::string name_;
+};
+
+// ---- events ----------------------------------------------------------------------------------
+class OpKernelInfo;
+struct OpRunEvent {
+  const OpKernelInfo *info;
+  bool after;  // false: BeforeOpKernelRun, true: AfterOpKernelRun
+};
+using OpRunListener = std::function<void(const OpRunEvent &)>;
+
+// ---- execution frame / context -----------------------------------------------------------------
+class Session;
+class ExecutionFrame {
+public:
+  // device pointer of a value id (entry argument, intermediate or alias)
+  void *GetAsyncValue(int value_id) const;
+  // per-frame state owned by op kernels (workspaces), keyed by op index
+  void *GetState(int op_index) const;
+  void SetState(int op_index, void *p);
+
+private:
+  friend class Session;
+  friend class RequestContext;
+  std::vector<void *> base_;        // per value: bound/allocated pointer (aliases resolved lazily)
+  std::vector<bool> owned_;         // allocated by the frame
+  std::vector<void *> state_;       // per op
+  const ir::ByREHandle *ir_ = nullptr;
+  bool prologue_done_ = false;
+  bool io_bound_ = false;
+};
+
+struct ExecutionContext {
+  ExecutionFrame *exec_frame;
+  WorkQueue *work_queue;
+  std::vector<OpRunListener> *listeners;
+};
+
+// ---- op kernels --------------------------------------------------------------------------------
+class ExecutionProvider;
+
+class OpKernelInfo {
+public:
+  OpKernelInfo(const ExecutionProvider &provider, const ir::ByREHandle &ir, int op_index,
+               const std::unordered_map<std::string, std::unique_ptr<IAllocator>> &allocators)
+      : provider_(provider), ir_(ir), op_index_(op_index), allocators_(allocators) {}
+  const ExecutionProvider &GetExecutionProvider() const { return provider_; }
+  const ir::ByREHandle &GetIR() const { return ir_; }
+  const ir::Op &GetOp() const { return ir_.ops[op_index_]; }
+  int GetOpId() const { return op_index_; }
+  IAllocator *GetAllocator(const std::string &space) const;
+
+private:
+  const ExecutionProvider &provider_;
+  const ir::ByREHandle &ir_;
+  int op_index_;
+  const std::unordered_map<std::string, std::unique_ptr<IAllocator>> &allocators_;
+};
+
+// Reads operands and attributes of one op; the only window op kernels have on the IR.
+class OpAccessor {
+public:
+  explicit OpAccessor(const OpKernelInfo &info, ExecutionFrame *frame = nullptr) : info_(info), frame_(frame) {}
+  size_t GetNumArgs() const;
+  Shape GetArgShape(size_t i) const;
+  DTypeEnum GetArgDTypeEnum(size_t i) const;
+  std::string GetArgSpace(size_t i) const;
+  bool HasAttr(const std::string &name) const;
+  bool GetAttrAsBool(const std::string &name) const;
+  int64_t GetAttrAsInt(const std::string &name) const;
+  float GetAttrAsFloat(const std::string &name) const;
+  std::string GetAttrAsString(const std::string &name) const;
+  std::vector<int64_t> GetAttrAsIntArray(const std::string &name) const;
+  // malloc'ed, unpadded blob: i64 -> 8 bytes, f32 -> 4 bytes; caller frees
+  void *GetAttrAsVoidPtr(const std::string &name, size_t *size = nullptr) const;
+  std::string GetUID() const;
+  static int64_t GetNumElementsOfShape(const Shape &shape) { return LinearizedShape(shape); }
+  // needs a frame
+  void *GetArgAsyncValueRef(size_t i) const;
+
+private:
+  const ir::Attr &Find(const std::string &name) const;
+  const OpKernelInfo &info_;
+  ExecutionFrame *frame_;
+};
+
+class OpKernel {
+public:
+  explicit OpKernel(const OpKernelInfo &info) : info_(info) {}
+  virtual ~OpKernel() = default;
+  // enqueue on ctx.work_queue; never synchronises
+  virtual common::Status RunImpl(const ExecutionContext &ctx) = 0;
+  // once per frame before its first run / when the frame is destroyed (workspace life cycle)
+  virtual common::Status ProloguePerFrame(const ExecutionContext &) { return common::Status::OK(); }
+  virtual common::Status EpiloguePerFrame(const ExecutionContext &) { return common::Status::OK(); }
+  common::Status Run(const ExecutionContext &ctx);  // listeners + RunImpl
+  const OpKernelInfo &GetOpKernelInfo() const { return info_; }
+
+protected:
+  OpKernelInfo info_;
+};
+
+using KernelCreateFn = std::function<std::shared_ptr<OpKernel>(const OpKernelInfo &)>;
+
+class KernelRegistry {
+public:
+  common::Status Register(const std::string &key, KernelCreateFn fn) {
+    map_.emplace(key, std::move(fn));
+    return common::Status::OK();
+  }
+  bool HasKernel(const std::string &key) const { return map_.count(key) != 0; }
+  std::shared_ptr<OpKernel> operator()(const std::string &key, const OpKernelInfo &info) const {
+    auto it = map_.find(key);
+    return it == map_.end() ? nullptr : it->second(info);
+  }
+  std::vector<std::string> Keys() const;
+
+private:
+  std::unordered_map<std::string, KernelCreateFn> map_;
+};
+
+using KernelRegistration = std::function<void(KernelRegistry *)>;
+void AddKernelRegistration(const std::string &device_kind, const std::string &provider_name, KernelRegistration fn);
+void RegisterKernels(const std::string &device_kind, const std::string &provider_name, KernelRegistry *registry);
+
+#define BRT_STATIC_KERNEL_REGISTRATION(KIND, PROVIDER, FUNC) BRT_STATIC_KERNEL_REGISTRATION_1(KIND, PROVIDER, FUNC, __COUNTER__)
+#define BRT_STATIC_KERNEL_REGISTRATION_1(KIND, PROVIDER, FUNC, N) BRT_STATIC_KERNEL_REGISTRATION_2(KIND, PROVIDER, FUNC, N)
+#define BRT_STATIC_KERNEL_REGISTRATION_2(KIND, PROVIDER, FUNC, N) \
+  [[gnu::unused]] static bool brt_kernel_registration_##N = [] {  \
+    ::brt::AddKernelRegistration(KIND, PROVIDER, FUNC);           \
+    return true;                                                  \
+  }();
+
+namespace DeviceKind {
+constexpr const char *CPU = "CPU";
+constexpr const char *CUDA = "CUDA";
+constexpr const char *ROCM = "ROCM";
+}  // namespace DeviceKind
+namespace ProviderType {
+constexpr const char *BRT = "BRT";
+}
+
+class ExecutionProvider {
+public:
+  ExecutionProvider(const std::string &device_kind, const std::string &name);
+  virtual ~ExecutionProvider() = default;
+  KernelRegistry *GetKernelRegistry() const { return registry_.get(); }
+  const std::string &DeviceKindName() const { return device_kind_; }
+  const std::string &Type() const { return name_; }
+  // dlopen a shared library whose static initialisers call AddKernelRegistration; must run
+  // before the providers that should see those kernels are constructed
+  static common::Status StaticRegisterKernelsFromDynlib(const std::string &path);
+
+private:
+  std::string device_kind_, name_;
+  std::unique_ptr<KernelRegistry> registry_;
+};
+
+// ---- session / request context --------------------------------------------------------------------
+enum class BrtOwnershipType { OwnedByExternal, OwnedByRuntime };
+
+class RequestContext {
+public:
+  ~RequestContext();
+  common::Status BindArg(size_t offset, const void *value, BrtOwnershipType own = BrtOwnershipType::OwnedByExternal);
+  void *GetArg(size_t offset);
+  void FinishIOBinding();
+  common::Status Sync();
+  void AddOpRunListener(OpRunListener l) { listeners_.push_back(std::move(l)); }
+  ExecutionFrame *GetExecutionFrame() { return frame_.get(); }
+  WorkQueue *GetWorkQueue() { return wq_.get(); }
+
+private:
+  friend class Session;
+  explicit RequestContext(Session &s) : session_(s) {}
+  Session &session_;
+  std::unique_ptr<ExecutionFrame> frame_;
+  std::unique_ptr<WorkQueue> wq_;
+  std::vector<OpRunListener> listeners_;
+};
+
+class Session {
+public:
+  Session();
+  ~Session();
+  common::Status AddExecutionProvider(std::unique_ptr<ExecutionProvider> provider);
+  common::Status AddAllocator(std::unique_ptr<IAllocator> allocator);
+  IAllocator *GetAllocator(const std::string &key);
+
+  common::Status Load(const std::string &url, const std::string &fmt);         // fmt: "byre"
+  common::Status LoadFromMemory(const std::string &text, const std::string &fmt);
+  // the request context takes ownership of work_queue; without one, the first provider's
+  // default queue is created
+  common::Status NewRequestContext(std::unique_ptr<RequestContext> *request, WorkQueue *work_queue = nullptr);
+  common::Status Run(RequestContext &request);
+  void Cleanup(RequestContext &request) noexcept;
+
+  size_t GetArgNum() const;
+  int GetGraphArgOffset(const std::string &name) const;
+  const std::vector<size_t> &GetInputArgOffsets() const { return in_offsets_; }
+  const std::vector<size_t> &GetOutputArgOffsets() const { return out_offsets_; }
+  const std::vector<size_t> &GetWeightArgOffsets() const { return weight_offsets_; }
+  std::string GetArgName(size_t offset) const;
+  Shape GetStaticShape(size_t offset) const;
+  DTypeEnum GetDType(size_t offset) const;
+  std::string GetSpace(size_t offset) const;
+  size_t GetOpNum() const { return kernels_.size(); }
+  const std::string &GetOpKey(size_t i) const { return ir_->ops[i].key; }
+  const OpKernelInfo *GetOpKernelInfo(size_t i) const { return i < infos_.size() ? infos_[i].get() : nullptr; }
+  // default work-queue factory, set by the device layer (the reference hard-wires CUDA here,
+  // runtime/lib/core/framework/execution_plan.cc:592-601)
+  void SetWorkQueueFactory(std::function<WorkQueue *()> f) { wq_factory_ = std::move(f); }
+
+private:
+  friend class RequestContext;
+  common::Status BuildPlan();
+  std::vector<std::unique_ptr<ExecutionProvider>> providers_;
+  std::unordered_map<std::string, std::unique_ptr<IAllocator>> allocators_;
+  std::unique_ptr<ir::ByREHandle> ir_;
+  std::vector<std::shared_ptr<OpKernel>> kernels_;
+  std::vector<std::unique_ptr<OpKernelInfo>> infos_;
+  std::vector<size_t> in_offsets_, out_offsets_, weight_offsets_;
+  std::function<WorkQueue *()> wq_factory_;
+};
+
+// ---- ROCm device layer (rocm_provider.cc) ------------------------------------------------------------
+// Allocators answering to the memory spaces "cuda" (so existing ByRE modules run unchanged) and
+// "cpu"; work queues on an owned or a caller-supplied HIP stream; the provider itself.
+using ExternalAllocFn = void *(*)(size_t);
+using ExternalFreeFn = void (*)(void *);
+std::unique_ptr<IAllocator> MakeRocmAllocator(const std::string &key = "cuda");
+std::unique_ptr<IAllocator> MakeExternalAllocator(const std::string &key, ExternalAllocFn a, ExternalFreeFn f);
+std::unique_ptr<IAllocator> MakeHostAllocator(const std::string &key = "cpu");
+WorkQueue *MakeRocmSingleStreamWorkQueue(int device_id);
+WorkQueue *MakeRocmExternalStreamWorkQueue(void *stream);
+common::Status DefaultROCMExecutionProviderFactory(Session *session, int device_id = 0);
+common::Status ROCMAllocatorFactory(Session *session, int device_id = 0);
+
+}  // namespace brt

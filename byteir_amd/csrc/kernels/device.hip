@@ -3,9 +3,32 @@
 // headers and reaches the runtime only through these calls.
 #include <hip/hip_runtime.h>
 
+#include <cstdint>
+
 #include "brt_rocm_kernels.h"
 
+namespace {
+// grid-stride 128-bit copy; n16 = number of 16-byte words
+__global__ void __launch_bounds__(256) copy16_kernel(uint4 *__restrict__ dst, const uint4 *__restrict__ src, size_t n16) {
+  size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * 256;
+  for (; i < n16; i += stride) dst[i] = src[i];
+}
+}  // namespace
+
 extern "C" {
+
+int brt_rocm_copy_kernel(void *dst, const void *src, size_t bytes, void *stream) {
+  if (bytes % 16 != 0 || ((reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src)) & 15u))
+    return hipErrorInvalidValue;
+  const size_t n16 = bytes / 16;
+  if (n16 == 0) return hipSuccess;
+  size_t blocks = (n16 + 255) / 256;
+  if (blocks > 256 * 32) blocks = 256 * 32;
+  copy16_kernel<<<dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(
+      static_cast<uint4 *>(dst), static_cast<const uint4 *>(src), n16);
+  return hipGetLastError();
+}
 
 const char *brt_rocm_version(void) { return "byteir-amd 0.1 (gfx950)"; }
 const char *brt_rocm_error_string(int err) { return hipGetErrorString(static_cast<hipError_t>(err)); }

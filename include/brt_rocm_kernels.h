@@ -51,6 +51,11 @@ int brt_rocm_memcpy_h2d(void *dst, const void *src, size_t bytes, void *stream);
 int brt_rocm_memcpy_d2h(void *dst, const void *src, size_t bytes, void *stream);
 int brt_rocm_memcpy_d2d(void *dst, const void *src, size_t bytes, void *stream);
 int brt_rocm_memset(void *dst, int value, size_t bytes, void *stream);
+/* device-to-device copy done by a plain compute kernel (128-bit loads and stores) rather than
+ * a DMA engine: the cuda2cuda copy of runtime/lib/backends/cuda/providers/default/copy/copy.cc
+ * for buffers that are multiples of 16 bytes and 16-byte aligned, and the known-traffic
+ * reference launch against which hardware byte counters are scaled. */
+int brt_rocm_copy_kernel(void *dst, const void *src, size_t bytes, void *stream);
 int brt_rocm_stream_create(void **stream);
 int brt_rocm_stream_destroy(void *stream);
 int brt_rocm_stream_synchronize(void *stream);

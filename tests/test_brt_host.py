@@ -1,0 +1,189 @@
+"""Host logic of the BRT-shaped runtime, on a plan-only session (no GPU): the ByRE text reader,
+the kernel registry, plan-time checks of the op kernels, the extra_args blob, and the export
+lists of the three C ABI libraries."""
+import os
+import re
+import struct
+
+import pytest
+
+from byre_text import memref, reduction_module, softmax_module
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture()
+def session():
+    from byteir_amd import brt
+    s = brt.Session(device_id=-1)
+    yield s
+    s.close()
+
+
+def exported_functions(header):
+    text = open(os.path.join(ROOT, "include", header)).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    text = re.sub(r"typedef[^;]*;", "", text)
+    names = re.findall(r"\b([a-z][a-zA-Z0-9_]*)\s*\([^;{]*\)\s*;", text)
+    return sorted(set(n for n in names if not n.endswith("_fn") and n != "brt_op_listener"))
+
+
+@pytest.mark.parametrize("header,loader", [("brt_rocm_kernels.h", "kernels"), ("flash_api.h", "flash_attn"), ("brt_c_api.h", "brt")])
+def test_c_abi_exports_every_declared_symbol(header, loader):
+    from byteir_amd import _lib
+    L = getattr(_lib, loader)()
+    names = exported_functions(header)
+    assert len(names) >= 4
+    for n in names:
+        assert hasattr(L, n), f"{header}: {n} is not exported"
+    if header == "flash_api.h":
+        import ctypes
+        ver = ctypes.c_char_p.in_dll(L, "VERSION")  # a pointer variable, as in the reference
+        assert ver.value == b"2.5.3"
+
+
+def test_reference_flash_attn_modules_load_unchanged(session, golden_dir):
+    # runtime/test/test_files/flash_attn_fwd.mlir, byte for byte
+    session.load(os.path.join(golden_dir, "flash_attn_fwd.mlir"))
+    assert session.get_arg_num() == 7
+    assert session.get_op_keys() == ["custom"]
+    assert [session.get_arg_name(i) for i in range(7)] == ["Q", "K", "V", "Out", "SoftmaxLse", "SoftmaxPtr", "RngState"]
+    assert session.get_static_shape(0) == [1, 128, 3, 32] and session.get_data_type(0) == "float16"
+    assert session.get_static_shape(4) == [1, 3, 128] and session.get_data_type(4) == "float32"
+    assert session.get_static_shape(6) == [2] and session.get_data_type(6) == "int64"
+    assert session.get_space(0) == "cuda"
+    assert session.get_output_arg_offsets() == list(range(7))  # every arg carries byre.argtype = 2
+    # the blob handed to the library: 17 i64, f32, 4 i64, f32, 2 i64, unpadded
+    fields = [12288] * 4 + [96] * 4 + [32] * 4 + [1, 3, 3, 32, 32, 0.5, 128, 128, 128, 128, 0.0, -1, 0]
+    want = b"".join(struct.pack("<f", f) if isinstance(f, float) else struct.pack("<q", f) for f in fields)
+    assert session.get_op_attr_blob(0, "extra_args") == want
+    session.load(os.path.join(golden_dir, "flash_attn_bwd.mlir"))
+    assert session.get_op_keys() == ["custom", "custom"] and session.get_arg_num() == 13
+    assert session.get_graph_arg_offset("d_Q") == 6 and session.get_graph_arg_offset("nope") == -1
+
+
+def test_reader_accepts_the_compiler_s_attribute_forms(session):
+    # dense<[..]>, splat dense<1> : tensor<1xi64>, unsorted dims, ArrayAttr, rank-0 memref,
+    # memref.alloc and byre.alias (runtime/test/test_files/resnet18_fw_bw_host_cuda.mlir:59,178,185,300)
+    text = """
+module attributes {byre.container_module} {
+  func.func @main(%arg0: memref<4x1000xf32, "cuda"> {byre.argname = "in", byre.argtype = 1 : i32},
+                  %arg1: memref<f32, "cuda"> {byre.argname = "out0", byre.argtype = 2 : i32},
+                  %arg2: memref<4xf32, "cuda"> {byre.argname = "out1", byre.argtype = 2 : i32},
+                  %arg3: memref<2x3x8x5xf32, "cuda"> {byre.argname = "in2", byre.argtype = 1 : i32},
+                  %arg4: memref<2x3xf32, "cuda"> {byre.argname = "out2", byre.argtype = 2 : i32}) attributes {byre.entry_point, device_file_name = "x.ptx"} {
+    // intermediates
+    %alloc = memref.alloc() : memref<1024xi8, "cuda">
+    %0 = "byre.alias"(%alloc) {device = "cuda", offset = 256 : i64} : (memref<1024xi8, "cuda">) -> memref<4xf32, "cuda">
+    byre.compute @ReduceSumOp_f32_f32(%arg0, %arg1) {device = "cuda", dimensions = dense<[0, 1]> : tensor<2xi64>, memory_effects = [1 : i32, 2 : i32]} : memref<4x1000xf32, "cuda">, memref<f32, "cuda">
+    byre.compute @ReduceMaxOp_f32_f32(%arg0, %0) {dimensions = dense<1> : tensor<1xi64>} : memref<4x1000xf32, "cuda">, memref<4xf32, "cuda">
+    byre.compute @ReduceSumOp_f32_f32(%arg0, %arg2) {dimensions = [1 : i64]} : memref<4x1000xf32, "cuda">, memref<4xf32, "cuda">
+    byre.compute @ReduceSumOp_f32_f32(%arg3, %arg4) {dimensions = dense<[3, 2]> : tensor<2xi64>} : memref<2x3x8x5xf32, "cuda">, memref<2x3xf32, "cuda">
+    return
+  }
+}
+"""
+    session.load_from_memory(text)
+    assert session.get_op_keys() == ["ReduceSumOp_f32_f32", "ReduceMaxOp_f32_f32", "ReduceSumOp_f32_f32", "ReduceSumOp_f32_f32"]
+    assert session.get_static_shape(1) == [] and session.get_input_arg_offsets() == [0, 3]
+    req = session.new_request_context()
+    req.finish_io_binding()  # allocates args and the memref.alloc intermediate (host memory here)
+    assert req.get_arg(0) != 0
+    with pytest.raises(RuntimeError, match="without a device"):
+        req.run()
+
+
+def test_registry_has_the_reference_keys(session):
+    for key in ("ReduceSumOp_f32_f32", "ReduceSumOp_f16_f16", "ReduceMaxOp_f32_f32", "ReduceMaxOp_f16_f16",
+                "custom", "byteir.softmax", "cpu2cuda", "cuda2cpu", "cuda2cuda"):
+        assert session.has_kernel(key), key
+    assert not session.has_kernel("MatmulOp_f32f32_f32")
+
+
+def test_unknown_op_fails_at_load(session):
+    # execution_plan.cc:435-438: "No providers support Op <key>"
+    text = reduction_module("cuda", [4, 8], [1], "ReduceProdOp_f32_f32")
+    with pytest.raises(RuntimeError, match="No providers support Op ReduceProdOp_f32_f32"):
+        session.load_from_memory(text)
+
+
+def test_unknown_memory_space_fails_at_load(session):
+    with pytest.raises(RuntimeError, match="no allocator for memory space"):
+        session.load_from_memory(reduction_module("tpu", [4, 8], [1], "ReduceSumOp_f32_f32"))
+
+
+def test_reduce_plan_time_checks(session):
+    # non-consecutive dims (reduce_impl.h:41-42)
+    with pytest.raises(RuntimeError, match="consecutive"):
+        session.load_from_memory(reduction_module("cuda", [2, 16, 32], [0, 2], "ReduceSumOp_f32_f32"))
+    # {0, 2} over [1, 16, 32] is fine: size-1 dims are dropped first
+    session.load_from_memory(reduction_module("cuda", [1, 16, 32], [0, 2], "ReduceSumOp_f32_f32"))
+    # keep-dims output shape is rejected (reduce_impl.h:35)
+    tin, tout = memref([4, 8], "f32", "cuda"), memref([4, 1], "f32", "cuda")
+    bad = f"""func.func @t(%a : {tin}, %b : {tout}) attributes {{byre.entry_point}} {{
+      byre.compute @ReduceSumOp_f32_f32(%a, %b) {{dimensions = dense<[1]> : tensor<1xi64>}} : {tin}, {tout}
+      return }}"""
+    with pytest.raises(RuntimeError, match="output shape"):
+        session.load_from_memory(bad)
+    # out-of-range dimension
+    with pytest.raises(RuntimeError, match="invalid dimension"):
+        session.load_from_memory(bad.replace("dense<[1]>", "dense<[2]>").replace("4x1xf32", "4x8xf32"))
+    # element type must match the key
+    with pytest.raises(RuntimeError, match="element type"):
+        session.load_from_memory(reduction_module("cuda", [4, 8], [1], "ReduceSumOp_f16_f16", dtype="f32"))
+    # missing attribute
+    with pytest.raises(RuntimeError, match="dimensions is not set"):
+        session.load_from_memory(reduction_module("cuda", [4, 8], [1], "ReduceSumOp_f32_f32").replace("dimensions = dense<[1]> : tensor<1xi64>, ", ""))
+
+
+def test_softmax_plan_time_checks(session):
+    session.load_from_memory(softmax_module("cuda", [10, 128], "bf16", 1))
+    session.load_from_memory(softmax_module("cuda", [8, 12, 256, 256], "f32", -1))
+    with pytest.raises(RuntimeError, match="last axis"):
+        session.load_from_memory(softmax_module("cuda", [10, 128], "f32", 0))
+    with pytest.raises(RuntimeError, match="f32, f16 or bf16"):
+        session.load_from_memory(softmax_module("cuda", [10, 128], "i32", 1))
+
+
+def test_custom_op_load_errors(session, golden_dir):
+    text = open(os.path.join(golden_dir, "flash_attn_fwd.mlir")).read()
+    with pytest.raises(RuntimeError, match="load failed"):
+        session.load_from_memory(text.replace("libflash_attn.so", "libdoes_not_exist.so"))
+    with pytest.raises(RuntimeError, match="Couldn't find function: run_flash_attn_nope"):
+        session.load_from_memory(text.replace("run_flash_attn_fwd", "run_flash_attn_nope"))
+    # a library without a VERSION symbol is refused (custom.cc:50-51)
+    from byteir_amd import _lib
+    with pytest.raises(RuntimeError, match="Version doesn't exist"):
+        session.load_from_memory(text.replace("test/test_files/external_libs/libflash_attn.so", _lib.lib_path("libbrt_rocm_kernels.so"))
+                                 .replace("run_flash_attn_fwd", "brt_rocm_softmax"))
+
+
+def test_parse_errors_are_reported_with_a_line(session):
+    with pytest.raises(RuntimeError, match="ByRE parse error: line 2"):
+        session.load_from_memory('func.func @t(%a : memref<4xf32, "cuda">) attributes {byre.entry_point} {\n  byre.compute @X(%b) : memref<4xf32, "cuda">\n return }')
+    with pytest.raises(RuntimeError, match="dynamic"):
+        session.load_from_memory('func.func @t(%a : memref<?x4xf32, "cuda">) attributes {byre.entry_point} { return }')
+    with pytest.raises(RuntimeError, match="entry_point"):
+        session.load_from_memory('func.func @t(%a : memref<4xf32, "cuda">) { return }')
+
+
+def test_python_side_canonicalisation_matches_oracle():
+    import oracle
+    from byteir_amd import ops
+    for shape, dims in [((1, 16, 32), (0,)), ((2, 16, 8, 64), (1, 2)), ((4, 8, 3, 5), (3, 2)), ((1, 7, 1), (0, 2))]:
+        out_shape = oracle.deduce_output_shape(shape, dims)
+        st, A, B, C = oracle.reduce_canonicalize(shape, out_shape, dims)
+        assert st == 0 and ops.canonicalize_reduce(list(shape), out_shape, list(dims)) == (A, B, C)
+    with pytest.raises(ValueError):
+        ops.canonicalize_reduce([2, 16, 32], [16], [0, 2])
+
+
+def test_flash_blob_packer_matches_oracle():
+    import numpy as np
+    import torch
+    import oracle
+    from byteir_amd import ops
+    q = torch.empty((4, 2048, 32, 128), dtype=torch.float16, device="meta")
+    blob = ops.pack_flash_args(q, q, q, q, float(np.float32(1 / np.sqrt(128))), (-1, 0))
+    a = oracle.fa_args(4, 2048, 2048, 32, 32, 128, 1 / np.sqrt(128), window=(-1, 0))
+    assert blob == oracle.fa_pack_args(a).tobytes()

@@ -1,0 +1,165 @@
+"""End-to-end through the BRT-shaped runtime on the GPU: a ByRE module is loaded into a Session
+with the ROCm provider, arguments are bound, Session::Run enqueues the op kernels and the results
+are compared with the CPU oracle -- the structure of the reference's op tests
+(runtime/test/backends/cuda/providers/default/kernel/{reduction,flash_attn_fwd,flash_attn_bwd}_test.cc)."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from byre_text import reduction_module, softmax_module
+from gpu_util import dev, host
+
+pytestmark = pytest.mark.gpu
+
+REF_CASES = [
+    ((1, 16, 32), (0,)), ((1, 16, 32), (1,)), ((1, 16, 32), (2,)), ((1, 16, 32), (0, 1)),
+    ((1, 16, 32), (0, 2)), ((1, 128, 128), (0, 1)), ((2, 128, 256), (0, 1)), ((2, 16, 8, 64), (1, 2)),
+    ((16384, 8192), (0,)),  # BASELINE configs[1]: needs the per-frame workspace
+]
+
+
+@pytest.fixture()
+def session():
+    from byteir_amd import brt
+    s = brt.Session(device="ROCM")
+    yield s
+    s.close()
+
+
+@pytest.mark.parametrize("op_name,op", [("ReduceSumOp_f32_f32", oracle.SUM), ("ReduceMaxOp_f32_f32", oracle.MAX)])
+@pytest.mark.parametrize("shape,dims", REF_CASES)
+def test_reduction_through_session_twice(session, shape, dims, op_name, op):
+    session.load_from_memory(reduction_module("cuda", list(shape), list(dims), op_name))
+    req = session.new_request_context()  # the request owns its stream
+    rng = np.random.default_rng(7)
+    out_shape = oracle.deduce_output_shape(shape, dims)
+    st, A, B, C = oracle.reduce_canonicalize(shape, out_shape, dims)
+    x = dev(rng.random(shape, dtype=np.float32))
+    y = torch.full(out_shape, -7.0, device="cuda")
+    req.bind_arg(0, x.data_ptr())
+    req.bind_arg(1, y.data_ptr())
+    req.finish_io_binding()
+    for run in range(2):  # second run on the same frame re-uses the workspace (reduction_test.cc:147-164)
+        if run:
+            x.copy_(dev(rng.random(shape, dtype=np.float32) - 0.5))
+            torch.cuda.synchronize()
+        req.run()
+        req.sync()
+        xh, got = host(x), host(y)
+        if op == oracle.MAX or not (A and B and C):
+            assert np.array_equal(got, oracle.reduce_op(op, xh, dims))
+        else:
+            s64, sabs = oracle.reduce_sum_f64(xh, A, B, C)
+            assert np.all(np.abs(got.reshape(-1) - s64) <= 1e-5 * np.maximum(np.abs(s64), 1e-2 * sabs) + 1e-30)
+    req.close()
+
+
+@pytest.mark.parametrize("op_name", ["ReduceSumOp_f32_f32", "ReduceMaxOp_f32_f32"])
+def test_nan_propagation_through_session(session, op_name):
+    # reduction_test.cc:182-215: 1024 elements, NaN first; runtime-allocated arguments
+    session.load_from_memory(reduction_module("cuda", [1024], [0], op_name))
+    req = session.new_request_context()
+    x = np.random.default_rng(8).random(1024, dtype=np.float32)
+    x[0] = np.nan
+    from byteir_amd import _lib
+    K = _lib.kernels()
+    p_in = req.get_arg(0)  # allocated by the frame, like request->GetArg(0) in the reference test
+    _lib.check(K.brt_rocm_memcpy_h2d(p_in, x.ctypes.data, x.nbytes, None))
+    _lib.check(K.brt_rocm_device_synchronize())
+    req.finish_io_binding()
+    req.run()
+    req.sync()
+    out = np.zeros(1, np.float32)
+    _lib.check(K.brt_rocm_memcpy_d2h(out.ctypes.data, req.get_arg(1), 4, None))
+    _lib.check(K.brt_rocm_device_synchronize())
+    assert np.isnan(out[0])
+
+
+def test_flash_attn_fwd_module_unchanged(session, golden_dir):
+    """SM80CUDATestFlashAttnFwd.Basic: the reference's fixture module and data; Q, K, V, Out and
+    SoftmaxLse are bound, SoftmaxPtr and RngState are left to the frame."""
+    session.load(os.path.join(golden_dir, "flash_attn_fwd.mlir"))
+    req = session.new_request_context(torch.cuda.current_stream().cuda_stream)
+    g = {n: np.load(os.path.join(golden_dir, f"fa_{n}.npy")) for n in ("q", "k", "v", "out")}
+    q, k, v = dev(g["q"]), dev(g["k"]), dev(g["v"])
+    o = torch.zeros_like(q)
+    lse = torch.zeros((1, 3, 128), device="cuda")
+    for i, t in enumerate((q, k, v, o, lse)):
+        req.bind_arg(i, t.data_ptr())
+    req.finish_io_binding()
+    req.run()
+    req.sync()
+    got, want = host(o).astype(np.float32), g["out"].astype(np.float32)
+    assert np.all(np.abs(got - want) <= 2.0 ** -10 * np.abs(want) + 1e-7)  # one fp16 ulp
+    _, lse_ref, _ = oracle.flash_fwd(g["q"], g["k"], g["v"], 0.5, (-1, 0))
+    np.testing.assert_allclose(host(lse), lse_ref, atol=1e-4)
+
+
+def test_flash_attn_bwd_module_unchanged(session, golden_dir):
+    """SM80CUDATestFlashAttnBwd.Basic: forward then backward in one module."""
+    session.load(os.path.join(golden_dir, "flash_attn_bwd.mlir"))
+    req = session.new_request_context(torch.cuda.current_stream().cuda_stream)
+    g = {n: np.load(os.path.join(golden_dir, f"fa_{n}.npy")) for n in ("q", "k", "v", "dout", "out", "dq", "dk", "dv")}
+    do, q, k, v = dev(g["dout"]), dev(g["q"]), dev(g["k"]), dev(g["v"])
+    o = torch.zeros_like(q)
+    lse = torch.zeros((1, 3, 128), device="cuda")
+    dq, dk, dv = torch.zeros_like(q), torch.zeros_like(q), torch.zeros_like(q)
+    for i, t in enumerate((do, q, k, v, o, lse, dq, dk, dv)):
+        req.bind_arg(i, t.data_ptr())
+    req.finish_io_binding()  # RngState, d_SoftmaxLse, d_Q_accum, SoftmaxPtr come from the frame
+    req.run()
+    req.sync()
+    for name, t in (("dq", dq), ("dk", dk), ("dv", dv)):
+        want = g[name].astype(np.float32)
+        err = np.abs(host(t).astype(np.float32) - want)
+        assert np.all(err <= 2 * 2.0 ** -10 * np.abs(want) + 4e-6), name
+
+
+@pytest.mark.parametrize("dtype,code", [("f32", oracle.F32), ("bf16", oracle.BF16), ("f16", oracle.F16)])
+def test_softmax_through_backend(dtype, code):
+    """byteir.softmax via BRTBackend (torch's caching allocator and current stream), on the
+    reference's own softmax test shapes."""
+    import tempfile
+    from byteir_amd.brt import BRTBackend
+    for shape, axis in (([10, 128], 1), ([2, 3, 256, 256], -1)):
+        with tempfile.NamedTemporaryFile("w", suffix=".mlir", delete=False) as f:
+            f.write(softmax_module("cuda", shape, dtype, axis))
+        be = BRTBackend("cuda", f.name)
+        x32 = (np.random.default_rng(9).standard_normal(shape) * 2).astype(np.float32)
+        xs = oracle.from_f32(x32, code)
+        (y,) = be.run([dev(xs)])
+        got, want = oracle.to_f32(host(y)), oracle.to_f32(oracle.softmax(xs))
+        rel = {oracle.F32: 1e-5, oracle.F16: 2.0 ** -10, oracle.BF16: 2.0 ** -7}[code]
+        assert np.all(np.abs(got - want) <= rel * np.abs(want) + 6e-8)
+        ms = be.profile_with_outputs([dev(xs)], [y], warmup=2, iters=3)
+        assert ms > 0
+        be.session.close()
+        os.unlink(f.name)
+
+
+def test_copy_ops_and_listener(session):
+    text = """func.func @t(%h : memref<1000xf32, "cpu"> {byre.argname = "h", byre.argtype = 1: i32},
+                      %o : memref<1000xf32, "cpu"> {byre.argname = "o", byre.argtype = 2: i32}) attributes {byre.entry_point} {
+      %d0 = memref.alloc() : memref<1000xf32, "cuda">
+      %d1 = memref.alloc() : memref<1000xf32, "cuda">
+      byre.compute @cpu2cuda(%h, %d0) {device = "cuda"} : memref<1000xf32, "cpu">, memref<1000xf32, "cuda">
+      byre.compute @cuda2cuda(%d0, %d1) : memref<1000xf32, "cuda">, memref<1000xf32, "cuda">
+      byre.compute @cuda2cpu(%d1, %o) : memref<1000xf32, "cuda">, memref<1000xf32, "cpu">
+      return }"""
+    session.load_from_memory(text)
+    req = session.new_request_context()
+    seen = []
+    req.add_op_listener(lambda key, idx, after: seen.append((key, idx, after)))
+    src = np.arange(1000, dtype=np.float32)
+    dst = np.zeros(1000, dtype=np.float32)
+    req.bind_arg(0, src.ctypes.data)
+    req.bind_arg(1, dst.ctypes.data)
+    req.finish_io_binding()
+    req.run()
+    req.sync()
+    assert np.array_equal(src, dst)
+    assert seen == [("cpu2cuda", 0, False), ("cpu2cuda", 0, True), ("cuda2cuda", 1, False), ("cuda2cuda", 1, True),
+                    ("cuda2cpu", 2, False), ("cuda2cpu", 2, True)]
