@@ -21,11 +21,18 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
+#include <cstdlib>
 
 #include "brt_rocm_kernels.h"
 
 namespace {
 
+#ifndef RED_ROW_U
+#define RED_ROW_U 4
+#endif
+#ifndef RED_COL_U
+#define RED_COL_U 8
+#endif
 constexpr int kBlock = 256;            // threads per workgroup (4 waves)
 constexpr uint64_t kFillThreads = 256ull * 1024;  // threads wanted in flight chip-wide
 
@@ -42,10 +49,13 @@ template <> struct Fold<BRT_ROCM_REDUCE_MAX> {
 };
 
 // ---- typed loads into float -----------------------------------------------------------
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 template <typename T, int VEC> struct Loader;
 template <> struct Loader<float, 4> {
   static __device__ __forceinline__ void load(const float *p, float (&v)[4]) {
-    const float4 t = *reinterpret_cast<const float4 *>(p);
+    // streamed once: a non-temporal load keeps the data from displacing cache lines
+    const f32x4 t = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(p));
     v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
   }
 };
@@ -54,7 +64,7 @@ template <> struct Loader<float, 1> {
 };
 template <> struct Loader<__half, 8> {
   static __device__ __forceinline__ void load(const __half *p, float (&v)[8]) {
-    const uint4 t = *reinterpret_cast<const uint4 *>(p);
+    const u32x4 t = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p));
     const __half2 *h = reinterpret_cast<const __half2 *>(&t);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -85,7 +95,7 @@ __global__ void __launch_bounds__(kBlock)
 reduce_row_kernel(const T *__restrict__ in, TO *__restrict__ out, uint64_t units, uint64_t B,
                   uint32_t S, uint64_t seg_len) {
   constexpr int GPB = kBlock / G;
-  constexpr int U = 4;
+  constexpr int U = RED_ROW_U;
   const int lane = threadIdx.x % G;
   uint64_t unit = (uint64_t)blockIdx.x * GPB + threadIdx.x / G;
   const bool valid = unit < units;
@@ -116,7 +126,9 @@ reduce_row_kernel(const T *__restrict__ in, TO *__restrict__ out, uint64_t units
 #pragma unroll
     for (int k = 0; k < VEC; ++k) acc[0] = Fold<OP>::apply(acc[0], v[k]);
   }
-  float r = Fold<OP>::apply(Fold<OP>::apply(acc[0], acc[1]), Fold<OP>::apply(acc[2], acc[3]));
+  float r = acc[0];
+#pragma unroll
+  for (int u = 1; u < U; ++u) r = Fold<OP>::apply(r, acc[u]);
   if constexpr (G <= 64) {
     r = wave_fold<OP>(r, G);
   } else {
@@ -138,7 +150,7 @@ __global__ void __launch_bounds__(kBlock)
 reduce_col_kernel(const T *__restrict__ in, TO *__restrict__ out, uint64_t B, uint64_t C,
                   uint32_t S, uint64_t seg_rows, uint32_t col_tiles) {
   constexpr int TY = kBlock / TX;
-  constexpr int U = 8;
+  constexpr int U = RED_COL_U;
   __shared__ float part[TY][TX * VEC + 1];
   const int tx = threadIdx.x % TX, ty = threadIdx.x / TX;
   uint64_t bid = blockIdx.x;
@@ -208,6 +220,9 @@ Plan make_plan(int dtype, uint64_t A, uint64_t B, uint64_t C, bool allow_split) 
     p.vec = (B % vec_full == 0) ? vec_full : 1;
     const uint64_t nvec = ceil_div(B, p.vec);
     p.g = nvec >= 2048 ? 256 : nvec >= 96 ? 64 : nvec >= 24 ? 16 : 4;
+#ifdef BRT_TUNE
+    if (getenv("RED_G")) p.g = atoi(getenv("RED_G"));
+#endif
     uint64_t S = 1;
     if (allow_split && A * p.g < kFillThreads) {
       const uint64_t want = ceil_div(kFillThreads, A * p.g);
@@ -223,17 +238,34 @@ Plan make_plan(int dtype, uint64_t A, uint64_t B, uint64_t C, bool allow_split) 
   p.kind = 2;
   p.vec = (C % vec_full == 0) ? vec_full : 1;
   const uint64_t ncolv = ceil_div(C, p.vec);
-  p.g = ncolv > 32 ? 64 : ncolv > 8 ? 32 : 8;
+  if (allow_split) {
+    // first (or only) pass: a block spans up to 256 lanes x 128 bits = 4 KiB of one row
+    p.g = ncolv >= 256 ? 256 : ncolv > 32 ? 64 : ncolv > 8 ? 32 : 8;
+  } else {
+    // second pass over few rows of partials: narrow tiles so that enough blocks exist
+    p.g = 64;
+    if (A * ceil_div(ncolv, 64) < 256) p.g = 32;
+    if (A * ceil_div(ncolv, 32) < 256) p.g = 8;
+  }
+#ifdef BRT_TUNE
+  if (allow_split && getenv("RED_TX")) p.g = atoi(getenv("RED_TX"));
+#endif
   const int ty = kBlock / p.g;
   p.col_tiles = (uint32_t)ceil_div(ncolv, p.g);
   const uint64_t blocks0 = A * p.col_tiles;
   uint64_t S = 1;
-  if (allow_split && blocks0 < 1024 && B > (uint64_t)ty * 8) {
-    const uint64_t want = ceil_div(2048, blocks0);
+  // Long sequential streams from about two resident workgroups per CU measured fastest on
+  // MI355X (more, shorter segments lose HBM efficiency), so the split aims at 512 workgroups.
+  constexpr uint64_t kWantBlocks = 512;
+  if (allow_split && blocks0 < kWantBlocks && B > (uint64_t)ty * 8) {
+    const uint64_t want = ceil_div(kWantBlocks, blocks0);
     const uint64_t room = ceil_div(B, (uint64_t)ty * 8);
     S = want < room ? want : room;
     if (S > 1024) S = 1024;
   }
+#ifdef BRT_TUNE
+  if (allow_split && getenv("RED_S")) S = atoi(getenv("RED_S"));
+#endif
   p.seg = round_up(ceil_div(B, S), ty);
   p.S = (uint32_t)ceil_div(B, p.seg);
   return p;
@@ -272,6 +304,7 @@ hipError_t launch(const Plan &p, const T *in, TO *out, uint64_t A, uint64_t B, u
   switch (p.g) {
   case 8: COL(8); break;
   case 32: COL(32); break;
+  case 256: COL(256); break;
   default: COL(64); break;
   }
 #undef COL
@@ -280,14 +313,19 @@ hipError_t launch(const Plan &p, const T *in, TO *out, uint64_t A, uint64_t B, u
 
 template <typename T, int OP>
 hipError_t run(const T *in, T *out, uint64_t A, uint64_t B, uint64_t C, void *ws, size_t ws_bytes,
-               int dtype, hipStream_t stream) {
+               int dtype, hipStream_t stream, hipEvent_t first_pass_done) {
   const Plan p = make_plan(dtype, A, B, C, true);
-  if (p.S == 1) return launch<T, T, OP>(p, in, out, A, B, C, stream);
+  if (p.S == 1) {
+    const hipError_t e = launch<T, T, OP>(p, in, out, A, B, C, stream);
+    if (e == hipSuccess && first_pass_done) return hipEventRecord(first_pass_done, stream);
+    return e;
+  }
   const size_t need = sizeof(float) * A * p.S * C;
   if (ws == nullptr || ws_bytes < need) return hipErrorInvalidValue;
   float *part = static_cast<float *>(ws);
   hipError_t e = launch<T, float, OP>(p, in, part, A, B, C, stream);
   if (e != hipSuccess) return e;
+  if (first_pass_done && (e = hipEventRecord(first_pass_done, stream)) != hipSuccess) return e;
   const Plan p2 = make_plan(BRT_ROCM_F32, A, p.S, C, false);
   return launch<float, T, OP>(p2, part, out, A, p.S, C, stream);
 }
@@ -300,10 +338,11 @@ extern "C" size_t brt_rocm_reduce_workspace_bytes(int dtype, size_t A, size_t B,
   return p.S > 1 ? sizeof(float) * A * p.S * C : 0;
 }
 
-extern "C" int brt_rocm_reduce(int op, int dtype, const void *input, void *output, size_t A,
-                               size_t B, size_t C, void *workspace, size_t workspace_bytes,
-                               void *stream_) {
+extern "C" int brt_rocm_reduce_ex(int op, int dtype, const void *input, void *output, size_t A,
+                                  size_t B, size_t C, void *workspace, size_t workspace_bytes,
+                                  void *stream_, void *first_pass_done_) {
   hipStream_t stream = static_cast<hipStream_t>(stream_);
+  hipEvent_t first_pass_done = static_cast<hipEvent_t>(first_pass_done_);
   if ((op != BRT_ROCM_REDUCE_SUM && op != BRT_ROCM_REDUCE_MAX) ||
       (dtype != BRT_ROCM_F32 && dtype != BRT_ROCM_F16))
     return hipErrorInvalidValue;
@@ -318,12 +357,18 @@ extern "C" int brt_rocm_reduce(int op, int dtype, const void *input, void *outpu
     const float *in = static_cast<const float *>(input);
     float *out = static_cast<float *>(output);
     return op == BRT_ROCM_REDUCE_SUM
-               ? run<float, BRT_ROCM_REDUCE_SUM>(in, out, A, B, C, workspace, workspace_bytes, dtype, stream)
-               : run<float, BRT_ROCM_REDUCE_MAX>(in, out, A, B, C, workspace, workspace_bytes, dtype, stream);
+               ? run<float, BRT_ROCM_REDUCE_SUM>(in, out, A, B, C, workspace, workspace_bytes, dtype, stream, first_pass_done)
+               : run<float, BRT_ROCM_REDUCE_MAX>(in, out, A, B, C, workspace, workspace_bytes, dtype, stream, first_pass_done);
   }
   const __half *in = static_cast<const __half *>(input);
   __half *out = static_cast<__half *>(output);
   return op == BRT_ROCM_REDUCE_SUM
-             ? run<__half, BRT_ROCM_REDUCE_SUM>(in, out, A, B, C, workspace, workspace_bytes, dtype, stream)
-             : run<__half, BRT_ROCM_REDUCE_MAX>(in, out, A, B, C, workspace, workspace_bytes, dtype, stream);
+             ? run<__half, BRT_ROCM_REDUCE_SUM>(in, out, A, B, C, workspace, workspace_bytes, dtype, stream, first_pass_done)
+             : run<__half, BRT_ROCM_REDUCE_MAX>(in, out, A, B, C, workspace, workspace_bytes, dtype, stream, first_pass_done);
+}
+
+extern "C" int brt_rocm_reduce(int op, int dtype, const void *input, void *output, size_t A,
+                               size_t B, size_t C, void *workspace, size_t workspace_bytes,
+                               void *stream) {
+  return brt_rocm_reduce_ex(op, dtype, input, output, A, B, C, workspace, workspace_bytes, stream, nullptr);
 }

@@ -39,6 +39,16 @@ template <> struct Elem<__bf16> {
   static __device__ __forceinline__ __bf16 make(float v) { return (__bf16)v; }  // RNE
 };
 
+// the tensor is read once and written once: non-temporal accesses keep it out of the caches
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint4 load_stream(const uint4 *p) {
+  const u32x4 t = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p));
+  return uint4{t.x, t.y, t.z, t.w};
+}
+__device__ __forceinline__ void store_stream(uint4 *p, const uint4 &v) {
+  __builtin_nontemporal_store(u32x4{v.x, v.y, v.z, v.w}, reinterpret_cast<u32x4 *>(p));
+}
+
 __device__ __forceinline__ float fast_exp(float x) { return __builtin_amdgcn_exp2f(x * kLog2e); }
 
 __device__ __forceinline__ float wave_max(float v) {
@@ -67,7 +77,7 @@ softmax_wave_kernel(const T *__restrict__ in, T *__restrict__ out, uint64_t rows
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
     const uint32_t v = lane + 64u * i;
-    if (v < nvec) raw[i] = src[v];
+    if (v < nvec) raw[i] = load_stream(src + v);
   }
   float x[NV][EPV];
   float m = -INFINITY;
@@ -100,7 +110,7 @@ softmax_wave_kernel(const T *__restrict__ in, T *__restrict__ out, uint64_t rows
       T *e = reinterpret_cast<T *>(&o);
 #pragma unroll
       for (int k = 0; k < EPV; ++k) e[k] = Elem<T>::make(x[i][k] * inv);
-      dst[v] = o;
+      store_stream(dst + v, o);
     }
   }
 }

@@ -84,6 +84,13 @@ int brt_rocm_event_elapsed_ms(float *ms, void *start, void *stop);
 size_t brt_rocm_reduce_workspace_bytes(int dtype, size_t A, size_t B, size_t C);
 int brt_rocm_reduce(int op, int dtype, const void *input, void *output, size_t A, size_t B,
                     size_t C, void *workspace, size_t workspace_bytes, void *stream);
+/* The same call with a timing hook: `first_pass_done`, when not NULL, is a hipEvent_t that is
+ * recorded on `stream` right after the first (or only) pass has been enqueued, so that a caller
+ * can time the split first pass apart from the combine pass.  No counterpart in the reference
+ * (its hooks are host-side Before/AfterOpKernelRun events, framework/event.h:27-74). */
+int brt_rocm_reduce_ex(int op, int dtype, const void *input, void *output, size_t A, size_t B,
+                       size_t C, void *workspace, size_t workspace_bytes, void *stream,
+                       void *first_pass_done);
 
 /* ---- fused row softmax ----------------------------------------------------------- */
 /* y[r, :] = exp(x[r, :] - max_j x[r, j]) / sum_j exp(...) over the last axis of a dense
