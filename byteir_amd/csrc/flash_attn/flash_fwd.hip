@@ -1,32 +1,46 @@
 // Flash-attention forward for gfx950: O = softmax(scale * Q K^T + mask) V, LSE = ln sum exp.
 //
-// One workgroup (4 waves) owns 128 query rows of one (batch, head); each wave owns 32 of
-// them for the whole kernel.  K/V are streamed in 64-row tiles through LDS.  Per tile a wave
-// computes S^T = K Q^T (keys on rows, queries on columns, so every softmax statistic is
-// lane-local), does the online-softmax update in registers, rounds P^T to the storage type
-// and feeds it straight back as the B operand of O^T += V^T P^T; V^T comes out of the
-// row-major LDS tile through the transposing LDS read.  The next tile's global loads are
-// issued before the math of the current one.
+// One workgroup (8 waves, one per CU, two waves per SIMD) owns 256 query rows of one (batch,
+// head); each wave owns 32 of them for the whole kernel.  K/V are streamed in 64-row tiles
+// through a three-deep LDS ring with one barrier per tile.  Per unit of 32 keys a wave computes
+// S^T = K Q^T (keys on rows, queries on columns, so every softmax statistic is lane-local),
+// does the online-softmax update in registers, rounds P^T to the storage type and feeds it
+// straight back as the B operand of O^T += V^T P^T; V^T comes out of the row-major LDS tile
+// through the transposing LDS read.  Measured limiter: LDS read bandwidth (every wave reads the
+// whole K and V unit, 16 KiB per 16 MFMAs), not the exponentials and not LDS latency.
+//
+// The key dimension is consumed in units of 32 keys and the loop is software pipelined inside
+// each wave: S^T of unit u+1 is produced (MFMA) in the same basic block in which unit u goes
+// through exp/max/convert (VALU) and O^T += V^T P^T, so the vector work of the softmax runs in
+// the shadow of matrix instructions.  The ring is three deep: tile t is read by everyone,
+// K of tile t+1 is read by the look-ahead, and tile t+2 is being written.
 //
 // Arithmetic follows the reference kernel (external_libs/runtime/flash_attn/lib/
 // flash_fwd_kernel.h:276-469, softmax.h:128-178): fp32 accumulation, exp2 with
 // scale*log2(e) folded in, unrounded row sums, P rounded to the storage type before P V,
 // O divided by the row sum at the end, LSE = max*scale + ln(sum); a row that keeps no key
-// gives O = 0 and LSE = +inf.
+// gives O = 0 and LSE = +inf.  One deviation: the running maximum is only raised when it
+// would grow by more than kRescaleSlack (in log2 units), or from -inf; exp2 then stays below
+// 2^kRescaleSlack, the identities O = acc / sum and LSE = max*scale + ln(sum) hold for any
+// reference maximum, and the accumulator rescale (D/2 multiplies per lane per tile) rarely runs.
 #include "flash_common.h"
 
 namespace fa {
 
-constexpr int kBM = 128;  // query rows per workgroup
-constexpr int kBN = 64;   // key rows per tile
+constexpr int kBN = 64;        // key rows per tile
+constexpr int kStages = 3;     // LDS ring depth
+constexpr float kRescaleSlack = 8.0f;
 
-template <typename T, int D>
-__global__ void __launch_bounds__(256, 2) flash_fwd_kernel(const Params p) {
+// QB: 32-row halves per wave (1 or 2); NW: waves per workgroup; the workgroup owns 32*QB*NW rows
+template <typename T, int D, int QB, int NW>
+__global__ void __launch_bounds__(NW * 64, NW * QB >= 16 ? 2 : (QB == 2 ? 1 : 2)) flash_fwd_kernel(const Params p) {
+  constexpr int kThreads = NW * 64;
+  constexpr int kBM = 32 * QB * NW;
   using vec8 = typename Traits<T>::vec8;
   constexpr int KS = Pad<D>::kPlain;  // K tile row stride
   constexpr int VS = Pad<D>::kTr;     // V tile row stride
-  __shared__ __attribute__((aligned(16))) T Ks[kBN * KS];
-  __shared__ __attribute__((aligned(16))) T Vs[kBN * VS];
+  __shared__ __attribute__((aligned(16))) T Ks[kStages][kBN * KS];
+  __shared__ __attribute__((aligned(16))) T Vs[kStages][kBN * VS];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r32 = lane & 31, g = lane >> 5;
@@ -46,15 +60,19 @@ __global__ void __launch_bounds__(256, 2) flash_fwd_kernel(const Params p) {
   }
   const int bi = bh / p.h, hi = bh % p.h, hk = hi / (p.h / p.h_k);
   const int m0 = m_block * kBM;
-  const int wq0 = m0 + wave * 32;
-  const int qrow = wq0 + r32;
+  const int wq0 = m0 + wave * 32 * QB;
 
-  int lo_lim, hi_lim;
-  row_limits(p, qrow, lo_lim, hi_lim);
-  // limits of the wave's first and last row bound what the wave can see
-  int w_lo_first, w_hi_first, w_lo_last, w_hi_last;
-  row_limits(p, wq0, w_lo_first, w_hi_first);
-  row_limits(p, wq0 + 31, w_lo_last, w_hi_last);
+  int qrow[QB], lo_lim[QB], hi_lim[QB];
+  // limits of each half's first and last row bound what the half can see
+  int h_lo_first[QB], h_hi_first[QB], h_lo_last[QB], h_hi_last[QB];
+#pragma unroll
+  for (int qb = 0; qb < QB; ++qb) {
+    qrow[qb] = wq0 + qb * 32 + r32;
+    row_limits(p, qrow[qb], lo_lim[qb], hi_lim[qb]);
+    row_limits(p, wq0 + qb * 32, h_lo_first[qb], h_hi_first[qb]);
+    row_limits(p, wq0 + qb * 32 + 31, h_lo_last[qb], h_hi_last[qb]);
+  }
+  const int w_lo_first = h_lo_first[0], w_hi_last = h_hi_last[QB - 1];  // the wave's widest window
   // tile range of the workgroup
   int b_lo, b_hi, t0, t1;
   row_limits(p, m0, b_lo, t0);
@@ -62,163 +80,262 @@ __global__ void __launch_bounds__(256, 2) flash_fwd_kernel(const Params p) {
   const int n_min = b_lo / kBN;
   const int n_max = b_hi > 0 ? (b_hi + kBN - 1) / kBN : 0;
 
-  const T *qg = static_cast<const T *>(p.q) + bi * p.q_bs + (int64_t)qrow * p.q_rs + hi * p.q_hs;
   const T *kg = static_cast<const T *>(p.k) + bi * p.k_bs + hk * p.k_hs;
   const T *vg = static_cast<const T *>(p.v) + bi * p.v_bs + hk * p.v_hs;
 
-  vec8 qf[D / 16];
+  vec8 qf[QB][D / 16];
 #pragma unroll
-  for (int ks = 0; ks < D / 16; ++ks) {
-    if (qrow < p.sq) qf[ks] = *reinterpret_cast<const vec8 *>(qg + ks * 16 + g * 8);
-    else qf[ks] = vec8{0};
+  for (int qb = 0; qb < QB; ++qb) {
+    const T *qg = static_cast<const T *>(p.q) + bi * p.q_bs + (int64_t)qrow[qb] * p.q_rs + hi * p.q_hs;
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ++ks) {
+      if (qrow[qb] < p.sq) qf[qb][ks] = *reinterpret_cast<const vec8 *>(qg + ks * 16 + g * 8);
+      else qf[qb][ks] = vec8{0};
+    }
   }
+  // Consume the Q fragments once here: the wait for their global loads is then placed before
+  // the loop instead of in front of the first MFMA of every iteration, where it would also
+  // drain the K/V prefetch that has just been issued.
+#pragma unroll
+  for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ++ks) asm volatile("" : "+v"(qf[qb][ks]));
 
-  constexpr int CPR = D / 8;       // 16-byte chunks per tile row
-  constexpr int RPP = 256 / CPR;   // rows covered by one pass of the workgroup
-  constexpr int NP = kBN / RPP;    // passes per tile
+  constexpr int CPR = D / 8;                       // 16-byte chunks per tile row
+  constexpr int RPP = kThreads / CPR;              // rows covered by one pass of the workgroup
+  constexpr int NP = RPP >= kBN ? 1 : kBN / RPP;   // passes per tile
   const int ld_c = tid % CPR, ld_r = tid / CPR;
+  const bool ld_on = RPP <= kBN || ld_r < kBN;     // narrow heads: surplus threads stay idle
   uint4 kreg[NP], vreg[NP];
-  auto gload = [&](int t) {
+  // running pointers to this thread's first chunk of the next tile to fetch
+  const T *kp = kg + (int64_t)(n_min * kBN + ld_r) * p.k_rs + ld_c * 8;
+  const T *vp = vg + (int64_t)(n_min * kBN + ld_r) * p.v_rs + ld_c * 8;
+  const int64_t k_pass = (int64_t)RPP * p.k_rs, v_pass = (int64_t)RPP * p.v_rs;
+  const int64_t k_tile = (int64_t)kBN * p.k_rs, v_tile = (int64_t)kBN * p.v_rs;
+  int ld_kv = n_min * kBN + ld_r;  // key row of pass 0 of the next tile to fetch
+  auto gload = [&]() {
 #pragma unroll
     for (int s = 0; s < NP; ++s) {
-      const int kv = t * kBN + s * RPP + ld_r;
-      if (kv < p.sk) {
-        kreg[s] = *reinterpret_cast<const uint4 *>(kg + (int64_t)kv * p.k_rs + ld_c * 8);
-        vreg[s] = *reinterpret_cast<const uint4 *>(vg + (int64_t)kv * p.v_rs + ld_c * 8);
+      if (ld_on && ld_kv + s * RPP < p.sk) {
+        kreg[s] = *reinterpret_cast<const uint4 *>(kp + s * k_pass);
+        vreg[s] = *reinterpret_cast<const uint4 *>(vp + s * v_pass);
       } else {  // zero rows: 0 * finite stays finite in P V
         kreg[s] = uint4{0, 0, 0, 0};
         vreg[s] = uint4{0, 0, 0, 0};
       }
     }
+    kp += k_tile; vp += v_tile; ld_kv += kBN;
   };
-  auto lstore = [&]() {
+  const int st_off_k = ld_r * KS + ld_c * 8, st_off_v = ld_r * VS + ld_c * 8;
+  auto lstore = [&](int buf) {
 #pragma unroll
     for (int s = 0; s < NP; ++s) {
-      const int row = s * RPP + ld_r;
-      *reinterpret_cast<uint4 *>(&Ks[row * KS + ld_c * 8]) = kreg[s];
-      *reinterpret_cast<uint4 *>(&Vs[row * VS + ld_c * 8]) = vreg[s];
+      if (ld_on) {
+        *reinterpret_cast<uint4 *>(&Ks[buf][st_off_k + s * RPP * KS]) = kreg[s];
+        *reinterpret_cast<uint4 *>(&Vs[buf][st_off_v + s * RPP * VS]) = vreg[s];
+      }
     }
   };
 
-  float16v o_acc[D / 32];
+  float16v o_acc[QB][D / 32];
 #pragma unroll
-  for (int i = 0; i < D / 32; ++i) o_acc[i] = float16v{0};
-  float m_run = -INFINITY, l_run = 0.f;
+  for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+    for (int i = 0; i < D / 32; ++i) o_acc[qb][i] = float16v{0};
+  float m_run[QB], l_run[QB];
+#pragma unroll
+  for (int qb = 0; qb < QB; ++qb) { m_run[qb] = -INFINITY; l_run[qb] = 0.f; }
   const float c = p.scale_log2;
+  const int k_rd = r32 * KS + g * 8;  // this lane's K fragment offset inside a 32-row block
 
-  if (n_min < n_max) {
-    gload(n_min);
-    lstore();
-    __syncthreads();
-  }
-  for (int t = n_min; t < n_max; ++t) {
-    const int kv0 = t * kBN;
-    if (t + 1 < n_max) gload(t + 1);
-    // the wave sees nothing of this tile when it lies wholly outside the widest row window
-    const bool skip = kv0 >= w_hi_last || kv0 + kBN <= w_lo_first;
-    if (!skip) {
-      float16v s[2];
+  // The key dimension is consumed in units of 32 keys (half an LDS tile).  The loop is software
+  // pipelined inside each wave: the MFMAs of S^T for unit u+1 are independent of the softmax of
+  // unit u, so they share a basic block and the exp/max/convert work runs in the MFMA shadow.
+  // a wave sees nothing of a unit that lies wholly outside its widest row window
+  auto skipped = [&](int kv0) { return kv0 >= w_hi_last || kv0 + 32 <= w_lo_first; };
+
+  struct Unit { float16v s[QB]; };  // S^T of one unit: [half]
+
+  auto qk = [&](const T *Kt, int kvb, Unit &out) {  // S^T (32 keys x 64 queries) = K Q^T
 #pragma unroll
-      for (int kvb = 0; kvb < 2; ++kvb) {
-        s[kvb] = float16v{0};
+    for (int qb = 0; qb < QB; ++qb) out.s[qb] = float16v{0};
 #pragma unroll
-        for (int ks = 0; ks < D / 16; ++ks) {
-          const vec8 a = lds_read8<T>(&Ks[(kvb * 32 + r32) * KS + ks * 16 + g * 8]);
-          s[kvb] = Traits<T>::mfma(a, qf[ks], s[kvb]);
+    for (int ks = 0; ks < D / 16; ++ks) {
+      const vec8 a = lds_read8<T>(&Kt[k_rd + kvb * 32 * KS + ks * 16]);
+#pragma unroll
+      for (int qb = 0; qb < QB; ++qb) out.s[qb] = Traits<T>::mfma(a, qf[qb][ks], out.s[qb]);
+    }
+  };
+
+  // online softmax of one unit, first part: mask, running maximum, rare accumulator rescale
+  auto sm_head = [&](Unit &u, int kv0) {
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) {
+      float16v &sc = u.s[qb];
+      if (kv0 + 32 > h_hi_first[qb] || kv0 < h_lo_last[qb]) {  // a unit on the edge of the window
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int kv = kv0 + (i >> 2) * 8 + g * 4 + (i & 3);
+          if (kv >= hi_lim[qb] || kv < lo_lim[qb]) sc[i] = -INFINITY;
         }
-      }
-      const bool need_mask = kv0 + kBN > w_hi_first || kv0 < w_lo_last;
-      if (need_mask) {
-#pragma unroll
-        for (int kvb = 0; kvb < 2; ++kvb)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) {
-            const int kv = kv0 + kvb * 32 + (i >> 2) * 8 + g * 4 + (i & 3);
-            if (kv >= hi_lim || kv < lo_lim) s[kvb][i] = -INFINITY;
-          }
       }
       float mx = -INFINITY;
 #pragma unroll
-      for (int kvb = 0; kvb < 2; ++kvb)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[kvb][i]);
+      for (int i = 0; i < 16; ++i) mx = fmaxf(mx, sc[i]);
       mx = fmaxf(mx, partner32(mx));
-      const float m_new = fmaxf(m_run, mx);
-      const float m_use = m_new == -INFINITY ? 0.f : m_new;
-      const float alpha = exp2_fast((m_run - m_use) * c);
-      const float m_scaled = m_use * c;
-      float rs = 0.f;
+      // raise the reference maximum only when it would grow by more than the slack
+      const bool grow = (mx - m_run[qb]) * c > kRescaleSlack;  // false for -inf - -inf (NaN)
+      const bool first = m_run[qb] == -INFINITY && mx != -INFINITY;
+      if (__builtin_amdgcn_ballot_w64(grow || first) != 0) {
+        const float m_new = (grow || first) ? mx : m_run[qb];
+        const float m_use = m_new == -INFINITY ? 0.f : m_new;
+        const float alpha = exp2_fast((m_run[qb] - m_use) * c);
+        l_run[qb] *= alpha;
+        m_run[qb] = m_new;
 #pragma unroll
-      for (int kvb = 0; kvb < 2; ++kvb)
+        for (int db = 0; db < D / 32; ++db)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const float e = exp2_fast(fmaf(s[kvb][i], c, -m_scaled));
-          s[kvb][i] = e;
-          rs += e;
-        }
-      l_run = l_run * alpha + rs;
-      m_run = m_new;
-#pragma unroll
-      for (int db = 0; db < D / 32; ++db)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) o_acc[db][i] *= alpha;
-      // O^T += V^T P^T, 16 keys per step
-#pragma unroll
-      for (int w = 0; w < 4; ++w) {
-        float pf[8];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) pf[j] = s[w >> 1][(w & 1) * 8 + j];
-        const vec8 pb = pack8<T>(pf);
-#pragma unroll
-        for (int db = 0; db < D / 32; ++db) {
-          const vec8 a = lds_read_operand_tr<T>(Vs, VS, w * 16, db * 32);
-          o_acc[db] = Traits<T>::mfma(a, pb, o_acc[db]);
-        }
+          for (int i = 0; i < 16; ++i) o_acc[qb][db][i] *= alpha;
       }
     }
-    __syncthreads();  // every wave is done with the tile in LDS
-    if (t + 1 < n_max) lstore();
+  };
+
+  // exponentials, row sums and P^T of one unit (branch free)
+  auto sm_exp = [&](Unit &u, vec8 (&pb)[QB][2]) {
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) {
+      float16v &sc = u.s[qb];
+      const float m_scaled = (m_run[qb] == -INFINITY ? 0.f : m_run[qb]) * c;
+      float rs = 0.f;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const float e = exp2_fast(fmaf(sc[i], c, -m_scaled));
+        sc[i] = e;
+        rs += e;
+      }
+      l_run[qb] += rs;
+#pragma unroll
+      for (int w = 0; w < 2; ++w) {
+        float pf[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) pf[j] = sc[w * 8 + j];
+        pb[qb][w] = pack8<T>(pf);
+      }
+    }
+  };
+
+  // O^T += V^T P^T for the unit's two 16-key windows; each V^T fragment serves both halves
+  auto pv = [&](const T *Vt, int kvb, const vec8 (&pb)[QB][2]) {
+#pragma unroll
+    for (int w = 0; w < 2; ++w)
+#pragma unroll
+      for (int db = 0; db < D / 32; ++db) {
+        const vec8 a = lds_read_operand_tr<T>(Vt, VS, kvb * 32 + w * 16, db * 32);
+#pragma unroll
+        for (int qb = 0; qb < QB; ++qb) o_acc[qb][db] = Traits<T>::mfma(a, pb[qb][w], o_acc[qb][db]);
+      }
+  };
+
+  // one pipeline step: finish unit `cur` (softmax, P V) and, in the same basic block, start
+  // unit `nxt` (S^T) so that matrix and vector instructions interleave
+  auto step = [&](bool do_cur, Unit &cur, int kv0, const T *Vt, int kvb, bool do_nxt, Unit &nxt,
+                  const T *Knext, int kvb_next) {
+    if (do_cur) sm_head(cur, kv0);
+    vec8 pb[QB][2];
+    if (do_cur && do_nxt) {
+      qk(Knext, kvb_next, nxt);
+      sm_exp(cur, pb);
+      pv(Vt, kvb, pb);
+    } else if (do_cur) {
+      sm_exp(cur, pb);
+      pv(Vt, kvb, pb);
+    } else if (do_nxt) {
+      qk(Knext, kvb_next, nxt);
+    }
+  };
+
+  // prologue: tiles n_min and n_min+1 into the ring, tile n_min+2 into registers
+  const int n_tiles = n_max > n_min ? n_max - n_min : 0;
+  Unit ua, ub;  // S^T of the unit being consumed / being produced
+  if (n_tiles > 0) {
+    gload();
+    lstore(0);
+    if (n_tiles > 1) { gload(); lstore(1); }
+    if (n_tiles > 2) gload();
     __syncthreads();
+    if (!skipped(n_min * kBN)) qk(Ks[0], 0, ua);
+  }
+  int buf = 0;  // ring slot of tile t
+  for (int t = n_min; t < n_max; ++t) {
+    const int buf1 = buf + 1 == kStages ? 0 : buf + 1;
+    const int buf2 = buf1 + 1 == kStages ? 0 : buf1 + 1;
+    const int kv0 = t * kBN;
+    // unit 0 of tile t (S in ua) while S of unit 1 is produced into ub
+    step(!skipped(kv0), ua, kv0, Vs[buf], 0, !skipped(kv0 + 32), ub, Ks[buf], 1);
+    __syncthreads();  // tile t+1 is visible; every wave has left tile t-1
+    // tile t+2: registers -> the ring slot tile t-1 occupied; tile t+3 in flight
+    if (t + 2 < n_max) lstore(buf2);
+    if (t + 3 < n_max) gload();
+    // unit 1 of tile t (S in ub) while S of unit 0 of tile t+1 is produced into ua
+    step(!skipped(kv0 + 32), ub, kv0 + 32, Vs[buf], 1, t + 1 < n_max && !skipped(kv0 + kBN), ua, Ks[buf1], 0);
+    buf = buf1;
   }
 
   // epilogue: normalise, write O and LSE
-  const float l_tot = l_run + partner32(l_run);
-  const bool empty = l_tot == 0.f || l_tot != l_tot;
-  const float inv = empty ? 1.f : 1.f / l_tot;
-  if (qrow < p.sq) {
-    T *og = static_cast<T *>(p.o_w) + bi * p.o_bs + (int64_t)qrow * p.o_rs + hi * p.o_hs;
 #pragma unroll
-    for (int db = 0; db < D / 32; ++db)
+  for (int qb = 0; qb < QB; ++qb) {
+    const float l_tot = l_run[qb] + partner32(l_run[qb]);
+    const bool empty = l_tot == 0.f || l_tot != l_tot;
+    const float inv = empty ? 1.f : 1.f / l_tot;
+    if (qrow[qb] < p.sq) {
+      T *og = static_cast<T *>(p.o_w) + bi * p.o_bs + (int64_t)qrow[qb] * p.o_rs + hi * p.o_hs;
 #pragma unroll
-      for (int i4 = 0; i4 < 4; ++i4) {
-        typedef T vec4 __attribute__((ext_vector_type(4)));
-        vec4 v;
+      for (int db = 0; db < D / 32; ++db)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) v[j] = (T)(o_acc[db][i4 * 4 + j] * inv);
-        *reinterpret_cast<vec4 *>(og + db * 32 + i4 * 8 + g * 4) = v;
-      }
-    if (g == 0)
-      p.lse[((int64_t)bi * p.h + hi) * p.sq + qrow] =
-          empty ? INFINITY : m_run * p.scale + log2_fast(l_tot) * kLn2;
+        for (int i4 = 0; i4 < 4; ++i4) {
+          typedef T vec4 __attribute__((ext_vector_type(4)));
+          vec4 v;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) v[j] = (T)(o_acc[qb][db][i4 * 4 + j] * inv);
+          *reinterpret_cast<vec4 *>(og + db * 32 + i4 * 8 + g * 4) = v;
+        }
+      if (g == 0)
+        p.lse[((int64_t)bi * p.h + hi) * p.sq + qrow[qb]] =
+            empty ? INFINITY : m_run[qb] * p.scale + log2_fast(l_tot) * kLn2;
+    }
   }
 }
 
-template <typename T>
-hipError_t launch_fwd_t(const Params &p, hipStream_t stream) {
-  const dim3 grid((unsigned)(p.n_mblocks * p.b * p.h)), block(256);
-  switch (p.d) {
-  case 32: flash_fwd_kernel<T, 32><<<grid, block, 0, stream>>>(p); break;
-  case 64: flash_fwd_kernel<T, 64><<<grid, block, 0, stream>>>(p); break;
-  case 128: flash_fwd_kernel<T, 128><<<grid, block, 0, stream>>>(p); break;
-  default: return hipErrorInvalidValue;
-  }
+// Geometry: 8 waves of 32 rows, two waves per SIMD.  The kernel is written for 32*QB rows per
+// wave; QB = 2 halves the LDS traffic per MFMA, but either needs a whole SIMD per wave
+// (head_dim 128: slower, the compiler's schedule leaves the single wave stalled) or brought no
+// gain when it fits (head_dim 64), so QB = 1 is what is instantiated.
+template <int D> struct FwdGeom { static constexpr int QB = 1, NW = 8; };
+
+template <typename T, int D>
+hipError_t launch_fwd_d(Params &p, hipStream_t stream) {
+  constexpr int QB = FwdGeom<D>::QB, NW = FwdGeom<D>::NW;
+  constexpr int BM = 32 * QB * NW;
+  p.n_mblocks = (p.sq + BM - 1) / BM;
+  if (p.n_mblocks == 0) return hipSuccess;
+  const dim3 grid((unsigned)(p.n_mblocks * p.b * p.h)), block(NW * 64);
+  flash_fwd_kernel<T, D, QB, NW><<<grid, block, 0, stream>>>(p);
   return hipGetLastError();
 }
 
+template <typename T>
+hipError_t launch_fwd_t(Params &p, hipStream_t stream) {
+  switch (p.d) {
+  case 32: return launch_fwd_d<T, 32>(p, stream);
+  case 64: return launch_fwd_d<T, 64>(p, stream);
+  case 128: return launch_fwd_d<T, 128>(p, stream);
+  default: return hipErrorInvalidValue;
+  }
+}
+
 hipError_t launch_fwd(Params &p, int dtype, hipStream_t stream) {
-  p.n_mblocks = (p.sq + kBM - 1) / kBM;
   p.xcd_remap = ((p.b * p.h) % 8 == 0) ? 1 : 0;
-  if (p.n_mblocks == 0 || p.b * p.h == 0) return hipSuccess;
+  if (p.b * p.h == 0 || p.sq == 0) return hipSuccess;
   return dtype == 1 ? launch_fwd_t<_Float16>(p, stream) : launch_fwd_t<__bf16>(p, stream);
 }
 
