@@ -1,8 +1,8 @@
 // Flash-attention backward for gfx950.  Three launches, no atomics, deterministic:
 //   1. dot_do_o_kernel : D[b,h,i] = sum_d dO[i,d] * O[i,d]                      (fp32)
-//   2. dkdv_kernel     : one workgroup per 128 keys, loops over query tiles;
+//   2. dkdv_kernel     : one workgroup per 128 or 256 keys, loops over query tiles;
 //                        dV = P^T dO, dK = scale * dS^T Q accumulate in registers
-//   3. dq_kernel       : one workgroup per 128 queries, loops over key tiles;
+//   3. dq_kernel       : one workgroup per 128 or 256 queries, loops over key tiles;
 //                        dQ = scale * dS K accumulates in registers
 // P = exp2(scale*log2e * S - log2e * LSE) is recomputed from the forward's LSE in both main
 // kernels; dS = P * (dO V^T - D).  P and dS are rounded to the storage type before they
@@ -77,14 +77,18 @@ struct TileLoader {
 };
 
 // ---- 2. dK, dV ------------------------------------------------------------------------------
-template <typename T, int D>
+// KB: 32-key blocks per wave.  Every Q / dO fragment fetched from LDS (plain or transposed)
+// is used for all KB blocks, so LDS traffic per MFMA falls as 1/KB; LDS read bandwidth is what
+// bounds this kernel.  The workgroup covers 128*KB keys.
+template <typename T, int D, int KB>
 __global__ void __launch_bounds__(256) dkdv_kernel(const Params p) {
   using vec8 = typename Traits<T>::vec8;
   constexpr int QS = D + 16;  // tiles are read both plainly and transposed
-  __shared__ __attribute__((aligned(16))) T Qs[kQTile * QS];
-  __shared__ __attribute__((aligned(16))) T dOs[kQTile * QS];
-  __shared__ float lse_s[kQTile];
-  __shared__ float dsm_s[kQTile];
+  constexpr int kKeys = kKvBlock * KB;
+  __shared__ __attribute__((aligned(16))) T Qs[2][kQTile * QS];
+  __shared__ __attribute__((aligned(16))) T dOs[2][kQTile * QS];
+  __shared__ float lse_s[2][kQTile];
+  __shared__ float dsm_s[2][kQTile];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r32 = lane & 31, g = lane >> 5;
@@ -101,36 +105,48 @@ __global__ void __launch_bounds__(256) dkdv_kernel(const Params p) {
     }
   }
   const int bi = bh / p.h, hi = bh % p.h;
-  const int kvb0 = n_block * kKvBlock;
-  const int kvcol = kvb0 + wave * 32 + r32;  // the key this lane owns
+  const int kvb0 = n_block * kKeys;
+  const int wkv0 = kvb0 + wave * 32 * KB;  // first key of the wave
   const int off = p.sk - p.sq;
 
   const T *qg = static_cast<const T *>(p.q) + bi * p.q_bs + hi * p.q_hs;
   const T *dog = static_cast<const T *>(p.dout) + bi * p.o_bs + hi * p.o_hs;
-  const T *kg = static_cast<const T *>(p.k) + bi * p.k_bs + (int64_t)kvcol * p.k_rs + hi * p.k_hs;
-  const T *vg = static_cast<const T *>(p.v) + bi * p.v_bs + (int64_t)kvcol * p.v_rs + hi * p.v_hs;
   const float *lse_g = p.lse + ((int64_t)bi * p.h + hi) * p.sq;
   const float *dsm_g = p.dsoftmax + ((int64_t)bi * p.h + hi) * p.sq_rounded;
 
-  vec8 kf[D / 16], vf[D / 16];
+  int kvcol[KB];  // the keys this lane owns
+  vec8 kf[KB][D / 16], vf[KB][D / 16];
 #pragma unroll
-  for (int ks = 0; ks < D / 16; ++ks) {
-    if (kvcol < p.sk) {
-      kf[ks] = *reinterpret_cast<const vec8 *>(kg + ks * 16 + g * 8);
-      vf[ks] = *reinterpret_cast<const vec8 *>(vg + ks * 16 + g * 8);
-    } else {
-      kf[ks] = vec8{0};
-      vf[ks] = vec8{0};
+  for (int kb = 0; kb < KB; ++kb) {
+    kvcol[kb] = wkv0 + kb * 32 + r32;
+    const T *kg = static_cast<const T *>(p.k) + bi * p.k_bs + (int64_t)kvcol[kb] * p.k_rs + hi * p.k_hs;
+    const T *vg = static_cast<const T *>(p.v) + bi * p.v_bs + (int64_t)kvcol[kb] * p.v_rs + hi * p.v_hs;
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ++ks) {
+      if (kvcol[kb] < p.sk) {
+        kf[kb][ks] = *reinterpret_cast<const vec8 *>(kg + ks * 16 + g * 8);
+        vf[kb][ks] = *reinterpret_cast<const vec8 *>(vg + ks * 16 + g * 8);
+      } else {
+        kf[kb][ks] = vec8{0};
+        vf[kb][ks] = vec8{0};
+      }
     }
   }
-  float16v dk_acc[D / 32], dv_acc[D / 32];
+  // consume the fragments once so that the wait for their loads sits here, not inside the loop
 #pragma unroll
-  for (int i = 0; i < D / 32; ++i) { dk_acc[i] = float16v{0}; dv_acc[i] = float16v{0}; }
+  for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ++ks) asm volatile("" : "+v"(kf[kb][ks]), "+v"(vf[kb][ks]));
+  float16v dk_acc[KB][D / 32], dv_acc[KB][D / 32];
+#pragma unroll
+  for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+    for (int i = 0; i < D / 32; ++i) { dk_acc[kb][i] = float16v{0}; dv_acc[kb][i] = float16v{0}; }
 
-  // query tiles that can see keys [kvb0, kvb0 + 128)
+  // query tiles that can see keys [kvb0, kvb0 + kKeys)
   int q_lo = 0, q_hi = p.sq;
-  if (p.wr >= 0) q_lo = max(0, kvb0 - off - p.wr);                 // hi(q) = q+1+off+wr > kvb0
-  if (p.wl >= 0) q_hi = min(p.sq, kvb0 + kKvBlock - off + p.wl);   // lo(q) = q+off-wl < kvb0+128
+  if (p.wr >= 0) q_lo = max(0, kvb0 - off - p.wr);              // hi(q) = q+1+off+wr > kvb0
+  if (p.wl >= 0) q_hi = min(p.sq, kvb0 + kKeys - off + p.wl);   // lo(q) = q+off-wl < kvb0+kKeys
   const int m_min = q_lo / kQTile;
   const int m_max = q_hi > 0 ? (q_hi + kQTile - 1) / kQTile : 0;
   const float c = p.scale_log2;
@@ -146,97 +162,129 @@ __global__ void __launch_bounds__(256) dkdv_kernel(const Params p) {
       dsm_r = q < p.sq ? dsm_g[q] : 0.f;
     }
   };
-  auto lstore = [&]() {
-    lq.lstore(Qs, QS);
-    ldo.lstore(dOs, QS);
-    if (tid < kQTile) { lse_s[tid] = lse_r * kLog2e; dsm_s[tid] = dsm_r; }
+  auto lstore = [&](int buf) {
+    lq.lstore(Qs[buf], QS);
+    ldo.lstore(dOs[buf], QS);
+    if (tid < kQTile) { lse_s[buf][tid] = lse_r * kLog2e; dsm_s[buf][tid] = dsm_r; }
   };
 
+  // double-buffered tiles, one barrier per tile: tile m is read from buffer b while tile m+1
+  // is written to the other one (free since the barrier that closed tile m-1) and tile m+2 is
+  // in flight from global memory
   if (m_min < m_max) {
     gload(m_min);
-    lstore();
+    lstore(0);
+    if (m_min + 1 < m_max) gload(m_min + 1);
     __syncthreads();
   }
   for (int m = m_min; m < m_max; ++m) {
-    if (m + 1 < m_max) gload(m + 1);
+    const int buf = (m - m_min) & 1;
+    if (m + 1 < m_max) lstore(buf ^ 1);
+    if (m + 2 < m_max) gload(m + 2);
+    const T *Qt = Qs[buf];
+    const T *dOt = dOs[buf];
 #pragma unroll
     for (int qs = 0; qs < kQTile / 32; ++qs) {
       const int q0 = m * kQTile + qs * 32;  // first query row of this 32-row sub-tile
-      // wave-uniform visibility of the sub-tile against the wave's 32 keys
-      const int wkv0 = kvb0 + wave * 32;
+      // wave-uniform visibility of the sub-tile against the wave's keys
       int lo_first, hi_first, lo_last, hi_last;
       row_limits(p, q0, lo_first, hi_first);
       row_limits(p, q0 + 31, lo_last, hi_last);
-      if (wkv0 >= hi_last || wkv0 + 32 <= lo_first) continue;  // nothing kept
-      const bool need_mask = wkv0 + 32 > hi_first || wkv0 < lo_last || q0 + 32 > p.sq;
+      if (wkv0 >= hi_last || wkv0 + 32 * KB <= lo_first) continue;  // nothing kept
+      const bool need_mask = wkv0 + 32 * KB > hi_first || wkv0 < lo_last || q0 + 32 > p.sq;
 
-      float16v s = float16v{0}, dp = float16v{0};
+      float16v s[KB], dp[KB];
+#pragma unroll
+      for (int kb = 0; kb < KB; ++kb) { s[kb] = float16v{0}; dp[kb] = float16v{0}; }
 #pragma unroll
       for (int ks = 0; ks < D / 16; ++ks) {
-        const vec8 aq = lds_read8<T>(&Qs[(qs * 32 + r32) * QS + ks * 16 + g * 8]);
-        s = Traits<T>::mfma(aq, kf[ks], s);
-        const vec8 ad = lds_read8<T>(&dOs[(qs * 32 + r32) * QS + ks * 16 + g * 8]);
-        dp = Traits<T>::mfma(ad, vf[ks], dp);
+        const vec8 aq = lds_read8<T>(&Qt[(qs * 32 + r32) * QS + ks * 16 + g * 8]);
+        const vec8 ad = lds_read8<T>(&dOt[(qs * 32 + r32) * QS + ks * 16 + g * 8]);
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb) {
+          s[kb] = Traits<T>::mfma(aq, kf[kb][ks], s[kb]);
+          dp[kb] = Traits<T>::mfma(ad, vf[kb][ks], dp[kb]);
+        }
       }
-      float pv[16], dsv[16];
+      float lse_q[16], dsm_q[16];
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         const int ql = qs * 32 + (i >> 2) * 8 + g * 4 + (i & 3);  // row inside the LDS tile
-        float pe = exp2_fast(fmaf(s[i], c, -lse_s[ql]));
-        if (need_mask) {
-          int lo, hi_;
-          row_limits(p, m * kQTile + ql, lo, hi_);
-          if (kvcol >= hi_ || kvcol < lo) pe = 0.f;
+        lse_q[i] = lse_s[buf][ql];
+        dsm_q[i] = dsm_s[buf][ql];
+      }
+      vec8 pb[KB][2], dsb[KB][2];  // P and dS as B operands: [key block][16-query window]
+#pragma unroll
+      for (int kb = 0; kb < KB; ++kb) {
+        float pv[16], dsv[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          float pe = exp2_fast(fmaf(s[kb][i], c, -lse_q[i]));
+          if (need_mask) {
+            const int ql = qs * 32 + (i >> 2) * 8 + g * 4 + (i & 3);
+            int lo, hi_;
+            row_limits(p, m * kQTile + ql, lo, hi_);
+            if (kvcol[kb] >= hi_ || kvcol[kb] < lo) pe = 0.f;
+          }
+          pv[i] = pe;
+          dsv[i] = pe * (dp[kb][i] - dsm_q[i]);
         }
-        pv[i] = pe;
-        dsv[i] = pe * (dp[i] - dsm_s[ql]);
+#pragma unroll
+        for (int w = 0; w < 2; ++w) {
+          pb[kb][w] = pack8<T>(&pv[w * 8]);
+          dsb[kb][w] = pack8<T>(&dsv[w * 8]);
+        }
       }
 #pragma unroll
-      for (int w = 0; w < 2; ++w) {
-        const vec8 pb = pack8<T>(&pv[w * 8]);
-        const vec8 dsb = pack8<T>(&dsv[w * 8]);
+      for (int w = 0; w < 2; ++w)
 #pragma unroll
         for (int db = 0; db < D / 32; ++db) {
-          const vec8 a_do = lds_read_operand_tr<T>(dOs, QS, qs * 32 + w * 16, db * 32);
-          dv_acc[db] = Traits<T>::mfma(a_do, pb, dv_acc[db]);
-          const vec8 a_q = lds_read_operand_tr<T>(Qs, QS, qs * 32 + w * 16, db * 32);
-          dk_acc[db] = Traits<T>::mfma(a_q, dsb, dk_acc[db]);
+          const vec8 a_do = lds_read_operand_tr<T>(dOt, QS, qs * 32 + w * 16, db * 32);
+          const vec8 a_q = lds_read_operand_tr<T>(Qt, QS, qs * 32 + w * 16, db * 32);
+#pragma unroll
+          for (int kb = 0; kb < KB; ++kb) {
+            dv_acc[kb][db] = Traits<T>::mfma(a_do, pb[kb][w], dv_acc[kb][db]);
+            dk_acc[kb][db] = Traits<T>::mfma(a_q, dsb[kb][w], dk_acc[kb][db]);
+          }
         }
-      }
     }
-    __syncthreads();
-    if (m + 1 < m_max) lstore();
-    __syncthreads();
+    __syncthreads();  // tile m is consumed, tile m+1 is visible
   }
 
-  if (kvcol < p.sk) {
-    T *dkg = static_cast<T *>(p.dk) + bi * p.k_bs + (int64_t)kvcol * p.k_rs + hi * p.k_hs;
-    T *dvg = static_cast<T *>(p.dv) + bi * p.v_bs + (int64_t)kvcol * p.v_rs + hi * p.v_hs;
-    typedef T vec4 __attribute__((ext_vector_type(4)));
 #pragma unroll
-    for (int db = 0; db < D / 32; ++db)
+  for (int kb = 0; kb < KB; ++kb) {
+    if (kvcol[kb] < p.sk) {
+      T *dkg = static_cast<T *>(p.dk) + bi * p.k_bs + (int64_t)kvcol[kb] * p.k_rs + hi * p.k_hs;
+      T *dvg = static_cast<T *>(p.dv) + bi * p.v_bs + (int64_t)kvcol[kb] * p.v_rs + hi * p.v_hs;
+      typedef T vec4 __attribute__((ext_vector_type(4)));
 #pragma unroll
-      for (int i4 = 0; i4 < 4; ++i4) {
-        vec4 a, b;
+      for (int db = 0; db < D / 32; ++db)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          a[j] = (T)(dk_acc[db][i4 * 4 + j] * p.scale);
-          b[j] = (T)(dv_acc[db][i4 * 4 + j]);
+        for (int i4 = 0; i4 < 4; ++i4) {
+          vec4 a, b;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            a[j] = (T)(dk_acc[kb][db][i4 * 4 + j] * p.scale);
+            b[j] = (T)(dv_acc[kb][db][i4 * 4 + j]);
+          }
+          *reinterpret_cast<vec4 *>(dkg + db * 32 + i4 * 8 + g * 4) = a;
+          *reinterpret_cast<vec4 *>(dvg + db * 32 + i4 * 8 + g * 4) = b;
         }
-        *reinterpret_cast<vec4 *>(dkg + db * 32 + i4 * 8 + g * 4) = a;
-        *reinterpret_cast<vec4 *>(dvg + db * 32 + i4 * 8 + g * 4) = b;
-      }
+    }
   }
 }
 
 // ---- 3. dQ ----------------------------------------------------------------------------------
-template <typename T, int D>
+// QB: 32-query blocks per wave.  Every K / V fragment fetched from LDS is used for all QB
+// blocks.  The workgroup covers 128*QB queries.
+template <typename T, int D, int QB>
 __global__ void __launch_bounds__(256) dq_kernel(const Params p) {
   using vec8 = typename Traits<T>::vec8;
   constexpr int KS = D + 16;          // K tile: plain and transposed reads
   constexpr int VS = Pad<D>::kPlain;  // V tile: plain reads only
-  __shared__ __attribute__((aligned(16))) T Ks[kKvTile * KS];
-  __shared__ __attribute__((aligned(16))) T Vs[kKvTile * VS];
+  constexpr int kQueries = kQBlock * QB;
+  __shared__ __attribute__((aligned(16))) T Ks[2][kKvTile * KS];
+  __shared__ __attribute__((aligned(16))) T Vs[2][kKvTile * VS];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r32 = lane & 31, g = lane >> 5;
@@ -254,116 +302,161 @@ __global__ void __launch_bounds__(256) dq_kernel(const Params p) {
     m_block = p.n_mblocks - 1 - m_block;
   }
   const int bi = bh / p.h, hi = bh % p.h;
-  const int m0 = m_block * kQBlock;
-  const int wq0 = m0 + wave * 32;
-  const int qrow = wq0 + r32;
+  const int m0 = m_block * kQueries;
+  const int wq0 = m0 + wave * 32 * QB;
 
-  int lo_lim, hi_lim, w_lo_first, w_hi_first, w_lo_last, w_hi_last, b_lo, b_hi, t0, t1;
-  row_limits(p, qrow, lo_lim, hi_lim);
-  row_limits(p, wq0, w_lo_first, w_hi_first);
-  row_limits(p, wq0 + 31, w_lo_last, w_hi_last);
+  int qrow[QB], lo_lim[QB], hi_lim[QB], h_lo_first[QB], h_hi_first[QB], h_lo_last[QB], h_hi_last[QB];
+#pragma unroll
+  for (int qb = 0; qb < QB; ++qb) {
+    qrow[qb] = wq0 + qb * 32 + r32;
+    row_limits(p, qrow[qb], lo_lim[qb], hi_lim[qb]);
+    row_limits(p, wq0 + qb * 32, h_lo_first[qb], h_hi_first[qb]);
+    row_limits(p, wq0 + qb * 32 + 31, h_lo_last[qb], h_hi_last[qb]);
+  }
+  const int w_lo_first = h_lo_first[0], w_hi_last = h_hi_last[QB - 1];
+  int b_lo, b_hi, t0, t1;
   row_limits(p, m0, b_lo, t0);
-  row_limits(p, m0 + kQBlock - 1, t1, b_hi);
+  row_limits(p, m0 + kQueries - 1, t1, b_hi);
   const int n_min = b_lo / kKvTile;
   const int n_max = b_hi > 0 ? (b_hi + kKvTile - 1) / kKvTile : 0;
 
-  const T *qg = static_cast<const T *>(p.q) + bi * p.q_bs + (int64_t)qrow * p.q_rs + hi * p.q_hs;
-  const T *dog = static_cast<const T *>(p.dout) + bi * p.o_bs + (int64_t)qrow * p.o_rs + hi * p.o_hs;
   const T *kg = static_cast<const T *>(p.k) + bi * p.k_bs + hi * p.k_hs;
   const T *vg = static_cast<const T *>(p.v) + bi * p.v_bs + hi * p.v_hs;
 
-  vec8 qf[D / 16], dof[D / 16];
-  float lse_l = INFINITY, dsm_l = 0.f;
-  if (qrow < p.sq) {
+  vec8 qf[QB][D / 16], dof[QB][D / 16];
+  float lse_l[QB], dsm_l[QB];
 #pragma unroll
-    for (int ks = 0; ks < D / 16; ++ks) {
-      qf[ks] = *reinterpret_cast<const vec8 *>(qg + ks * 16 + g * 8);
-      dof[ks] = *reinterpret_cast<const vec8 *>(dog + ks * 16 + g * 8);
+  for (int qb = 0; qb < QB; ++qb) {
+    lse_l[qb] = INFINITY;
+    dsm_l[qb] = 0.f;
+    if (qrow[qb] < p.sq) {
+      const T *qg = static_cast<const T *>(p.q) + bi * p.q_bs + (int64_t)qrow[qb] * p.q_rs + hi * p.q_hs;
+      const T *dog = static_cast<const T *>(p.dout) + bi * p.o_bs + (int64_t)qrow[qb] * p.o_rs + hi * p.o_hs;
+#pragma unroll
+      for (int ks = 0; ks < D / 16; ++ks) {
+        qf[qb][ks] = *reinterpret_cast<const vec8 *>(qg + ks * 16 + g * 8);
+        dof[qb][ks] = *reinterpret_cast<const vec8 *>(dog + ks * 16 + g * 8);
+      }
+      lse_l[qb] = p.lse[((int64_t)bi * p.h + hi) * p.sq + qrow[qb]] * kLog2e;
+      dsm_l[qb] = p.dsoftmax[((int64_t)bi * p.h + hi) * p.sq_rounded + qrow[qb]];
+    } else {
+#pragma unroll
+      for (int ks = 0; ks < D / 16; ++ks) { qf[qb][ks] = vec8{0}; dof[qb][ks] = vec8{0}; }
     }
-    lse_l = p.lse[((int64_t)bi * p.h + hi) * p.sq + qrow] * kLog2e;
-    dsm_l = p.dsoftmax[((int64_t)bi * p.h + hi) * p.sq_rounded + qrow];
-  } else {
-#pragma unroll
-    for (int ks = 0; ks < D / 16; ++ks) { qf[ks] = vec8{0}; dof[ks] = vec8{0}; }
   }
-  float16v dq_acc[D / 32];
+  // consume the fragments once so that the wait for their loads sits here, not inside the loop
 #pragma unroll
-  for (int i = 0; i < D / 32; ++i) dq_acc[i] = float16v{0};
+  for (int qb = 0; qb < QB; ++qb) {
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ++ks) asm volatile("" : "+v"(qf[qb][ks]), "+v"(dof[qb][ks]));
+    asm volatile("" : "+v"(lse_l[qb]), "+v"(dsm_l[qb]));
+  }
+  float16v dq_acc[QB][D / 32];
+#pragma unroll
+  for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+    for (int i = 0; i < D / 32; ++i) dq_acc[qb][i] = float16v{0};
   const float c = p.scale_log2;
 
+  // double-buffered tiles, one barrier per tile (see dkdv_kernel)
   TileLoader<T, D, kKvTile> lk, lv;
   if (n_min < n_max) {
     lk.gload(kg, p.k_rs, n_min * kKvTile, p.sk);
     lv.gload(vg, p.v_rs, n_min * kKvTile, p.sk);
-    lk.lstore(Ks, KS);
-    lv.lstore(Vs, VS);
+    lk.lstore(Ks[0], KS);
+    lv.lstore(Vs[0], VS);
+    if (n_min + 1 < n_max) {
+      lk.gload(kg, p.k_rs, (n_min + 1) * kKvTile, p.sk);
+      lv.gload(vg, p.v_rs, (n_min + 1) * kKvTile, p.sk);
+    }
     __syncthreads();
   }
   for (int t = n_min; t < n_max; ++t) {
+    const int buf = (t - n_min) & 1;
     const int kv0 = t * kKvTile;
-    if (t + 1 < n_max) {
-      lk.gload(kg, p.k_rs, (t + 1) * kKvTile, p.sk);
-      lv.gload(vg, p.v_rs, (t + 1) * kKvTile, p.sk);
+    if (t + 1 < n_max) { lk.lstore(Ks[buf ^ 1], KS); lv.lstore(Vs[buf ^ 1], VS); }
+    if (t + 2 < n_max) {
+      lk.gload(kg, p.k_rs, (t + 2) * kKvTile, p.sk);
+      lv.gload(vg, p.v_rs, (t + 2) * kKvTile, p.sk);
     }
+    const T *Kt = Ks[buf];
+    const T *Vt = Vs[buf];
     const bool skip = kv0 >= w_hi_last || kv0 + kKvTile <= w_lo_first;
     if (!skip) {
-      const bool need_mask = kv0 + kKvTile > w_hi_first || kv0 < w_lo_last;
-      float16v s[2], dp[2];
+      float16v s[QB][2], dp[QB][2];
 #pragma unroll
       for (int kvb = 0; kvb < 2; ++kvb) {
-        s[kvb] = float16v{0};
-        dp[kvb] = float16v{0};
+#pragma unroll
+        for (int qb = 0; qb < QB; ++qb) { s[qb][kvb] = float16v{0}; dp[qb][kvb] = float16v{0}; }
 #pragma unroll
         for (int ks = 0; ks < D / 16; ++ks) {
-          const vec8 ak = lds_read8<T>(&Ks[(kvb * 32 + r32) * KS + ks * 16 + g * 8]);
-          s[kvb] = Traits<T>::mfma(ak, qf[ks], s[kvb]);
-          const vec8 av = lds_read8<T>(&Vs[(kvb * 32 + r32) * VS + ks * 16 + g * 8]);
-          dp[kvb] = Traits<T>::mfma(av, dof[ks], dp[kvb]);
+          const vec8 ak = lds_read8<T>(&Kt[(kvb * 32 + r32) * KS + ks * 16 + g * 8]);
+          const vec8 av = lds_read8<T>(&Vt[(kvb * 32 + r32) * VS + ks * 16 + g * 8]);
+#pragma unroll
+          for (int qb = 0; qb < QB; ++qb) {
+            s[qb][kvb] = Traits<T>::mfma(ak, qf[qb][ks], s[qb][kvb]);
+            dp[qb][kvb] = Traits<T>::mfma(av, dof[qb][ks], dp[qb][kvb]);
+          }
+        }
+      }
+      vec8 dsb[QB][4];  // dS^T as B operands: [query block][16-key window]
+#pragma unroll
+      for (int qb = 0; qb < QB; ++qb) {
+        const bool need_mask = kv0 + kKvTile > h_hi_first[qb] || kv0 < h_lo_last[qb];
+#pragma unroll
+        for (int kvb = 0; kvb < 2; ++kvb)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            float pe = exp2_fast(fmaf(s[qb][kvb][i], c, -lse_l[qb]));
+            if (need_mask) {
+              const int kv = kv0 + kvb * 32 + (i >> 2) * 8 + g * 4 + (i & 3);
+              if (kv >= hi_lim[qb] || kv < lo_lim[qb]) pe = 0.f;
+            }
+            s[qb][kvb][i] = pe * (dp[qb][kvb][i] - dsm_l[qb]);  // dS^T
+          }
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          float f[8];
+#pragma unroll
+          for (int j = 0; j < 8; ++j) f[j] = s[qb][w >> 1][(w & 1) * 8 + j];
+          dsb[qb][w] = pack8<T>(f);
         }
       }
 #pragma unroll
-      for (int kvb = 0; kvb < 2; ++kvb)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          float pe = exp2_fast(fmaf(s[kvb][i], c, -lse_l));
-          if (need_mask) {
-            const int kv = kv0 + kvb * 32 + (i >> 2) * 8 + g * 4 + (i & 3);
-            if (kv >= hi_lim || kv < lo_lim) pe = 0.f;
-          }
-          s[kvb][i] = pe * (dp[kvb][i] - dsm_l);  // dS^T
-        }
-#pragma unroll
-      for (int w = 0; w < 4; ++w) {
-        float f[8];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) f[j] = s[w >> 1][(w & 1) * 8 + j];
-        const vec8 dsb = pack8<T>(f);
+      for (int w = 0; w < 4; ++w)
 #pragma unroll
         for (int db = 0; db < D / 32; ++db) {
-          const vec8 a = lds_read_operand_tr<T>(Ks, KS, w * 16, db * 32);
-          dq_acc[db] = Traits<T>::mfma(a, dsb, dq_acc[db]);
+          const vec8 a = lds_read_operand_tr<T>(Kt, KS, w * 16, db * 32);
+#pragma unroll
+          for (int qb = 0; qb < QB; ++qb) dq_acc[qb][db] = Traits<T>::mfma(a, dsb[qb][w], dq_acc[qb][db]);
         }
-      }
     }
-    __syncthreads();
-    if (t + 1 < n_max) { lk.lstore(Ks, KS); lv.lstore(Vs, VS); }
-    __syncthreads();
+    __syncthreads();  // tile t is consumed, tile t+1 is visible
   }
 
-  if (qrow < p.sq) {
-    T *dqg = static_cast<T *>(p.dq) + bi * p.q_bs + (int64_t)qrow * p.q_rs + hi * p.q_hs;
-    typedef T vec4 __attribute__((ext_vector_type(4)));
 #pragma unroll
-    for (int db = 0; db < D / 32; ++db)
+  for (int qb = 0; qb < QB; ++qb) {
+    if (qrow[qb] < p.sq) {
+      T *dqg = static_cast<T *>(p.dq) + bi * p.q_bs + (int64_t)qrow[qb] * p.q_rs + hi * p.q_hs;
+      typedef T vec4 __attribute__((ext_vector_type(4)));
 #pragma unroll
-      for (int i4 = 0; i4 < 4; ++i4) {
-        vec4 a;
+      for (int db = 0; db < D / 32; ++db)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) a[j] = (T)(dq_acc[db][i4 * 4 + j] * p.scale);
-        *reinterpret_cast<vec4 *>(dqg + db * 32 + i4 * 8 + g * 4) = a;
-      }
+        for (int i4 = 0; i4 < 4; ++i4) {
+          vec4 a;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) a[j] = (T)(dq_acc[qb][db][i4 * 4 + j] * p.scale);
+          *reinterpret_cast<vec4 *>(dqg + db * 32 + i4 * 8 + g * 4) = a;
+        }
+    }
   }
 }
+
+// 32-key blocks per wave in dkdv: two where the accumulators fit in the register file
+template <int D> struct DkdvGeom { static constexpr int KB = D <= 64 ? 2 : 1; };
+// 32-query blocks per wave in dq: two blocks cost the second wave per SIMD and measured
+// slower (1.76 ms vs 1.28 ms on the bf16 head_dim-64 benchmark), so one
+template <int D> struct DqGeom { static constexpr int QB = 1; };
 
 template <typename T, int D>
 hipError_t launch_bwd_td(const Params &p, hipStream_t stream) {
@@ -372,10 +465,16 @@ hipError_t launch_bwd_td(const Params &p, hipStream_t stream) {
     constexpr int RPB = 256 / (D / 8);
     dot_do_o_kernel<T, D><<<dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(256), 0, stream>>>(p);
   }
-  if (p.n_nblocks > 0)
-    dkdv_kernel<T, D><<<dim3((unsigned)(p.n_nblocks * p.b * p.h)), dim3(256), 0, stream>>>(p);
-  if (p.n_mblocks > 0)
-    dq_kernel<T, D><<<dim3((unsigned)(p.n_mblocks * p.b * p.h)), dim3(256), 0, stream>>>(p);
+  constexpr int KB = DkdvGeom<D>::KB;
+  Params pk = p;
+  pk.n_nblocks = (p.sk + kKvBlock * KB - 1) / (kKvBlock * KB);
+  if (pk.n_nblocks > 0)
+    dkdv_kernel<T, D, KB><<<dim3((unsigned)(pk.n_nblocks * p.b * p.h)), dim3(256), 0, stream>>>(pk);
+  constexpr int QB = DqGeom<D>::QB;
+  Params pq = p;
+  pq.n_mblocks = (p.sq + kQBlock * QB - 1) / (kQBlock * QB);
+  if (pq.n_mblocks > 0)
+    dq_kernel<T, D, QB><<<dim3((unsigned)(pq.n_mblocks * p.b * p.h)), dim3(256), 0, stream>>>(pq);
   return hipGetLastError();
 }
 
