@@ -187,3 +187,57 @@ def test_flash_blob_packer_matches_oracle():
     blob = ops.pack_flash_args(q, q, q, q, float(np.float32(1 / np.sqrt(128))), (-1, 0))
     a = oracle.fa_args(4, 2048, 2048, 32, 32, 128, 1 / np.sqrt(128), window=(-1, 0))
     assert blob == oracle.fa_pack_args(a).tobytes()
+
+
+PLUGIN_SRC = r"""
+// An op-kernel library outside the runtime: registers one kernel under the ROCm provider from a
+// static initialiser, the way runtime/test/external_kernels/cuda/kernels.cc:91-99 does.
+#include "brt.h"
+namespace {
+class Noop final : public brt::OpKernel {
+public:
+  explicit Noop(const brt::OpKernelInfo &info) : brt::OpKernel(info) {
+    brt::OpAccessor acc(info);
+    BRT_ENFORCE(acc.GetNumArgs() == 2, "test.external_noop takes two operands");
+  }
+  brt::common::Status RunImpl(const brt::ExecutionContext &) override { return brt::common::Status::OK(); }
+};
+void RegisterExternal(brt::KernelRegistry *r) {
+  r->Register("test.external_noop", [](const brt::OpKernelInfo &info) -> std::shared_ptr<brt::OpKernel> {
+    return std::make_shared<Noop>(info);
+  });
+}
+}  // namespace
+BRT_STATIC_KERNEL_REGISTRATION(brt::DeviceKind::ROCM, brt::ProviderType::BRT, RegisterExternal)
+"""
+
+
+def test_external_kernel_library_registers_statically(tmp_path):
+    """ExecutionProvider::StaticRegisterKernelsFromDynlib (execution_provider.cc:29-41; used by
+    runtime/test/unittest_main/test_main.cc:33-35): a library loaded before the session is created
+    adds its kernels to the provider's registry; its constructor-time checks run at load."""
+    import subprocess
+    from byteir_amd import _lib, brt
+    B = _lib.brt()
+    src = tmp_path / "external_kernels.cc"
+    src.write_text(PLUGIN_SRC)
+    lib = tmp_path / "libexternal_kernels.so"
+    libdir = os.path.join(ROOT, "byteir_amd", "lib")
+    subprocess.run(["g++", "-std=c++17", "-O1", "-shared", "-fPIC", f"-I{os.path.join(ROOT, 'byteir_amd', 'csrc', 'brt')}",
+                    str(src), "-o", str(lib), f"-L{libdir}", "-lbrt", f"-Wl,-rpath,{libdir}"], check=True)
+    assert B.brt_register_kernels_from_dynlib(str(tmp_path / "missing.so").encode()) != 0
+    assert B.brt_register_kernels_from_dynlib(str(lib).encode()) == 0, B.brt_last_error().decode()
+    s = brt.Session(device_id=-1)
+    try:
+        assert s.has_kernel("test.external_noop")
+        t = memref([4], "f32", "cuda")
+        mod = f"""func.func @t(%a : {t} {{byre.argname = "a", byre.argtype = 1: i32}},
+                     %b : {t} {{byre.argname = "b", byre.argtype = 2: i32}}) attributes {{byre.entry_point}} {{
+          byre.compute @test.external_noop(%a, %b) : {t}, {t}
+          return }}"""
+        s.load_from_memory(mod)
+        assert s.get_op_keys() == ["test.external_noop"]
+        with pytest.raises(RuntimeError, match="takes two operands"):
+            s.load_from_memory(mod.replace("(%a, %b) : " + t + ", " + t, "(%a) : " + t))
+    finally:
+        s.close()

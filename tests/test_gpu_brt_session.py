@@ -163,3 +163,178 @@ def test_copy_ops_and_listener(session):
     assert np.array_equal(src, dst)
     assert seen == [("cpu2cuda", 0, False), ("cpu2cuda", 0, True), ("cuda2cuda", 1, False), ("cuda2cuda", 1, True),
                     ("cuda2cpu", 2, False), ("cuda2cpu", 2, True)]
+
+
+# ---- request context, frames and work queues -------------------------------------------------
+# Mirrors of CUDARequestContextTest.{NoBindArg,BindArg1,BindArg2}
+# (runtime/test/backends/cuda/providers/default/request_context_test.cc:48-200),
+# BRTInferenceExecutionFrameTest.TestStateInfoSharing (runtime/test/context/exec_frame_test.cc:94)
+# and CUDAWorkQueueTest.{CUDASingleStreamWorkQueue,CUDAExternalStreamWorkQueue}
+# (runtime/test/backends/cuda/device/cuda_work_queue_test.cc:82,190), with a reduction standing in
+# for the reference's AddOp.
+
+def _h2d(ptr, arr):
+    from byteir_amd import _lib
+    K = _lib.kernels()
+    _lib.check(K.brt_rocm_memcpy_h2d(ptr, arr.ctypes.data, arr.nbytes, None))
+    _lib.check(K.brt_rocm_device_synchronize())
+
+
+def _d2h(ptr, shape, dtype=np.float32):
+    from byteir_amd import _lib
+    K = _lib.kernels()
+    out = np.empty(shape, dtype)
+    _lib.check(K.brt_rocm_memcpy_d2h(out.ctypes.data, ptr, out.nbytes, None))
+    _lib.check(K.brt_rocm_device_synchronize())
+    return out
+
+
+def test_request_context_without_binding(session):
+    """Nothing bound: the frame allocates every entry argument, get_arg hands out the pointers."""
+    session.load_from_memory(reduction_module("cuda", [64, 4096], [1], "ReduceMaxOp_f32_f32"))
+    req = session.new_request_context()
+    x = np.random.default_rng(3).standard_normal((64, 4096)).astype(np.float32)
+    p_in, p_out = req.get_arg(0), req.get_arg(1)
+    assert p_in and p_out and p_in != p_out
+    _h2d(p_in, x)
+    req.finish_io_binding()
+    req.run()
+    req.sync()
+    assert req.get_arg(1) == p_out
+    assert np.array_equal(_d2h(p_out, (64,)), x.max(axis=1))
+    req.close()
+
+
+def test_request_context_partial_binding_and_rebinding(session):
+    """One argument bound by the caller, the other owned by the frame; binding over a
+    frame-owned argument releases it; a rebound argument is what the next run uses."""
+    session.load_from_memory(reduction_module("cuda", [64, 4096], [1], "ReduceMaxOp_f32_f32"))
+    req = session.new_request_context()
+    rng = np.random.default_rng(4)
+    x0 = rng.standard_normal((64, 4096)).astype(np.float32)
+    x1 = rng.standard_normal((64, 4096)).astype(np.float32)
+    y = torch.zeros(64, device="cuda")
+    p_in = req.get_arg(0)           # frame-owned input
+    req.bind_arg(1, y.data_ptr())   # caller-owned output
+    _h2d(p_in, x0)
+    req.finish_io_binding()
+    req.run()
+    req.sync()
+    assert np.array_equal(host(y), x0.max(axis=1))
+    dx1 = dev(x1)
+    req.bind_arg(0, dx1.data_ptr())  # replaces (and frees) the frame-owned buffer
+    assert req.get_arg(0) == dx1.data_ptr()
+    req.finish_io_binding()
+    req.run()
+    req.sync()
+    assert np.array_equal(host(y), x1.max(axis=1))
+    req.close()
+
+
+def test_run_before_finish_io_binding_is_an_error(session):
+    session.load_from_memory(reduction_module("cuda", [8, 8], [1], "ReduceSumOp_f32_f32"))
+    req = session.new_request_context()
+    with pytest.raises(RuntimeError, match="FinishIOBinding"):
+        req.run()
+    req.close()
+
+
+def test_two_requests_of_one_session_are_independent(session):
+    """Two frames of one plan: each has its own arguments and its own reduce workspace, runs
+    interleave on two streams."""
+    shape = (16384, 2048)
+    session.load_from_memory(reduction_module("cuda", list(shape), [0], "ReduceSumOp_f32_f32"))
+    reqs, xs, ys = [], [], []
+    gen = torch.Generator(device="cuda").manual_seed(11)
+    for i in range(2):
+        r = session.new_request_context()
+        x = torch.rand(shape, generator=gen, device="cuda") - 0.5
+        y = torch.empty(shape[1], device="cuda")
+        r.bind_arg(0, x.data_ptr())
+        r.bind_arg(1, y.data_ptr())
+        r.finish_io_binding()
+        reqs.append(r), xs.append(x), ys.append(y)
+    torch.cuda.synchronize()
+    for _ in range(3):
+        for r in reqs:
+            r.run()
+    for r in reqs:
+        r.sync()
+    for x, y in zip(xs, ys):
+        want = x.double().sum(dim=0)
+        sabs = x.double().abs().sum(dim=0)
+        assert bool(((y.double() - want).abs() <= 1e-5 * torch.maximum(want.abs(), 1e-2 * sabs)).all())
+    for r in reqs:
+        r.close()
+
+
+def test_workspace_is_allocated_once_per_frame_and_freed_with_it():
+    """The reduce workspace is per-frame state: allocated at the frame's first run through the
+    session's allocator, reused by later runs, released when the request goes away."""
+    from byteir_amd import brt
+    live, allocs = {}, []
+
+    def alloc(n):
+        p = torch.cuda.caching_allocator_alloc(n)
+        live[p] = n
+        allocs.append(n)
+        return p
+
+    def free(p):
+        del live[p]
+        torch.cuda.caching_allocator_delete(p)
+
+    s = brt.Session(device="ROCM", alloc_func=alloc, free_func=free)
+    shape = (16384, 8192)
+    s.load_from_memory(reduction_module("cuda", list(shape), [0], "ReduceMaxOp_f32_f32"))
+    from byteir_amd import ops
+    need = ops.reduce_workspace_bytes(torch.float32, 1, *shape)
+    assert need > 0
+    x = torch.rand(shape, device="cuda")
+    y = torch.empty(shape[1], device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    reqs = []
+    for _ in range(2):
+        r = s.new_request_context(stream)
+        r.bind_arg(0, x.data_ptr())
+        r.bind_arg(1, y.data_ptr())
+        r.finish_io_binding()
+        reqs.append(r)
+    assert allocs == []                      # nothing is allocated before the first run
+    reqs[0].run()
+    assert allocs == [need]
+    for _ in range(3):
+        reqs[0].run()
+    assert allocs == [need]                  # later runs of the same frame reuse it
+    reqs[1].run()
+    assert allocs == [need, need]            # a second frame has its own
+    reqs[0].sync()
+    assert torch.equal(y, x.amax(dim=0))
+    reqs[0].close()
+    assert len(live) == 1
+    reqs[1].close()
+    assert live == {}
+    s.close()
+
+
+def test_external_stream_work_queue_keeps_stream_order(session):
+    """A request on a caller's stream is ordered after the work already enqueued there (the
+    producer of its input) without any host synchronisation; a request that owns its stream is
+    synchronised by its own sync()."""
+    shape = (8192, 8192)
+    session.load_from_memory(reduction_module("cuda", list(shape), [1], "ReduceMaxOp_f32_f32"))
+    side = torch.cuda.Stream()
+    x = torch.zeros(shape, device="cuda")
+    y = torch.zeros(shape[0], device="cuda")
+    torch.cuda.synchronize()
+    req = session.new_request_context(side.cuda_stream)
+    req.bind_arg(0, x.data_ptr())
+    req.bind_arg(1, y.data_ptr())
+    req.finish_io_binding()
+    with torch.cuda.stream(side):
+        for k in range(1, 9):           # eight full passes over 256 MiB, then the reduction, no host wait
+            x.add_(float(k))
+        req.run()
+    req.sync()                          # waits for the caller's stream
+    assert torch.equal(y, torch.full((shape[0],), 36.0, device="cuda"))
+    req.close()
