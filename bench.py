@@ -228,6 +228,15 @@ def main():
                       "loop nests, which cannot be built here)",
             "seconds": round(t_cpu, 3), "host_cores_available": os.cpu_count(),
         }
+        # the same loop nests with OpenMP over the independent outputs, on this job's CPU share
+        n_thr = max(1, min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16"))))
+        oracle.set_threads(n_thr)
+        t_par = cpu_time(lambda: (oracle.reduce_abc(oracle.MAX, xh, 1, R, Cc), oracle.reduce_abc(oracle.SUM, xh, 1, R, Cc),
+                                  oracle.reduce_abc(oracle.MAX, xh, R, Cc, 1), oracle.reduce_abc(oracle.SUM, xh, R, Cc, 1)),
+                         repeat=2)
+        oracle.set_threads(1)
+        result["cpu_baseline"]["openmp"] = {"value": round(step_bytes / t_par / 1e9, 3), "unit": "GB/s", "cores": n_thr,
+                                            "seconds": round(t_par, 3)}
         del xh
 
     if not args.no_extras:

@@ -90,7 +90,10 @@ __global__ void __launch_bounds__(256) dkdv_kernel(const Params p) {
   __shared__ float lse_s[2][kQTile];
   __shared__ float dsm_s[2][kQTile];
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  // the wave index in a scalar register: everything derived from it (row windows, skip and
+  // mask decisions) then stays scalar and branches on it are real branches
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r32 = lane & 31, g = lane >> 5;
   int n_block, bh;
   {
@@ -150,6 +153,10 @@ __global__ void __launch_bounds__(256) dkdv_kernel(const Params p) {
   const int m_min = q_lo / kQTile;
   const int m_max = q_hi > 0 ? (q_hi + kQTile - 1) / kQTile : 0;
   const float c = p.scale_log2;
+  // a key is kept for a query when key - (query + sk - sq) lies in [win_lo, win_lo + win_span]
+  // (mask.h:160-200 of the reference; an unbounded side becomes +-2^30)
+  const int win_lo = p.wl >= 0 ? -p.wl : -(1 << 30);
+  const unsigned win_span = (unsigned)((p.wr >= 0 ? p.wr : (1 << 30)) - win_lo);
 
   TileLoader<T, D, kQTile> lq, ldo;
   float lse_r = 0.f, dsm_r = 0.f;
@@ -183,16 +190,9 @@ __global__ void __launch_bounds__(256) dkdv_kernel(const Params p) {
     if (m + 2 < m_max) gload(m + 2);
     const T *Qt = Qs[buf];
     const T *dOt = dOs[buf];
-#pragma unroll
-    for (int qs = 0; qs < kQTile / 32; ++qs) {
-      const int q0 = m * kQTile + qs * 32;  // first query row of this 32-row sub-tile
-      // wave-uniform visibility of the sub-tile against the wave's keys
-      int lo_first, hi_first, lo_last, hi_last;
-      row_limits(p, q0, lo_first, hi_first);
-      row_limits(p, q0 + 31, lo_last, hi_last);
-      if (wkv0 >= hi_last || wkv0 + 32 * KB <= lo_first) continue;  // nothing kept
-      const bool need_mask = wkv0 + 32 * KB > hi_first || wkv0 < lo_last || q0 + 32 > p.sq;
-
+    // one 32-query sub-tile against the wave's keys; kMask: the window edge crosses it
+    auto sub_tile = [&](auto mask_tag, int qs, int q0) {
+      constexpr bool kMask = decltype(mask_tag)::value;
       float16v s[KB], dp[KB];
 #pragma unroll
       for (int kb = 0; kb < KB; ++kb) { s[kb] = float16v{0}; dp[kb] = float16v{0}; }
@@ -220,11 +220,10 @@ __global__ void __launch_bounds__(256) dkdv_kernel(const Params p) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
           float pe = exp2_fast(fmaf(s[kb][i], c, -lse_q[i]));
-          if (need_mask) {
-            const int ql = qs * 32 + (i >> 2) * 8 + g * 4 + (i & 3);
-            int lo, hi_;
-            row_limits(p, m * kQTile + ql, lo, hi_);
-            if (kvcol[kb] >= hi_ || kvcol[kb] < lo) pe = 0.f;
+          if constexpr (kMask) {
+            // key - (query + sk - sq) must lie in [-wl, wr]: one unsigned compare
+            const unsigned rel = (unsigned)(kvcol[kb] - off - q0 - g * 4 - ((i >> 2) * 8 + (i & 3)) - win_lo);
+            if (rel > win_span) pe = 0.f;
           }
           pv[i] = pe;
           dsv[i] = pe * (dp[kb][i] - dsm_q[i]);
@@ -247,6 +246,17 @@ __global__ void __launch_bounds__(256) dkdv_kernel(const Params p) {
             dk_acc[kb][db] = Traits<T>::mfma(a_q, dsb[kb][w], dk_acc[kb][db]);
           }
         }
+    };
+#pragma unroll
+    for (int qs = 0; qs < kQTile / 32; ++qs) {
+      const int q0 = m * kQTile + qs * 32;  // first query row of this 32-row sub-tile
+      // wave-uniform visibility of the sub-tile against the wave's keys
+      int lo_first, hi_first, lo_last, hi_last;
+      row_limits(p, q0, lo_first, hi_first);
+      row_limits(p, q0 + 31, lo_last, hi_last);
+      if (wkv0 >= hi_last || wkv0 + 32 * KB <= lo_first) continue;  // nothing kept
+      if (wkv0 + 32 * KB > hi_first || wkv0 < lo_last) sub_tile(std::true_type{}, qs, q0);
+      else sub_tile(std::false_type{}, qs, q0);
     }
     __syncthreads();  // tile m is consumed, tile m+1 is visible
   }
@@ -286,7 +296,10 @@ __global__ void __launch_bounds__(256) dq_kernel(const Params p) {
   __shared__ __attribute__((aligned(16))) T Ks[2][kKvTile * KS];
   __shared__ __attribute__((aligned(16))) T Vs[2][kKvTile * VS];
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  // the wave index in a scalar register: everything derived from it (row windows, skip and
+  // mask decisions) then stays scalar and branches on it are real branches
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r32 = lane & 31, g = lane >> 5;
   int m_block, bh;
   {
@@ -400,20 +413,25 @@ __global__ void __launch_bounds__(256) dq_kernel(const Params p) {
         }
       }
       vec8 dsb[QB][4];  // dS^T as B operands: [query block][16-key window]
-#pragma unroll
-      for (int qb = 0; qb < QB; ++qb) {
-        const bool need_mask = kv0 + kKvTile > h_hi_first[qb] || kv0 < h_lo_last[qb];
+      // dS^T = P^T o (dP^T - D) in place of S^T; kMask: the window edge crosses this tile
+      auto ds_tile = [&](auto mask_tag, int qb) {
+        constexpr bool kMask = decltype(mask_tag)::value;
 #pragma unroll
         for (int kvb = 0; kvb < 2; ++kvb)
 #pragma unroll
           for (int i = 0; i < 16; ++i) {
             float pe = exp2_fast(fmaf(s[qb][kvb][i], c, -lse_l[qb]));
-            if (need_mask) {
+            if constexpr (kMask) {
               const int kv = kv0 + kvb * 32 + (i >> 2) * 8 + g * 4 + (i & 3);
               if (kv >= hi_lim[qb] || kv < lo_lim[qb]) pe = 0.f;
             }
-            s[qb][kvb][i] = pe * (dp[qb][kvb][i] - dsm_l[qb]);  // dS^T
+            s[qb][kvb][i] = pe * (dp[qb][kvb][i] - dsm_l[qb]);
           }
+      };
+#pragma unroll
+      for (int qb = 0; qb < QB; ++qb) {
+        if (kv0 + kKvTile > h_hi_first[qb] || kv0 < h_lo_last[qb]) ds_tile(std::true_type{}, qb);
+        else ds_tile(std::false_type{}, qb);
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
           float f[8];
