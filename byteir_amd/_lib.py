@@ -82,7 +82,8 @@ def flash_attn():
     if _flash is None:
         L = _load("libflash_attn.so", ctypes.RTLD_GLOBAL)
         vp = ctypes.c_void_p
-        for n in ("run_flash_attn_fwd", "run_flash_attn_bwd", "run_flash_attn_fwd_bf16", "run_flash_attn_bwd_bf16"):
+        for n in ("run_flash_attn_fwd", "run_flash_attn_bwd", "run_flash_attn_fwd_bf16", "run_flash_attn_bwd_bf16",
+                  "run_flash_attn_kvcache", "run_flash_attn_kvcache_bf16"):
             f = getattr(L, n)
             f.argtypes = [ctypes.POINTER(vp), vp, vp]
             f.restype = None

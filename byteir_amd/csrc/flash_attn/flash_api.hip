@@ -16,6 +16,7 @@
 namespace fa {
 hipError_t launch_fwd(Params &p, int dtype, hipStream_t stream);
 hipError_t launch_bwd(Params &p, int dtype, hipStream_t stream);
+hipError_t launch_append_kv(const Params &p, int dtype, hipStream_t stream);
 }  // namespace fa
 
 namespace {
@@ -91,6 +92,35 @@ int fill(const Blob &a, fa::Params &p) {
   return 0;
 }
 
+// extra_args of run_flash_attn_kvcache (flash_api.cu:727-773): 18 strides, 6 sizes, the scale,
+// 4 sequence lengths, 2 window sizes; 31 fields, 244 bytes, unpadded.
+struct KvBlob {
+  int64_t q_bs, k_bs, v_bs, knew_bs, vnew_bs, o_bs;
+  int64_t q_rs, k_rs, v_rs, knew_rs, vnew_rs, o_rs;
+  int64_t q_hs, k_hs, v_hs, knew_hs, vnew_hs, o_hs;
+  int64_t b, h, h_k, d, d_rounded, seqlen_knew;
+  float softmax_scale;
+  int64_t seqlen_q, seqlen_k, seqlen_q_rounded, seqlen_k_rounded;
+  int64_t window_size_left, window_size_right;
+};
+
+KvBlob parse_kv(const void *extra_args) {
+  const unsigned char *s = static_cast<const unsigned char *>(extra_args);
+  size_t pos = 0;
+  auto i64 = [&]() { int64_t v; memcpy(&v, s + pos, 8); pos += 8; return v; };
+  auto f32 = [&]() { float v; memcpy(&v, s + pos, 4); pos += 4; return v; };
+  KvBlob a;
+  a.q_bs = i64(); a.k_bs = i64(); a.v_bs = i64(); a.knew_bs = i64(); a.vnew_bs = i64(); a.o_bs = i64();
+  a.q_rs = i64(); a.k_rs = i64(); a.v_rs = i64(); a.knew_rs = i64(); a.vnew_rs = i64(); a.o_rs = i64();
+  a.q_hs = i64(); a.k_hs = i64(); a.v_hs = i64(); a.knew_hs = i64(); a.vnew_hs = i64(); a.o_hs = i64();
+  a.b = i64(); a.h = i64(); a.h_k = i64(); a.d = i64(); a.d_rounded = i64(); a.seqlen_knew = i64();
+  a.softmax_scale = f32();
+  a.seqlen_q = i64(); a.seqlen_k = i64(); a.seqlen_q_rounded = i64(); a.seqlen_k_rounded = i64();
+  a.window_size_left = (int32_t)i64();  // read as int (flash_api.cu:771-772)
+  a.window_size_right = (int32_t)i64();
+  return a;
+}
+
 }  // namespace
 
 extern "C" {
@@ -139,6 +169,50 @@ int flash_attn_bwd_checked(void **tensors, const void *extra_args, int dtype, vo
   return fa::launch_bwd(p, dtype, static_cast<hipStream_t>(stream));
 }
 
+int flash_attn_kvcache_checked(void **tensors, const void *extra_args, int dtype, void *stream_) {
+  if (!tensors || !extra_args) return fail("null argument");
+  if (dtype != 1 && dtype != 2) return fail("dtype %d is not supported (1 = fp16, 2 = bf16)", dtype);
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  const KvBlob k = parse_kv(extra_args);
+  Blob a{};
+  a.q_bs = k.q_bs; a.k_bs = k.k_bs; a.v_bs = k.v_bs; a.o_bs = k.o_bs;
+  a.q_rs = k.q_rs; a.k_rs = k.k_rs; a.v_rs = k.v_rs; a.o_rs = k.o_rs;
+  a.q_hs = k.q_hs; a.k_hs = k.k_hs; a.v_hs = k.v_hs; a.o_hs = k.o_hs;
+  a.b = k.b; a.h = k.h; a.h_k = k.h_k; a.d = k.d; a.d_rounded = k.d_rounded;
+  a.softmax_scale = k.softmax_scale;
+  a.seqlen_q = k.seqlen_q; a.seqlen_k = k.seqlen_k;
+  a.seqlen_q_rounded = k.seqlen_q_rounded; a.seqlen_k_rounded = k.seqlen_k_rounded;
+  a.p_dropout = 0.f;
+  a.window_size_left = k.window_size_left; a.window_size_right = k.window_size_right;
+  fa::Params p{};
+  if (int r = fill(a, p)) return r;
+  // tensors: q, k cache, v cache, k new, v new, seqlens_k, o, softmax_lse (flash_api.cu:775-777)
+  p.q = tensors[0]; p.k = tensors[1]; p.v = tensors[2];
+  p.k_new = tensors[3]; p.v_new = tensors[4];
+  p.seqlens_k = static_cast<const int *>(tensors[5]);
+  p.o_w = tensors[6];
+  p.lse = static_cast<float *>(tensors[7]);
+  if (p.b == 0 || p.sq == 0) return 0;
+  if (!p.q || !p.o_w || !p.lse || (p.sk > 0 && (!p.k || !p.v))) return fail("null tensor pointer");
+  if (!aligned16(p.q) || !aligned16(p.k) || !aligned16(p.v) || !aligned16(p.o_w))
+    return fail("q, k, v and o must be 16-byte aligned");
+  if ((p.k_new == nullptr) != (p.v_new == nullptr)) return fail("k_new and v_new must be given together");
+  if (p.k_new) {
+    if (k.seqlen_knew < 0 || k.seqlen_knew > (1 << 30)) return fail("bad seqlen_knew %ld", (long)k.seqlen_knew);
+    if (!p.seqlens_k) return fail("appending to the cache needs seqlens_k");
+    if (!aligned16(p.k_new) || !aligned16(p.v_new)) return fail("k_new and v_new must be 16-byte aligned");
+    const int64_t strides[] = {k.knew_bs, k.vnew_bs, k.knew_rs, k.vnew_rs, k.knew_hs, k.vnew_hs};
+    for (int64_t st : strides)
+      if (st % 8 != 0) return fail("stride %ld is not a multiple of 8 elements (16-byte rows needed)", (long)st);
+    p.seqlen_knew = (int)k.seqlen_knew;
+    p.knew_bs = k.knew_bs; p.vnew_bs = k.vnew_bs; p.knew_rs = k.knew_rs; p.vnew_rs = k.vnew_rs;
+    p.knew_hs = k.knew_hs; p.vnew_hs = k.vnew_hs;
+    if (hipError_t e = fa::launch_append_kv(p, dtype, stream)) return e;
+  }
+  // without seqlens_k every batch attends to all seqlen_k cache rows (BlockInfo, block_info.h:27-37)
+  return fa::launch_fwd(p, dtype, stream);
+}
+
 static void die(const char *who, int r) {
   if (r < 0) fprintf(stderr, "libflash_attn: %s: unsupported arguments: %s\n", who, g_err);
   else fprintf(stderr, "libflash_attn: %s: %s\n", who, hipGetErrorString(static_cast<hipError_t>(r)));
@@ -153,6 +227,12 @@ void run_flash_attn_bwd(void **tensors, void *extra_args, void *stream) {
 }
 void run_flash_attn_fwd_bf16(void **tensors, void *extra_args, void *stream) {
   if (int r = flash_attn_fwd_checked(tensors, extra_args, 2, stream)) die("run_flash_attn_fwd_bf16", r);
+}
+void run_flash_attn_kvcache(void **tensors, void *extra_args, void *stream) {
+  if (int r = flash_attn_kvcache_checked(tensors, extra_args, 1, stream)) die("run_flash_attn_kvcache", r);
+}
+void run_flash_attn_kvcache_bf16(void **tensors, void *extra_args, void *stream) {
+  if (int r = flash_attn_kvcache_checked(tensors, extra_args, 2, stream)) die("run_flash_attn_kvcache_bf16", r);
 }
 void run_flash_attn_bwd_bf16(void **tensors, void *extra_args, void *stream) {
   if (int r = flash_attn_bwd_checked(tensors, extra_args, 2, stream)) die("run_flash_attn_bwd_bf16", r);

@@ -117,14 +117,24 @@ struct Params {
   int wl, wr;                         // window sizes after normalisation; < 0 = unbounded
   int n_mblocks, n_nblocks;
   int xcd_remap;                      // 1: blocks of one (batch, head) share an XCD
+  // key/value cache calls only: per-batch number of keys already in the cache (the cache
+  // holds p.sk rows), rows appended from k_new / v_new before attending
+  const int *seqlens_k;
+  int seqlen_knew;
+  const void *k_new, *v_new;
+  int64_t knew_bs, vnew_bs, knew_rs, vnew_rs, knew_hs, vnew_hs;
 };
 
-// Kept key range [lo, hi) for query row `q` (reference: lib/mask.h:160-200).
-__device__ __forceinline__ void row_limits(const Params &p, int q, int &lo, int &hi) {
-  lo = 0; hi = p.sk;
-  const int off = p.sk - p.sq;
-  if (p.wr >= 0) hi = min(p.sk, q + 1 + off + p.wr);
+// Kept key range [lo, hi) for query row `q` when the sequence has `sk` keys
+// (reference: lib/mask.h:160-200).
+__device__ __forceinline__ void row_limits_sk(const Params &p, int sk, int q, int &lo, int &hi) {
+  lo = 0; hi = sk;
+  const int off = sk - p.sq;
+  if (p.wr >= 0) hi = min(sk, q + 1 + off + p.wr);
   if (p.wl >= 0) lo = max(0, q + off - p.wl);
+}
+__device__ __forceinline__ void row_limits(const Params &p, int q, int &lo, int &hi) {
+  row_limits_sk(p, p.sk, q, lo, hi);
 }
 
 }  // namespace fa

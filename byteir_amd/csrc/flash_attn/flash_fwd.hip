@@ -32,7 +32,8 @@ constexpr int kStages = 3;     // LDS ring depth
 constexpr float kRescaleSlack = 8.0f;
 
 // QB: 32-row halves per wave (1 or 2); NW: waves per workgroup; the workgroup owns 32*QB*NW rows
-template <typename T, int D, int QB, int NW>
+// VarK: the number of keys is read per batch (key/value cache calls): seqlens_k[b] + seqlen_knew
+template <typename T, int D, int QB, int NW, bool VarK>
 __global__ void __launch_bounds__(NW * 64, NW * QB >= 16 ? 2 : (QB == 2 ? 1 : 2)) flash_fwd_kernel(const Params p) {
   constexpr int kThreads = NW * 64;
   constexpr int kBM = 32 * QB * NW;
@@ -62,6 +63,8 @@ __global__ void __launch_bounds__(NW * 64, NW * QB >= 16 ? 2 : (QB == 2 ? 1 : 2)
     m_block = p.n_mblocks - 1 - m_block;  // longest (causal) blocks first
   }
   const int bi = bh / p.h, hi = bh % p.h, hk = hi / (p.h / p.h_k);
+  int sk = p.sk;
+  if constexpr (VarK) sk = min(p.sk, p.seqlens_k[bi] + p.seqlen_knew);
   const int m0 = m_block * kBM;
   const int wq0 = m0 + wave * 32 * QB;
 
@@ -71,15 +74,15 @@ __global__ void __launch_bounds__(NW * 64, NW * QB >= 16 ? 2 : (QB == 2 ? 1 : 2)
 #pragma unroll
   for (int qb = 0; qb < QB; ++qb) {
     qrow[qb] = wq0 + qb * 32 + r32;
-    row_limits(p, qrow[qb], lo_lim[qb], hi_lim[qb]);
-    row_limits(p, wq0 + qb * 32, h_lo_first[qb], h_hi_first[qb]);
-    row_limits(p, wq0 + qb * 32 + 31, h_lo_last[qb], h_hi_last[qb]);
+    row_limits_sk(p, sk, qrow[qb], lo_lim[qb], hi_lim[qb]);
+    row_limits_sk(p, sk, wq0 + qb * 32, h_lo_first[qb], h_hi_first[qb]);
+    row_limits_sk(p, sk, wq0 + qb * 32 + 31, h_lo_last[qb], h_hi_last[qb]);
   }
   const int w_lo_first = h_lo_first[0], w_hi_last = h_hi_last[QB - 1];  // the wave's widest window
   // tile range of the workgroup
   int b_lo, b_hi, t0, t1;
-  row_limits(p, m0, b_lo, t0);
-  row_limits(p, m0 + kBM - 1, t1, b_hi);
+  row_limits_sk(p, sk, m0, b_lo, t0);
+  row_limits_sk(p, sk, m0 + kBM - 1, t1, b_hi);
   const int n_min = b_lo / kBN;
   const int n_max = b_hi > 0 ? (b_hi + kBN - 1) / kBN : 0;
 
@@ -119,7 +122,7 @@ __global__ void __launch_bounds__(NW * 64, NW * QB >= 16 ? 2 : (QB == 2 ? 1 : 2)
   auto gload = [&]() {
 #pragma unroll
     for (int s = 0; s < NP; ++s) {
-      if (ld_on && ld_kv + s * RPP < p.sk) {
+      if (ld_on && ld_kv + s * RPP < sk) {
         kreg[s] = *reinterpret_cast<const uint4 *>(kp + s * k_pass);
         vreg[s] = *reinterpret_cast<const uint4 *>(vp + s * v_pass);
       } else {  // zero rows: 0 * finite stays finite in P V
@@ -322,7 +325,8 @@ hipError_t launch_fwd_d(Params &p, hipStream_t stream) {
   p.n_mblocks = (p.sq + BM - 1) / BM;
   if (p.n_mblocks == 0) return hipSuccess;
   const dim3 grid((unsigned)(p.n_mblocks * p.b * p.h)), block(NW * 64);
-  flash_fwd_kernel<T, D, QB, NW><<<grid, block, 0, stream>>>(p);
+  if (p.seqlens_k) flash_fwd_kernel<T, D, QB, NW, true><<<grid, block, 0, stream>>>(p);
+  else flash_fwd_kernel<T, D, QB, NW, false><<<grid, block, 0, stream>>>(p);
   return hipGetLastError();
 }
 
@@ -334,6 +338,39 @@ hipError_t launch_fwd_t(Params &p, hipStream_t stream) {
   case 128: return launch_fwd_d<T, 128>(p, stream);
   default: return hipErrorInvalidValue;
   }
+}
+
+// Appends k_new / v_new [b, seqlen_knew, h_k, d] to the caches at row seqlens_k[b] of each
+// batch (reference: the Append_KV branch of compute_attn_1rowblock_splitkv,
+// flash_fwd_kernel.h:660-740, without rotary embedding).  One lane copies 16 bytes; rows that
+// would fall beyond the cache's p.sk rows are dropped.
+template <typename T>
+__global__ void __launch_bounds__(256) append_kv_kernel(const Params p) {
+  const int cpr = p.d / 8;  // 16-byte chunks per row
+  const int64_t total = (int64_t)p.b * p.seqlen_knew * p.h_k * cpr;
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= total) return;
+  const int c = (int)(idx % cpr);
+  const int hk = (int)((idx / cpr) % p.h_k);
+  const int i = (int)((idx / ((int64_t)cpr * p.h_k)) % p.seqlen_knew);
+  const int bi = (int)(idx / ((int64_t)cpr * p.h_k * p.seqlen_knew));
+  const int row = p.seqlens_k[bi] + i;
+  if (row < 0 || row >= p.sk) return;
+  const T *ks = static_cast<const T *>(p.k_new) + bi * p.knew_bs + (int64_t)i * p.knew_rs + hk * p.knew_hs + c * 8;
+  const T *vs = static_cast<const T *>(p.v_new) + bi * p.vnew_bs + (int64_t)i * p.vnew_rs + hk * p.vnew_hs + c * 8;
+  T *kd = const_cast<T *>(static_cast<const T *>(p.k)) + bi * p.k_bs + (int64_t)row * p.k_rs + hk * p.k_hs + c * 8;
+  T *vd = const_cast<T *>(static_cast<const T *>(p.v)) + bi * p.v_bs + (int64_t)row * p.v_rs + hk * p.v_hs + c * 8;
+  *reinterpret_cast<uint4 *>(kd) = *reinterpret_cast<const uint4 *>(ks);
+  *reinterpret_cast<uint4 *>(vd) = *reinterpret_cast<const uint4 *>(vs);
+}
+
+hipError_t launch_append_kv(const Params &p, int dtype, hipStream_t stream) {
+  const int64_t total = (int64_t)p.b * p.seqlen_knew * p.h_k * (p.d / 8);
+  if (total == 0) return hipSuccess;
+  const dim3 grid((unsigned)((total + 255) / 256)), block(256);
+  if (dtype == 1) append_kv_kernel<_Float16><<<grid, block, 0, stream>>>(p);
+  else append_kv_kernel<__bf16><<<grid, block, 0, stream>>>(p);
+  return hipGetLastError();
 }
 
 hipError_t launch_fwd(Params &p, int dtype, hipStream_t stream) {

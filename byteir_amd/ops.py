@@ -148,3 +148,34 @@ def flash_attn_bwd(dout, q, k, v, o, lse, scale, window=(-1, -1), stream=None):
     _call_custom(fn, [dout, q, k, v, o, lse, rng, dq, dk, dv, dsm, dq_accum],
                  pack_flash_args(q, k, v, o, scale, window), stream)
     return dq, dk, dv
+
+
+def pack_flash_kvcache_args(q, kcache, vcache, knew, vnew, o, scale, window):
+    """The 244-byte extra_args blob of run_flash_attn_kvcache: 24 i64, f32, 6 i64, unpadded
+    (field order external_libs/runtime/flash_attn/lib/flash_api.cu:727-773).  knew / vnew may
+    be None: their strides and seqlen_knew are then 0."""
+    b, sq, h, d = q.shape
+    sk, h_k = kcache.shape[1], kcache.shape[2]
+    kn = knew if knew is not None else None
+    st = lambda t, i: t.stride(i) if t is not None else 0
+    ints1 = [q.stride(0), kcache.stride(0), vcache.stride(0), st(kn, 0), st(vnew, 0), o.stride(0),
+             q.stride(1), kcache.stride(1), vcache.stride(1), st(kn, 1), st(vnew, 1), o.stride(1),
+             q.stride(2), kcache.stride(2), vcache.stride(2), st(kn, 2), st(vnew, 2), o.stride(2),
+             b, h, h_k, d, round_up(d, 32), knew.shape[1] if knew is not None else 0]
+    ints2 = [sq, sk, round_up(sq, 128), round_up(sk, 128), window[0], window[1]]
+    return struct.pack("<24q", *ints1) + struct.pack("<f", scale) + struct.pack("<6q", *ints2)
+
+
+def flash_attn_kvcache(q, kcache, vcache, knew, vnew, seqlens_k, scale, window=(-1, -1), stream=None):
+    """run_flash_attn_kvcache: tensors {q, k_cache, v_cache, k_new, v_new, seqlens_k, o,
+    softmax_lse} (flash_api.cu:727-811).  Appends knew / vnew to the caches IN PLACE at row
+    seqlens_k[b], then attends to the first seqlens_k[b] + seqlen_knew rows of each batch.
+    seqlens_k: int32 [b] device tensor. -> (o, lse[b,h,sq] f32)."""
+    L = _lib.flash_attn()
+    b, sq, h, d = q.shape
+    o = torch.empty_like(q)
+    lse = torch.empty((b, h, sq), dtype=torch.float32, device=q.device)
+    fn = L.run_flash_attn_kvcache if q.dtype == torch.float16 else L.run_flash_attn_kvcache_bf16
+    _call_custom(fn, [q, kcache, vcache, knew, vnew, seqlens_k, o, lse],
+                 pack_flash_kvcache_args(q, kcache, vcache, knew, vnew, o, scale, window), stream)
+    return o, lse

@@ -53,11 +53,28 @@ void run_flash_attn_bwd(void **tensors, void *extra_args, void *stream);
 void run_flash_attn_fwd_bf16(void **tensors, void *extra_args, void *stream);
 void run_flash_attn_bwd_bf16(void **tensors, void *extra_args, void *stream);
 
-/* Error-returning forms of the four calls above: 0 on success, a positive hipError_t when a
+/* Decoding against a key/value cache: run_flash_attn_kvcache of the reference
+ * (flash_api.cu:727-811 -> run_mha_fwd_with_kvcache :434-567).
+ * tensors: {q, k_cache, v_cache, k_new, v_new, seqlens_k, o, softmax_lse}.
+ *   q [b, seqlen_q, h, d]; k_cache, v_cache [b, seqlen_k, h_k, d] (seqlen_k = capacity);
+ *   k_new, v_new [b, seqlen_knew, h_k, d]; seqlens_k int32 [b] = rows already valid per batch.
+ * First k_new / v_new are written into the caches at rows seqlens_k[b] .. +seqlen_knew (in
+ * place), then q attends to rows [0, seqlens_k[b] + seqlen_knew) of its batch, with the window
+ * aligned to the end of that range (block_info.h:27-37, mask.h:160-200).  No rotary embedding
+ * (the reference sets rotary_dim = 0), one split.  k_new / v_new may both be NULL (no append);
+ * seqlens_k may be NULL only then (all seqlen_k rows are attended).
+ * extra_args (244 bytes): i64 q,k,v,knew,vnew,o batch_stride; the same six row_strides; the
+ * same six head_strides; i64 b, h, h_k, d, d_rounded, seqlen_knew; f32 softmax_scale;
+ * i64 seqlen_q, seqlen_k, seqlen_q_rounded, seqlen_k_rounded; i64 window_size_left, _right. */
+void run_flash_attn_kvcache(void **tensors, void *extra_args, void *stream);
+void run_flash_attn_kvcache_bf16(void **tensors, void *extra_args, void *stream);
+
+/* Error-returning forms of the calls above: 0 on success, a positive hipError_t when a
  * launch failed, -1 when the arguments are unsupported (reason copied to a thread-local
  * buffer readable through flash_attn_last_error()).  dtype: 1 = fp16, 2 = bf16. */
 int flash_attn_fwd_checked(void **tensors, const void *extra_args, int dtype, void *stream);
 int flash_attn_bwd_checked(void **tensors, const void *extra_args, int dtype, void *stream);
+int flash_attn_kvcache_checked(void **tensors, const void *extra_args, int dtype, void *stream);
 const char *flash_attn_last_error(void);
 
 #ifdef __cplusplus

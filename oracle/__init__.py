@@ -271,3 +271,45 @@ def flash_bwd(dout, q, k, v, o, lse, scale, window=(-1, -1), round_p=True):
     lib().oracle_flash_bwd(ctypes.byref(a), _code(q), int(round_p), _p(dout), _p(q), _p(k), _p(v),
                            _p(o), _p(lse), _p(dq), _p(dk), _p(dv), _p(dsm))
     return dq, dk, dv, dsm
+
+
+def fa_kvcache_pack_args(b, sq, sk, h, h_k, d, seqlen_knew, scale, window=(-1, -1)):
+    """The 244-byte extra_args blob of run_flash_attn_kvcache for dense [b, s, h, d] tensors:
+    18 strides (q, k, v, knew, vnew, o: batch, then row, then head), b, h, h_k, d, d_rounded,
+    seqlen_knew as i64, the scale as f32, seqlen_q, seqlen_k, their roundings to 128 and the
+    two window sizes as i64, no padding
+    (external_libs/runtime/flash_attn/lib/flash_api.cu:727-773)."""
+    import struct
+    qb, kb, nb = sq * h * d, sk * h_k * d, seqlen_knew * h_k * d
+    ints1 = [qb, kb, kb, nb, nb, qb,
+             h * d, h_k * d, h_k * d, h_k * d, h_k * d, h * d,
+             d, d, d, d, d, d,
+             b, h, h_k, d, round_up(d, 32), seqlen_knew]
+    ints2 = [sq, sk, round_up(sq, 128), round_up(sk, 128), window[0], window[1]]
+    return np.frombuffer(struct.pack("<24q", *ints1) + struct.pack("<f", scale) + struct.pack("<6q", *ints2),
+                         dtype=np.uint8).copy()
+
+
+def flash_kvcache(q, kcache, vcache, knew, vnew, seqlens_k, scale, window=(-1, -1), round_p=True):
+    """Decoding against a key/value cache as run_mha_fwd_with_kvcache does it
+    (flash_api.cu:434-567; BlockInfo, block_info.h:27-37; the Append_KV branch,
+    flash_fwd_kernel.h:660-740, with rotary_dim = 0): per batch, rows
+    [seqlens_k[b], seqlens_k[b] + seqlen_knew) of the caches are overwritten with knew / vnew,
+    then q attends to rows [0, seqlens_k[b] + seqlen_knew) with the window aligned to the end
+    of that range.  Restated on top of flash_fwd, one batch at a time.
+    -> (o, lse [b,h,sq] f32, kcache_out, vcache_out); the inputs are not modified."""
+    kc, vc = np.array(kcache, copy=True), np.array(vcache, copy=True)
+    b, sq, h, d = q.shape
+    n_new = 0 if knew is None else knew.shape[1]
+    o = np.empty_like(q)
+    lse = np.empty((b, h, sq), dtype=np.float32)
+    for bi in range(b):
+        n0 = int(seqlens_k[bi]) if seqlens_k is not None else kc.shape[1]
+        if knew is not None:
+            top = min(n0 + n_new, kc.shape[1])
+            kc[bi, n0:top] = knew[bi, :top - n0]
+            vc[bi, n0:top] = vnew[bi, :top - n0]
+        n = min(n0 + n_new, kc.shape[1])
+        ob, lb, _ = flash_fwd(q[bi:bi + 1], kc[bi:bi + 1, :n], vc[bi:bi + 1, :n], scale, window, round_p)
+        o[bi], lse[bi] = ob[0], lb[0]
+    return o, lse, kc, vc

@@ -241,3 +241,16 @@ def test_external_kernel_library_registers_statically(tmp_path):
             s.load_from_memory(mod.replace("(%a, %b) : " + t + ", " + t, "(%a) : " + t))
     finally:
         s.close()
+
+
+def test_reference_kvcache_module_loads_unchanged(session, golden_dir):
+    """flash_attn_kvcache.mlir of the reference: eight operands (one of them memref<2xi32>), the
+    library is found by file name, the 244-byte blob is what the oracle packs."""
+    import oracle
+    session.load(os.path.join(golden_dir, "flash_attn_kvcache.mlir"))
+    assert session.get_op_keys() == ["custom"]
+    assert session.get_arg_num() == 8
+    assert session.get_static_shape(5) == [2] and session.get_data_type(5) == "int32"
+    assert session.get_static_shape(1) == [2, 128, 3, 32]
+    blob = session.get_op_attr_blob(0, "extra_args")
+    assert blob == oracle.fa_kvcache_pack_args(2, 1, 128, 3, 3, 32, 1, 0.5, (-1, -1)).tobytes()

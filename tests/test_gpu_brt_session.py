@@ -338,3 +338,23 @@ def test_external_stream_work_queue_keeps_stream_order(session):
     req.sync()                          # waits for the caller's stream
     assert torch.equal(y, torch.full((shape[0],), 36.0, device="cuda"))
     req.close()
+
+
+def test_flash_attn_kvcache_module_unchanged(session, golden_dir):
+    """SM80CUDATestFlashAttnKVCache.Basic through the session: the reference's module text and
+    data, all eight arguments bound (flash_attn_fwd_test.cc:183-330)."""
+    session.load(os.path.join(golden_dir, "flash_attn_kvcache.mlir"))
+    req = session.new_request_context(torch.cuda.current_stream().cuda_stream)
+    g = {n: np.load(os.path.join(golden_dir, f"fa_kv_{n}.npy")) for n in
+         ("q", "knew", "vnew", "kcache", "vcache", "out", "kcache_out", "vcache_out", "seqlens")}
+    q, kc, vc, kn, vn, lens = (dev(g[n]) for n in ("q", "kcache", "vcache", "knew", "vnew", "seqlens"))
+    o = torch.zeros_like(q)
+    lse = torch.zeros((2, 3, 1), device="cuda")
+    for i, t in enumerate((q, kc, vc, kn, vn, lens, o, lse)):
+        req.bind_arg(i, t.data_ptr())
+    req.finish_io_binding()
+    req.run()
+    req.sync()
+    got, want = host(o).astype(np.float32), g["out"].astype(np.float32)
+    assert np.all(np.abs(got - want) <= 2.0 ** -10 * np.abs(want) + 1e-7)  # one fp16 ulp
+    assert np.array_equal(host(kc), g["kcache_out"]) and np.array_equal(host(vc), g["vcache_out"])

@@ -214,3 +214,81 @@ def test_baseline_config5_forward_backward_full_size():
     lhs = dv.float().sum(dim=1)
     rhs = do.float().sum(dim=1)
     assert float((lhs - rhs).abs().max()) <= 0.5  # 8192 bf16-rounded terms per entry
+
+
+# ---- key/value cache ----------------------------------------------------------------------------
+def test_kvcache_reference_golden_vectors(golden_dir):
+    """SM80CUDATestFlashAttnKVCache.Basic (flash_attn_fwd_test.cc:183-330): the new key and
+    value land in row 64 of each batch's cache, the output is attention over 65 rows."""
+    from byteir_amd import ops
+    g = {n: np.load(os.path.join(golden_dir, f"fa_kv_{n}.npy")) for n in
+         ("q", "knew", "vnew", "kcache", "vcache", "out", "kcache_out", "vcache_out", "seqlens")}
+    kc, vc = dev(g["kcache"]), dev(g["vcache"])
+    o, lse = ops.flash_attn_kvcache(dev(g["q"]), kc, vc, dev(g["knew"]), dev(g["vnew"]), dev(g["seqlens"]), 0.5)
+    assert np.array_equal(host(kc), g["kcache_out"])
+    assert np.array_equal(host(vc), g["vcache_out"])
+    d = ulp_diff_f16(host(o), g["out"])
+    assert d.max() <= 1, int(d.max())
+    _, lse_ref, _, _ = oracle.flash_kvcache(g["q"], g["kcache"], g["vcache"], g["knew"], g["vnew"], g["seqlens"], 0.5)
+    np.testing.assert_allclose(host(lse), lse_ref, atol=1e-4, rtol=1e-5)
+
+
+KV_CASES = [
+    # b, sq, h, h_k, d, capacity, n_new, seqlens, window, append
+    (3, 1, 4, 4, 64, 200, 1, [0, 77, 199], (-1, -1), True),
+    (2, 5, 8, 2, 128, 300, 5, [295, 12], (-1, 0), True),       # causal over the appended block, GQA
+    (4, 16, 2, 2, 32, 1024, 16, [1000, 3, 500, 64], (-1, 0), True),
+    (2, 3, 4, 4, 64, 130, 0, [130, 1], (-1, -1), False),        # no append: read-only cache
+    (2, 2, 4, 1, 64, 520, 2, [518, 300], (64, 0), True),        # sliding window, MQA
+]
+
+
+@pytest.mark.parametrize("code", [oracle.F16, oracle.BF16])
+@pytest.mark.parametrize("case", KV_CASES)
+def test_kvcache_matches_oracle(case, code):
+    from byteir_amd import ops
+    b, sq, h, h_k, d, cap, n_new, lens, window, append = case
+    rng = np.random.default_rng(abs(hash(case[:7])) % (2 ** 32))
+    mk = lambda *s: oracle.from_f32(rng.standard_normal(s).astype(np.float32), code)
+    q, kc, vc = mk(b, sq, h, d), mk(b, cap, h_k, d), mk(b, cap, h_k, d)
+    kn, vn = (mk(b, n_new, h_k, d), mk(b, n_new, h_k, d)) if append else (None, None)
+    lens = np.array(lens, dtype=np.int32)
+    scale = 1.0 / np.sqrt(d)
+    bf = code == oracle.BF16
+    dkc, dvc = dev(kc), dev(vc)
+    o, lse = ops.flash_attn_kvcache(dev(q), dkc, dvc, dev(kn) if append else None,
+                                    dev(vn) if append else None, dev(lens), scale, window)
+    o_ref, lse_ref, kc_ref, vc_ref = oracle.flash_kvcache(q, kc, vc, kn, vn, lens, scale, window)
+    o32, _, _, _ = oracle.flash_kvcache(q, kc, vc, kn, vn, lens, scale, window, round_p=False)
+    assert np.array_equal(host(dkc), kc_ref) and np.array_equal(host(dvc), vc_ref)
+    got = oracle.to_f32(host(o))
+    assert np.abs(got - oracle.to_f32(o32)).max() <= ATOL
+    ulp = 2.0 ** -7 if bf else 2.0 ** -10
+    assert np.all(np.abs(got - oracle.to_f32(o_ref)) <= 2 * ulp * np.abs(oracle.to_f32(o_ref)) + 2e-3)
+    np.testing.assert_allclose(host(lse), lse_ref, atol=2e-3, rtol=1e-4)
+
+
+def test_kvcache_unsupported_arguments_are_reported_not_run():
+    import ctypes
+    from byteir_amd import _lib, ops
+    L = _lib.flash_attn()
+    L.flash_attn_kvcache_checked.argtypes = [ctypes.POINTER(ctypes.c_void_p), ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p]
+    L.flash_attn_last_error.restype = ctypes.c_char_p
+    q = torch.zeros((1, 1, 2, 64), dtype=torch.float16, device="cuda")
+    kc = torch.zeros((1, 64, 2, 64), dtype=torch.float16, device="cuda")
+    kn = torch.zeros((1, 1, 2, 64), dtype=torch.float16, device="cuda")
+    o = torch.zeros_like(q)
+    lse = torch.zeros((1, 2, 1), device="cuda")
+    blob = ops.pack_flash_kvcache_args(q, kc, kc, kn, kn, o, 0.1, (-1, -1))
+    buf = ctypes.create_string_buffer(blob, len(blob))
+    # appending without seqlens_k
+    arr = (ctypes.c_void_p * 8)(q.data_ptr(), kc.data_ptr(), kc.data_ptr(), kn.data_ptr(), kn.data_ptr(), None,
+                                o.data_ptr(), lse.data_ptr())
+    assert L.flash_attn_kvcache_checked(arr, ctypes.cast(buf, ctypes.c_void_p), 1, None) == -1
+    assert b"seqlens_k" in L.flash_attn_last_error()
+    # k_new without v_new
+    lens = torch.zeros(1, dtype=torch.int32, device="cuda")
+    arr = (ctypes.c_void_p * 8)(q.data_ptr(), kc.data_ptr(), kc.data_ptr(), kn.data_ptr(), None, lens.data_ptr(),
+                                o.data_ptr(), lse.data_ptr())
+    assert L.flash_attn_kvcache_checked(arr, ctypes.cast(buf, ctypes.c_void_p), 1, None) == -1
+    torch.cuda.synchronize()

@@ -185,3 +185,69 @@ def test_extra_args_blob_known_answer():
     # BASELINE config 4 strides
     c4 = oracle.fa_args(4, 2048, 2048, 32, 32, 128, 1 / np.sqrt(128), window=(-1, 0))
     assert (c4.q_batch_stride, c4.q_row_stride, c4.q_head_stride) == (8388608, 4096, 128)
+
+
+# ---- key/value cache (run_flash_attn_kvcache) -------------------------------------------------
+def load_kv_golden(golden_dir):
+    g = {n: np.load(os.path.join(golden_dir, f"fa_kv_{n}.npy")) for n in
+         ("q", "knew", "vnew", "kcache", "vcache", "out", "kcache_out", "vcache_out", "seqlens")}
+    return g
+
+
+def test_kvcache_golden_inputs_are_the_documented_closed_form(golden_dir):
+    # generate_flash_attn_ground_truth.py:56-74: arange/30000, /40000, /50000; 64 valid rows
+    g = load_kv_golden(golden_dir)
+    small, cache = torch.arange(2 * 1 * 3 * 32, dtype=torch.float16), torch.arange(2 * 128 * 3 * 32, dtype=torch.float16)
+    assert np.array_equal(g["q"], (small / 30000).numpy().reshape(2, 1, 3, 32))
+    assert np.array_equal(g["knew"], (small / 40000).numpy().reshape(2, 1, 3, 32))
+    assert np.array_equal(g["vnew"], (small / 50000).numpy().reshape(2, 1, 3, 32))
+    assert np.array_equal(g["kcache"], (cache / 40000).numpy().reshape(2, 128, 3, 32))
+    assert np.array_equal(g["vcache"], (cache / 50000).numpy().reshape(2, 128, 3, 32))
+    assert g["seqlens"].tolist() == [64, 64]
+
+
+def test_kvcache_against_reference_golden_vectors(golden_dir):
+    """SM80CUDATestFlashAttnKVCache.Basic (flash_attn_fwd_test.cc:183-330): output and both
+    updated caches.  The caches must match exactly (a copy); the output within one fp16 ulp."""
+    g = load_kv_golden(golden_dir)
+    o, lse, kc, vc = oracle.flash_kvcache(g["q"], g["kcache"], g["vcache"], g["knew"], g["vnew"], g["seqlens"], 0.5)
+    assert np.array_equal(kc, g["kcache_out"])
+    assert np.array_equal(vc, g["vcache_out"])
+    # only row 64 of each batch changed, and it now holds the new key / value
+    assert np.array_equal(kc[:, 64], g["knew"][:, 0]) and np.array_equal(kc[:, :64], g["kcache"][:, :64])
+    assert np.array_equal(kc[:, 65:], g["kcache"][:, 65:])
+    d = ulp_diff_f16(o, g["out"])
+    assert d.max() <= 1, d.max()
+    assert np.all(np.isfinite(lse))
+
+
+def test_kvcache_equals_plain_attention_over_the_valid_rows():
+    """Closed form: decoding against a cache is plain attention over the concatenation of the
+    valid cache rows and the new rows, per batch, causal aligned to the end."""
+    rng = np.random.default_rng(5)
+    b, sq, h, h_k, d, cap, n_new = 3, 4, 4, 2, 32, 96, 4
+    q = rng.standard_normal((b, sq, h, d)).astype(np.float16)
+    kc = rng.standard_normal((b, cap, h_k, d)).astype(np.float16)
+    vc = rng.standard_normal((b, cap, h_k, d)).astype(np.float16)
+    kn = rng.standard_normal((b, n_new, h_k, d)).astype(np.float16)
+    vn = rng.standard_normal((b, n_new, h_k, d)).astype(np.float16)
+    lens = np.array([0, 17, 92], dtype=np.int32)
+    o, lse, kc2, vc2 = oracle.flash_kvcache(q, kc, vc, kn, vn, lens, 0.3, window=(-1, 0))
+    for bi in range(b):
+        n = int(lens[bi])
+        kk = np.concatenate([kc[bi, :n], kn[bi]])[None]
+        vv = np.concatenate([vc[bi, :n], vn[bi]])[None]
+        ob, lb, _ = oracle.flash_fwd(q[bi:bi + 1], kk, vv, 0.3, window=(-1, 0))
+        assert np.array_equal(o[bi], ob[0]) and np.array_equal(lse[bi], lb[0])
+        assert np.array_equal(kc2[bi, :n + n_new], kk[0]) and np.array_equal(kc2[bi, n + n_new:], kc[bi, n + n_new:])
+    # the inputs are left alone
+    assert not np.array_equal(kc2, kc)
+
+
+def test_kvcache_extra_args_blob_known_answer():
+    # runtime/test/test_files/flash_attn_kvcache.mlir:11 extra_args, packed as
+    # OpAccessor::GetAttrAsVoidPtr does (op_accessor.cc:212-242)
+    fields = [96, 12288, 12288, 96, 96, 96] + [96] * 6 + [32] * 6 + [2, 3, 3, 32, 32, 1, 0.5, 1, 128, 128, 128, -1, -1]
+    want = b"".join(struct.pack("<f", f) if isinstance(f, float) else struct.pack("<q", f) for f in fields)
+    assert len(want) == 244
+    assert oracle.fa_kvcache_pack_args(2, 1, 128, 3, 3, 32, 1, 0.5, (-1, -1)).tobytes() == want
