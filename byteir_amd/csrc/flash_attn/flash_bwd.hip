@@ -52,21 +52,35 @@ constexpr int kQTile = 64;     // query rows per LDS tile in dkdv
 constexpr int kQBlock = 128;   // queries per workgroup in dq (32 per wave)
 constexpr int kKvTile = 64;    // key rows per LDS tile in dq
 
-// copies a [ROWS x D] tile (rows row0.. of a [n_rows, D] strided matrix) into registers
+// Streams consecutive [ROWS x D] tiles of a [n_rows, D] strided matrix through registers: a
+// running pointer to this thread's first chunk of the next tile, advanced by one tile per
+// gload, instead of a 64-bit address computation per load.
 template <typename T, int D, int ROWS>
 struct TileLoader {
   static constexpr int CPR = D / 8;
   static constexpr int RPP = 256 / CPR;
   static constexpr int NP = ROWS / RPP;
   uint4 reg[NP];
-  __device__ __forceinline__ void gload(const T *base, int64_t row_stride, int row0, int n_rows) {
+  const T *ptr;
+  int64_t pass_stride, tile_stride;
+  int row, n_rows;
+  // the first gload fetches the tile that starts at row0
+  __device__ __forceinline__ void start(const T *base, int64_t row_stride, int row0, int n_rows_) {
     const int c = threadIdx.x % CPR, r = threadIdx.x / CPR;
+    row = row0 + r;
+    n_rows = n_rows_;
+    ptr = base + (int64_t)row * row_stride + c * 8;
+    pass_stride = (int64_t)RPP * row_stride;
+    tile_stride = (int64_t)ROWS * row_stride;
+  }
+  __device__ __forceinline__ void gload() {
 #pragma unroll
     for (int s = 0; s < NP; ++s) {
-      const int row = row0 + s * RPP + r;
-      if (row < n_rows) reg[s] = *reinterpret_cast<const uint4 *>(base + (int64_t)row * row_stride + c * 8);
+      if (row + s * RPP < n_rows) reg[s] = *reinterpret_cast<const uint4 *>(ptr + s * pass_stride);
       else reg[s] = uint4{0, 0, 0, 0};
     }
+    ptr += tile_stride;
+    row += ROWS;
   }
   __device__ __forceinline__ void lstore(T *tile, int stride) const {
     const int c = threadIdx.x % CPR, r = threadIdx.x / CPR;
@@ -159,10 +173,12 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) dkdv_kernel(const Params
   const unsigned win_span = (unsigned)((p.wr >= 0 ? p.wr : (1 << 30)) - win_lo);
 
   TileLoader<T, D, kQTile> lq, ldo;
+  lq.start(qg, p.q_rs, m_min * kQTile, p.sq);
+  ldo.start(dog, p.o_rs, m_min * kQTile, p.sq);
   float lse_r = 0.f, dsm_r = 0.f;
-  auto gload = [&](int m) {
-    lq.gload(qg, p.q_rs, m * kQTile, p.sq);
-    ldo.gload(dog, p.o_rs, m * kQTile, p.sq);
+  auto gload = [&](int m) {  // tiles are fetched in order, m_min first
+    lq.gload();
+    ldo.gload();
     if (tid < kQTile) {
       const int q = m * kQTile + tid;
       lse_r = q < p.sq ? lse_g[q] : INFINITY;  // +inf: the row contributes P = 0
@@ -190,10 +206,9 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) dkdv_kernel(const Params
     if (m + 2 < m_max) gload(m + 2);
     const T *Qt = Qs[buf];
     const T *dOt = dOs[buf];
-    // one 32-query sub-tile against the wave's keys; kMask: the window edge crosses it
-    auto sub_tile = [&](auto mask_tag, int qs, int q0) {
-      constexpr bool kMask = decltype(mask_tag)::value;
-      float16v s[KB], dp[KB];
+    // S = Q K^T and dP = dO V^T of one 32-query sub-tile (the zero accumulators stay next to
+    // their first MFMA, which then takes the constant 0 as its C operand)
+    auto scores = [&](int qs, float16v (&s)[KB], float16v (&dp)[KB]) {
 #pragma unroll
       for (int kb = 0; kb < KB; ++kb) { s[kb] = float16v{0}; dp[kb] = float16v{0}; }
 #pragma unroll
@@ -206,6 +221,13 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) dkdv_kernel(const Params
           dp[kb] = Traits<T>::mfma(ad, vf[kb][ks], dp[kb]);
         }
       }
+    };
+    // P and dS of the sub-tile as packed B operands [key block][16-query window]; kMask: the
+    // window edge crosses it.  Only this vector part exists twice: the accumulating MFMAs
+    // follow after the two variants have joined, so that dK / dV keep one set of registers.
+    auto softmax_grad = [&](auto mask_tag, int qs, int q0, float16v (&s)[KB], float16v (&dp)[KB],
+                            vec8 (&pb)[KB][2], vec8 (&dsb)[KB][2]) {
+      constexpr bool kMask = decltype(mask_tag)::value;
       float lse_q[16], dsm_q[16];
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
@@ -213,7 +235,6 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) dkdv_kernel(const Params
         lse_q[i] = lse_s[buf][ql];
         dsm_q[i] = dsm_s[buf][ql];
       }
-      vec8 pb[KB][2], dsb[KB][2];  // P and dS as B operands: [key block][16-query window]
 #pragma unroll
       for (int kb = 0; kb < KB; ++kb) {
         float pv[16], dsv[16];
@@ -234,6 +255,9 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) dkdv_kernel(const Params
           dsb[kb][w] = pack8<T>(&dsv[w * 8]);
         }
       }
+    };
+    // dV^T += dO^T P, dK^T += Q^T dS
+    auto accumulate = [&](int qs, const vec8 (&pb)[KB][2], const vec8 (&dsb)[KB][2]) {
 #pragma unroll
       for (int w = 0; w < 2; ++w)
 #pragma unroll
@@ -255,8 +279,12 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) dkdv_kernel(const Params
       row_limits(p, q0, lo_first, hi_first);
       row_limits(p, q0 + 31, lo_last, hi_last);
       if (wkv0 >= hi_last || wkv0 + 32 * KB <= lo_first) continue;  // nothing kept
-      if (wkv0 + 32 * KB > hi_first || wkv0 < lo_last) sub_tile(std::true_type{}, qs, q0);
-      else sub_tile(std::false_type{}, qs, q0);
+      float16v s[KB], dp[KB];
+      scores(qs, s, dp);
+      vec8 pb[KB][2], dsb[KB][2];
+      if (wkv0 + 32 * KB > hi_first || wkv0 < lo_last) softmax_grad(std::true_type{}, qs, q0, s, dp, pb, dsb);
+      else softmax_grad(std::false_type{}, qs, q0, s, dp, pb, dsb);
+      accumulate(qs, pb, dsb);
     }
     __syncthreads();  // tile m is consumed, tile m+1 is visible
   }
@@ -372,15 +400,17 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) dq_kernel(const Params p
   const float c = p.scale_log2;
 
   // double-buffered tiles, one barrier per tile (see dkdv_kernel)
-  TileLoader<T, D, kKvTile> lk, lv;
+  TileLoader<T, D, kKvTile> lk, lv;  // tiles are fetched in order, n_min first
+  lk.start(kg, p.k_rs, n_min * kKvTile, p.sk);
+  lv.start(vg, p.v_rs, n_min * kKvTile, p.sk);
   if (n_min < n_max) {
-    lk.gload(kg, p.k_rs, n_min * kKvTile, p.sk);
-    lv.gload(vg, p.v_rs, n_min * kKvTile, p.sk);
+    lk.gload();
+    lv.gload();
     lk.lstore(Ks[0], KS);
     lv.lstore(Vs[0], VS);
     if (n_min + 1 < n_max) {
-      lk.gload(kg, p.k_rs, (n_min + 1) * kKvTile, p.sk);
-      lv.gload(vg, p.v_rs, (n_min + 1) * kKvTile, p.sk);
+      lk.gload();
+      lv.gload();
     }
     __syncthreads();
   }
@@ -389,8 +419,8 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) dq_kernel(const Params p
     const int kv0 = t * kKvTile;
     if (t + 1 < n_max) { lk.lstore(Ks[buf ^ 1], KS); lv.lstore(Vs[buf ^ 1], VS); }
     if (t + 2 < n_max) {
-      lk.gload(kg, p.k_rs, (t + 2) * kKvTile, p.sk);
-      lv.gload(vg, p.v_rs, (t + 2) * kKvTile, p.sk);
+      lk.gload();
+      lv.gload();
     }
     const T *Kt = Ks[buf];
     const T *Vt = Vs[buf];

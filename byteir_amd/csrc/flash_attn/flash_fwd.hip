@@ -148,9 +148,9 @@ __global__ void __launch_bounds__(NW * 64, NW * QB >= 16 ? 2 : (QB == 2 ? 1 : 2)
   for (int qb = 0; qb < QB; ++qb)
 #pragma unroll
     for (int i = 0; i < D / 32; ++i) o_acc[qb][i] = float16v{0};
-  float m_run[QB], l_run[QB];
+  float m_run[QB], ms_run[QB], l_run[QB];  // reference maximum, the same times scale*log2e (0 for -inf), row sum
 #pragma unroll
-  for (int qb = 0; qb < QB; ++qb) { m_run[qb] = -INFINITY; l_run[qb] = 0.f; }
+  for (int qb = 0; qb < QB; ++qb) { m_run[qb] = -INFINITY; ms_run[qb] = 0.f; l_run[qb] = 0.f; }
   const float c = p.scale_log2;
   const int k_rd = r32 * KS + g * 8;  // this lane's K fragment offset inside a 32-row block
 
@@ -188,16 +188,19 @@ __global__ void __launch_bounds__(NW * 64, NW * QB >= 16 ? 2 : (QB == 2 ? 1 : 2)
       float mx = -INFINITY;
 #pragma unroll
       for (int i = 0; i < 16; ++i) mx = fmaxf(mx, sc[i]);
-      mx = fmaxf(mx, partner32(mx));
-      // raise the reference maximum only when it would grow by more than the slack
-      const bool grow = (mx - m_run[qb]) * c > kRescaleSlack;  // false for -inf - -inf (NaN)
-      const bool first = m_run[qb] == -INFINITY && mx != -INFINITY;
-      if (__builtin_amdgcn_ballot_w64(grow || first) != 0) {
-        const float m_new = (grow || first) ? mx : m_run[qb];
+      // Raise the reference maximum only when it would grow by more than the slack.  The test
+      // is made on this lane's half of the keys first: +inf for the first finite score of a
+      // row (m_run = -inf), NaN (false) for -inf - -inf; only when some lane of the wave
+      // fires do the two lanes of a row exchange their maxima.
+      if (__builtin_amdgcn_ballot_w64((mx - m_run[qb]) * c > kRescaleSlack) != 0) {
+        mx = fmaxf(mx, partner32(mx));
+        const bool grow = (mx - m_run[qb]) * c > kRescaleSlack;
+        const float m_new = grow ? mx : m_run[qb];
         const float m_use = m_new == -INFINITY ? 0.f : m_new;
         const float alpha = exp2_fast((m_run[qb] - m_use) * c);
         l_run[qb] *= alpha;
         m_run[qb] = m_new;
+        ms_run[qb] = m_use * c;
 #pragma unroll
         for (int db = 0; db < D / 32; ++db)
 #pragma unroll
@@ -211,7 +214,7 @@ __global__ void __launch_bounds__(NW * 64, NW * QB >= 16 ? 2 : (QB == 2 ? 1 : 2)
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb) {
       float16v &sc = u.s[qb];
-      const float m_scaled = (m_run[qb] == -INFINITY ? 0.f : m_run[qb]) * c;
+      const float m_scaled = ms_run[qb];
       float rs = 0.f;
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
