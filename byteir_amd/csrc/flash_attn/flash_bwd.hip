@@ -2,7 +2,7 @@
 //   1. dot_do_o_kernel : D[b,h,i] = sum_d dO[i,d] * O[i,d]                      (fp32)
 //   2. dkdv_kernel     : one workgroup per 128 or 256 keys, loops over query tiles;
 //                        dV = P^T dO, dK = scale * dS^T Q accumulate in registers
-//   3. dq_kernel       : one workgroup per 128 or 256 queries, loops over key tiles;
+//   3. dq_kernel       : one workgroup per 128 queries, loops over key tiles;
 //                        dQ = scale * dS K accumulates in registers
 // P = exp2(scale*log2e * S - log2e * LSE) is recomputed from the forward's LSE in both main
 // kernels; dS = P * (dO V^T - D).  P and dS are rounded to the storage type before they
@@ -313,20 +313,27 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) dkdv_kernel(const Params
 }
 
 // ---- 3. dQ ----------------------------------------------------------------------------------
-// QB: 32-query blocks per wave.  Every K / V fragment fetched from LDS is used for all QB
-// blocks.  The workgroup covers 128*QB queries.
-template <typename T, int D, int QB>
+// One workgroup (4 waves x 32 query rows) per 128 queries; Q and dO fragments, LSE and D of a
+// wave's rows stay in registers.  K and V go through a three-deep LDS ring in 64-row tiles with
+// one barrier per tile, and are consumed in units of 32 keys.  Per unit: A: S^T = K Q^T and
+// dP^T = V dO^T (MFMA); B: dS^T = P^T o (dP^T - D) in place of S^T, rounded and packed (vector
+// ALU); C: dQ^T += K^T dS^T (MFMA, K^T through the transposing LDS read).  The loop is
+// software pipelined like the forward kernel: one step holds A of the next unit together
+// with B and C of the current one in a single basic block, so that matrix instructions run
+// under the exponentials.  Window edges are applied beforehand, by setting the masked scores
+// of an edge unit to -inf in a block of their own, which keeps B free of branches.
+template <typename T, int D>
 __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) dq_kernel(const Params p) {
   using vec8 = typename Traits<T>::vec8;
   constexpr int KS = D + 16;          // K tile: plain and transposed reads
   constexpr int VS = Pad<D>::kPlain;  // V tile: plain reads only
-  constexpr int kQueries = kQBlock * QB;
-  __shared__ __attribute__((aligned(16))) T Ks[2][kKvTile * KS];
-  __shared__ __attribute__((aligned(16))) T Vs[2][kKvTile * VS];
+  constexpr int kRing = 3;
+  __shared__ __attribute__((aligned(16))) T Ks[kRing][kKvTile * KS];
+  __shared__ __attribute__((aligned(16))) T Vs[kRing][kKvTile * VS];
 
   const int tid = threadIdx.x, lane = tid & 63;
-  // the wave index in a scalar register: everything derived from it (row windows, skip and
-  // mask decisions) then stays scalar and branches on it are real branches
+  // the wave index in a scalar register: the skip and edge decisions derived from it are
+  // scalar and every combination is its own straight-line instance of the step
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r32 = lane & 31, g = lane >> 5;
   int m_block, bh;
@@ -343,172 +350,164 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) dq_kernel(const Params p
     m_block = p.n_mblocks - 1 - m_block;
   }
   const int bi = bh / p.h, hi = bh % p.h;
-  const int m0 = m_block * kQueries;
-  const int wq0 = m0 + wave * 32 * QB;
+  const int m0 = m_block * kQBlock;
+  const int wq0 = m0 + wave * 32;
+  const int qrow = wq0 + r32;
 
-  int qrow[QB], lo_lim[QB], hi_lim[QB], h_lo_first[QB], h_hi_first[QB], h_lo_last[QB], h_hi_last[QB];
-#pragma unroll
-  for (int qb = 0; qb < QB; ++qb) {
-    qrow[qb] = wq0 + qb * 32 + r32;
-    row_limits(p, qrow[qb], lo_lim[qb], hi_lim[qb]);
-    row_limits(p, wq0 + qb * 32, h_lo_first[qb], h_hi_first[qb]);
-    row_limits(p, wq0 + qb * 32 + 31, h_lo_last[qb], h_hi_last[qb]);
-  }
-  const int w_lo_first = h_lo_first[0], w_hi_last = h_hi_last[QB - 1];
+  int lo_lim, hi_lim, w_lo_first, w_hi_first, w_lo_last, w_hi_last;
+  row_limits(p, qrow, lo_lim, hi_lim);
+  row_limits(p, wq0, w_lo_first, w_hi_first);
+  row_limits(p, wq0 + 31, w_lo_last, w_hi_last);
   int b_lo, b_hi, t0, t1;
   row_limits(p, m0, b_lo, t0);
-  row_limits(p, m0 + kQueries - 1, t1, b_hi);
+  row_limits(p, m0 + kQBlock - 1, t1, b_hi);
   const int n_min = b_lo / kKvTile;
   const int n_max = b_hi > 0 ? (b_hi + kKvTile - 1) / kKvTile : 0;
 
   const T *kg = static_cast<const T *>(p.k) + bi * p.k_bs + hi * p.k_hs;
   const T *vg = static_cast<const T *>(p.v) + bi * p.v_bs + hi * p.v_hs;
 
-  vec8 qf[QB][D / 16], dof[QB][D / 16];
-  float lse_l[QB], dsm_l[QB];
+  vec8 qf[D / 16], dof[D / 16];
+  float lse_l = INFINITY, dsm_l = 0.f;  // +inf: a row beyond seqlen_q contributes P = 0
+  if (qrow < p.sq) {
+    const T *qg = static_cast<const T *>(p.q) + bi * p.q_bs + (int64_t)qrow * p.q_rs + hi * p.q_hs;
+    const T *dog = static_cast<const T *>(p.dout) + bi * p.o_bs + (int64_t)qrow * p.o_rs + hi * p.o_hs;
 #pragma unroll
-  for (int qb = 0; qb < QB; ++qb) {
-    lse_l[qb] = INFINITY;
-    dsm_l[qb] = 0.f;
-    if (qrow[qb] < p.sq) {
-      const T *qg = static_cast<const T *>(p.q) + bi * p.q_bs + (int64_t)qrow[qb] * p.q_rs + hi * p.q_hs;
-      const T *dog = static_cast<const T *>(p.dout) + bi * p.o_bs + (int64_t)qrow[qb] * p.o_rs + hi * p.o_hs;
-#pragma unroll
-      for (int ks = 0; ks < D / 16; ++ks) {
-        qf[qb][ks] = *reinterpret_cast<const vec8 *>(qg + ks * 16 + g * 8);
-        dof[qb][ks] = *reinterpret_cast<const vec8 *>(dog + ks * 16 + g * 8);
-      }
-      lse_l[qb] = p.lse[((int64_t)bi * p.h + hi) * p.sq + qrow[qb]] * kLog2e;
-      dsm_l[qb] = p.dsoftmax[((int64_t)bi * p.h + hi) * p.sq_rounded + qrow[qb]];
-    } else {
-#pragma unroll
-      for (int ks = 0; ks < D / 16; ++ks) { qf[qb][ks] = vec8{0}; dof[qb][ks] = vec8{0}; }
+    for (int ks = 0; ks < D / 16; ++ks) {
+      qf[ks] = *reinterpret_cast<const vec8 *>(qg + ks * 16 + g * 8);
+      dof[ks] = *reinterpret_cast<const vec8 *>(dog + ks * 16 + g * 8);
     }
+    lse_l = p.lse[((int64_t)bi * p.h + hi) * p.sq + qrow] * kLog2e;
+    dsm_l = p.dsoftmax[((int64_t)bi * p.h + hi) * p.sq_rounded + qrow];
+  } else {
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ++ks) { qf[ks] = vec8{0}; dof[ks] = vec8{0}; }
   }
   // consume the fragments once so that the wait for their loads sits here, not inside the loop
 #pragma unroll
-  for (int qb = 0; qb < QB; ++qb) {
+  for (int ks = 0; ks < D / 16; ++ks) asm volatile("" : "+v"(qf[ks]), "+v"(dof[ks]));
+  asm volatile("" : "+v"(lse_l), "+v"(dsm_l));
+  float16v dq_acc[D / 32];
 #pragma unroll
-    for (int ks = 0; ks < D / 16; ++ks) asm volatile("" : "+v"(qf[qb][ks]), "+v"(dof[qb][ks]));
-    asm volatile("" : "+v"(lse_l[qb]), "+v"(dsm_l[qb]));
-  }
-  float16v dq_acc[QB][D / 32];
-#pragma unroll
-  for (int qb = 0; qb < QB; ++qb)
-#pragma unroll
-    for (int i = 0; i < D / 32; ++i) dq_acc[qb][i] = float16v{0};
+  for (int i = 0; i < D / 32; ++i) dq_acc[i] = float16v{0};
   const float c = p.scale_log2;
 
-  // double-buffered tiles, one barrier per tile (see dkdv_kernel)
   TileLoader<T, D, kKvTile> lk, lv;  // tiles are fetched in order, n_min first
   lk.start(kg, p.k_rs, n_min * kKvTile, p.sk);
   lv.start(vg, p.v_rs, n_min * kKvTile, p.sk);
-  if (n_min < n_max) {
-    lk.gload();
-    lv.gload();
-    lk.lstore(Ks[0], KS);
-    lv.lstore(Vs[0], VS);
-    if (n_min + 1 < n_max) {
-      lk.gload();
-      lv.gload();
+  auto gload = [&]() { lk.gload(); lv.gload(); };
+  auto lstore = [&](int buf) { lk.lstore(Ks[buf], KS); lv.lstore(Vs[buf], VS); };
+
+  struct Unit { float16v s, dp; };
+  const int frag_k = r32 * KS + g * 8, frag_v = r32 * VS + g * 8;
+
+  // what the wave's 32 rows see of the 32 keys from kv0: 0 nothing, 1 all, 2 an edge crosses
+  auto visibility = [&](int kv0) {
+    if (kv0 >= w_hi_last || kv0 + 32 <= w_lo_first) return 0;
+    return (kv0 + 32 > w_hi_first || kv0 < w_lo_last) ? 2 : 1;
+  };
+  // A: S^T = K Q^T, dP^T = V dO^T for 32-key unit `kvb` of a tile
+  auto part_a = [&](const T *Kt, const T *Vt, int kvb, Unit &u) {
+    u.s = float16v{0};
+    u.dp = float16v{0};
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ++ks) {
+      const vec8 ak = lds_read8<T>(&Kt[kvb * 32 * KS + frag_k + ks * 16]);
+      const vec8 av = lds_read8<T>(&Vt[kvb * 32 * VS + frag_v + ks * 16]);
+      u.s = Traits<T>::mfma(ak, qf[ks], u.s);
+      u.dp = Traits<T>::mfma(av, dof[ks], u.dp);
     }
+  };
+  // the scores of an edge unit that fall outside the row's window become -inf (P = 0)
+  auto mask = [&](Unit &u, int kv0) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int kv = kv0 + (i >> 2) * 8 + g * 4 + (i & 3);
+      if (kv >= hi_lim || kv < lo_lim) u.s[i] = -INFINITY;
+    }
+  };
+  // B: dS^T in place of S^T, packed as B operands [16-key window]
+  auto part_b = [&](Unit &u, vec8 (&dsb)[2]) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const float pe = exp2_fast(fmaf(u.s[i], c, -lse_l));
+      u.s[i] = pe * (u.dp[i] - dsm_l);
+    }
+#pragma unroll
+    for (int w = 0; w < 2; ++w) {
+      float f[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) f[j] = u.s[w * 8 + j];
+      dsb[w] = pack8<T>(f);
+    }
+  };
+  // C: dQ^T += K^T dS^T
+  auto part_c = [&](const T *Kt, int kvb, const vec8 (&dsb)[2]) {
+#pragma unroll
+    for (int w = 0; w < 2; ++w)
+#pragma unroll
+      for (int db = 0; db < D / 32; ++db) {
+        const vec8 a = lds_read_operand_tr<T>(Kt, KS, kvb * 32 + w * 16, db * 32);
+        dq_acc[db] = Traits<T>::mfma(a, dsb[w], dq_acc[db]);
+      }
+  };
+  // One pipeline step: finish unit `cur` (B, C) and, in the same basic block, start `nxt` (A).
+  // The step has a single instance: a unit that a wave does not see at all is masked like an
+  // edge unit (P = 0, it adds nothing) instead of being skipped, and the look-ahead past the
+  // last tile reads a stale ring slot whose result is never used.  Variants of the step would
+  // each accumulate into dQ, and the register allocator then reconciles their assignments
+  // with 16 moves (and a drain of the matrix pipe) at the end of every step.
+  auto step = [&](int vis, Unit &cur, int kv0, int buf, int kvb, Unit &nxt, int nbuf, int nkvb) {
+    if (vis != 1) mask(cur, kv0);
+    vec8 dsb[2];
+    part_a(Ks[nbuf], Vs[nbuf], nkvb, nxt);
+    part_b(cur, dsb);
+    part_c(Ks[buf], kvb, dsb);
+  };
+
+  // prologue: tiles n_min and n_min+1 into the ring, tile n_min+2 into registers
+  const int n_tiles = n_max > n_min ? n_max - n_min : 0;
+  Unit ua, ub;
+  if (n_tiles > 0) {
+    gload();
+    lstore(0);
+    if (n_tiles > 1) { gload(); lstore(1); }
+    if (n_tiles > 2) gload();
     __syncthreads();
+    part_a(Ks[0], Vs[0], 0, ua);
   }
+  int buf = 0;  // ring slot of tile t
   for (int t = n_min; t < n_max; ++t) {
-    const int buf = (t - n_min) & 1;
+    const int buf1 = buf + 1 == kRing ? 0 : buf + 1;
+    const int buf2 = buf1 + 1 == kRing ? 0 : buf1 + 1;
     const int kv0 = t * kKvTile;
-    if (t + 1 < n_max) { lk.lstore(Ks[buf ^ 1], KS); lv.lstore(Vs[buf ^ 1], VS); }
-    if (t + 2 < n_max) {
-      lk.gload();
-      lv.gload();
-    }
-    const T *Kt = Ks[buf];
-    const T *Vt = Vs[buf];
-    const bool skip = kv0 >= w_hi_last || kv0 + kKvTile <= w_lo_first;
-    if (!skip) {
-      float16v s[QB][2], dp[QB][2];
-#pragma unroll
-      for (int kvb = 0; kvb < 2; ++kvb) {
-#pragma unroll
-        for (int qb = 0; qb < QB; ++qb) { s[qb][kvb] = float16v{0}; dp[qb][kvb] = float16v{0}; }
-#pragma unroll
-        for (int ks = 0; ks < D / 16; ++ks) {
-          const vec8 ak = lds_read8<T>(&Kt[(kvb * 32 + r32) * KS + ks * 16 + g * 8]);
-          const vec8 av = lds_read8<T>(&Vt[(kvb * 32 + r32) * VS + ks * 16 + g * 8]);
-#pragma unroll
-          for (int qb = 0; qb < QB; ++qb) {
-            s[qb][kvb] = Traits<T>::mfma(ak, qf[qb][ks], s[qb][kvb]);
-            dp[qb][kvb] = Traits<T>::mfma(av, dof[qb][ks], dp[qb][kvb]);
-          }
-        }
-      }
-      vec8 dsb[QB][4];  // dS^T as B operands: [query block][16-key window]
-      // dS^T = P^T o (dP^T - D) in place of S^T; kMask: the window edge crosses this tile
-      auto ds_tile = [&](auto mask_tag, int qb) {
-        constexpr bool kMask = decltype(mask_tag)::value;
-#pragma unroll
-        for (int kvb = 0; kvb < 2; ++kvb)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) {
-            float pe = exp2_fast(fmaf(s[qb][kvb][i], c, -lse_l[qb]));
-            if constexpr (kMask) {
-              const int kv = kv0 + kvb * 32 + (i >> 2) * 8 + g * 4 + (i & 3);
-              if (kv >= hi_lim[qb] || kv < lo_lim[qb]) pe = 0.f;
-            }
-            s[qb][kvb][i] = pe * (dp[qb][kvb][i] - dsm_l[qb]);
-          }
-      };
-#pragma unroll
-      for (int qb = 0; qb < QB; ++qb) {
-        if (kv0 + kKvTile > h_hi_first[qb] || kv0 < h_lo_last[qb]) ds_tile(std::true_type{}, qb);
-        else ds_tile(std::false_type{}, qb);
-#pragma unroll
-        for (int w = 0; w < 4; ++w) {
-          float f[8];
-#pragma unroll
-          for (int j = 0; j < 8; ++j) f[j] = s[qb][w >> 1][(w & 1) * 8 + j];
-          dsb[qb][w] = pack8<T>(f);
-        }
-      }
-#pragma unroll
-      for (int w = 0; w < 4; ++w)
-#pragma unroll
-        for (int db = 0; db < D / 32; ++db) {
-          const vec8 a = lds_read_operand_tr<T>(Kt, KS, w * 16, db * 32);
-#pragma unroll
-          for (int qb = 0; qb < QB; ++qb) dq_acc[qb][db] = Traits<T>::mfma(a, dsb[qb][w], dq_acc[qb][db]);
-        }
-    }
-    __syncthreads();  // tile t is consumed, tile t+1 is visible
+    // unit 0 of tile t (in ua) while unit 1 is produced into ub
+    step(visibility(kv0), ua, kv0, buf, 0, ub, buf, 1);
+    __syncthreads();  // tile t+1 is visible; every wave has left tile t-1
+    // tile t+2: registers -> the ring slot tile t-1 occupied; tile t+3 in flight
+    if (t + 2 < n_max) lstore(buf2);
+    if (t + 3 < n_max) gload();
+    // unit 1 of tile t (in ub) while unit 0 of tile t+1 is produced into ua
+    step(visibility(kv0 + 32), ub, kv0 + 32, buf, 1, ua, buf1, 0);
+    buf = buf1;
   }
 
+  if (qrow < p.sq) {
+    T *dqg = static_cast<T *>(p.dq) + bi * p.q_bs + (int64_t)qrow * p.q_rs + hi * p.q_hs;
+    typedef T vec4 __attribute__((ext_vector_type(4)));
 #pragma unroll
-  for (int qb = 0; qb < QB; ++qb) {
-    if (qrow[qb] < p.sq) {
-      T *dqg = static_cast<T *>(p.dq) + bi * p.q_bs + (int64_t)qrow[qb] * p.q_rs + hi * p.q_hs;
-      typedef T vec4 __attribute__((ext_vector_type(4)));
+    for (int db = 0; db < D / 32; ++db)
 #pragma unroll
-      for (int db = 0; db < D / 32; ++db)
+      for (int i4 = 0; i4 < 4; ++i4) {
+        vec4 a;
 #pragma unroll
-        for (int i4 = 0; i4 < 4; ++i4) {
-          vec4 a;
-#pragma unroll
-          for (int j = 0; j < 4; ++j) a[j] = (T)(dq_acc[qb][db][i4 * 4 + j] * p.scale);
-          *reinterpret_cast<vec4 *>(dqg + db * 32 + i4 * 8 + g * 4) = a;
-        }
-    }
+        for (int j = 0; j < 4; ++j) a[j] = (T)(dq_acc[db][i4 * 4 + j] * p.scale);
+        *reinterpret_cast<vec4 *>(dqg + db * 32 + i4 * 8 + g * 4) = a;
+      }
   }
 }
 
-// 32-key blocks per wave in dkdv.  Two blocks halve the LDS reads per MFMA but need more than
-// 256 registers, i.e. one wave per SIMD and MFMA accumulators in AccVGPRs, whose results then
-// reach the vector ALU through one v_accvgpr_read per value; one block with two waves per SIMD
-// measured 17 % faster (1.47 ms against 1.77 ms on the bf16 head_dim-64 benchmark).
 template <int D> struct DkdvGeom { static constexpr int KB = 1; };
-// 32-query blocks per wave in dq: two blocks cost the second wave per SIMD and measured
-// slower (1.76 ms vs 1.28 ms on the bf16 head_dim-64 benchmark), so one
-template <int D> struct DqGeom { static constexpr int QB = 1; };
-
 template <typename T, int D>
 hipError_t launch_bwd_td(const Params &p, hipStream_t stream) {
   const int64_t rows = (int64_t)p.b * p.h * p.sq;
@@ -521,11 +520,10 @@ hipError_t launch_bwd_td(const Params &p, hipStream_t stream) {
   pk.n_nblocks = (p.sk + kKvBlock * KB - 1) / (kKvBlock * KB);
   if (pk.n_nblocks > 0)
     dkdv_kernel<T, D, KB><<<dim3((unsigned)(pk.n_nblocks * p.b * p.h)), dim3(256), 0, stream>>>(pk);
-  constexpr int QB = DqGeom<D>::QB;
   Params pq = p;
-  pq.n_mblocks = (p.sq + kQBlock * QB - 1) / (kQBlock * QB);
+  pq.n_mblocks = (p.sq + kQBlock - 1) / kQBlock;
   if (pq.n_mblocks > 0)
-    dq_kernel<T, D, QB><<<dim3((unsigned)(pq.n_mblocks * p.b * p.h)), dim3(256), 0, stream>>>(pq);
+    dq_kernel<T, D><<<dim3((unsigned)(pq.n_mblocks * p.b * p.h)), dim3(256), 0, stream>>>(pq);
   return hipGetLastError();
 }
 
