@@ -1,6 +1,6 @@
 // Flash-attention backward for gfx950.  Three launches, no atomics, deterministic:
 //   1. dot_do_o_kernel : D[b,h,i] = sum_d dO[i,d] * O[i,d]                      (fp32)
-//   2. dkdv_kernel     : one workgroup per 128 or 256 keys, loops over query tiles;
+//   2. dkdv_kernel     : one workgroup per 128 keys, loops over query tiles;
 //                        dV = P^T dO, dK = scale * dS^T Q accumulate in registers
 //   3. dq_kernel       : one workgroup per 128 queries, loops over key tiles;
 //                        dQ = scale * dS K accumulates in registers
@@ -91,22 +91,32 @@ struct TileLoader {
 };
 
 // ---- 2. dK, dV ------------------------------------------------------------------------------
-// KB: 32-key blocks per wave.  Every Q / dO fragment fetched from LDS (plain or transposed)
-// is used for all KB blocks, so LDS traffic per MFMA falls as 1/KB; LDS read bandwidth is what
-// bounds this kernel.  The workgroup covers 128*KB keys.
-template <typename T, int D, int KB>
+// One workgroup (4 waves) per 128 keys; a wave keeps the K and V fragments of its 32 keys in
+// registers and walks the query axis in units of 32 rows, two units per 64-row LDS tile of Q,
+// dO, LSE and D.  The tiles go through a three-deep LDS ring with one barrier per tile.
+//
+// Per unit a wave does A: S = Q K^T, dP = dO V^T (MFMA); B: P = exp2(..), dS = P (dP - D),
+// rounded to the storage type and packed (vector ALU); C: dV^T += dO^T P, dK^T += Q^T dS
+// (MFMA).  The loop is software pipelined with C one unit behind: a step holds A and B of the
+// current unit and C of the previous one, whose MFMAs do not depend on the vector work of B
+// and run under it (delaying C costs 16 registers for a second set of packed P / dS;
+// producing S and dP one unit ahead would cost 32 and does not fit two waves per SIMD).
+// The step has a single instance: window edges are applied as -inf scores between A and B, a
+// unit that the wave's keys do not see at all is treated like an edge unit (it adds zeros),
+// and the first step accumulates a zero P / dS.
+template <typename T, int D>
 __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) dkdv_kernel(const Params p) {
   using vec8 = typename Traits<T>::vec8;
   constexpr int QS = D + 16;  // tiles are read both plainly and transposed
-  constexpr int kKeys = kKvBlock * KB;
-  __shared__ __attribute__((aligned(16))) T Qs[2][kQTile * QS];
-  __shared__ __attribute__((aligned(16))) T dOs[2][kQTile * QS];
-  __shared__ float lse_s[2][kQTile];
-  __shared__ float dsm_s[2][kQTile];
+  constexpr int kRing = 3;
+  __shared__ __attribute__((aligned(16))) T Qs[kRing][kQTile * QS];
+  __shared__ __attribute__((aligned(16))) T dOs[kRing][kQTile * QS];
+  __shared__ __attribute__((aligned(16))) float lse_s[kRing][kQTile];
+  __shared__ __attribute__((aligned(16))) float dsm_s[kRing][kQTile];
 
   const int tid = threadIdx.x, lane = tid & 63;
-  // the wave index in a scalar register: everything derived from it (row windows, skip and
-  // mask decisions) then stays scalar and branches on it are real branches
+  // the wave index in a scalar register: everything derived from it (row windows, edge
+  // decisions) then stays scalar and branches on it are real branches
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r32 = lane & 31, g = lane >> 5;
   int n_block, bh;
@@ -122,8 +132,8 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) dkdv_kernel(const Params
     }
   }
   const int bi = bh / p.h, hi = bh % p.h;
-  const int kvb0 = n_block * kKeys;
-  const int wkv0 = kvb0 + wave * 32 * KB;  // first key of the wave
+  const int kvb0 = n_block * kKvBlock;
+  const int wkv0 = kvb0 + wave * 32;  // first key of the wave
   const int off = p.sk - p.sq;
 
   const T *qg = static_cast<const T *>(p.q) + bi * p.q_bs + hi * p.q_hs;
@@ -131,39 +141,33 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) dkdv_kernel(const Params
   const float *lse_g = p.lse + ((int64_t)bi * p.h + hi) * p.sq;
   const float *dsm_g = p.dsoftmax + ((int64_t)bi * p.h + hi) * p.sq_rounded;
 
-  int kvcol[KB];  // the keys this lane owns
-  vec8 kf[KB][D / 16], vf[KB][D / 16];
-#pragma unroll
-  for (int kb = 0; kb < KB; ++kb) {
-    kvcol[kb] = wkv0 + kb * 32 + r32;
-    const T *kg = static_cast<const T *>(p.k) + bi * p.k_bs + (int64_t)kvcol[kb] * p.k_rs + hi * p.k_hs;
-    const T *vg = static_cast<const T *>(p.v) + bi * p.v_bs + (int64_t)kvcol[kb] * p.v_rs + hi * p.v_hs;
+  const int kvcol = wkv0 + r32;  // the key this lane owns
+  vec8 kf[D / 16], vf[D / 16];
+  {
+    const T *kg = static_cast<const T *>(p.k) + bi * p.k_bs + (int64_t)kvcol * p.k_rs + hi * p.k_hs;
+    const T *vg = static_cast<const T *>(p.v) + bi * p.v_bs + (int64_t)kvcol * p.v_rs + hi * p.v_hs;
 #pragma unroll
     for (int ks = 0; ks < D / 16; ++ks) {
-      if (kvcol[kb] < p.sk) {
-        kf[kb][ks] = *reinterpret_cast<const vec8 *>(kg + ks * 16 + g * 8);
-        vf[kb][ks] = *reinterpret_cast<const vec8 *>(vg + ks * 16 + g * 8);
+      if (kvcol < p.sk) {
+        kf[ks] = *reinterpret_cast<const vec8 *>(kg + ks * 16 + g * 8);
+        vf[ks] = *reinterpret_cast<const vec8 *>(vg + ks * 16 + g * 8);
       } else {
-        kf[kb][ks] = vec8{0};
-        vf[kb][ks] = vec8{0};
+        kf[ks] = vec8{0};
+        vf[ks] = vec8{0};
       }
     }
   }
   // consume the fragments once so that the wait for their loads sits here, not inside the loop
 #pragma unroll
-  for (int kb = 0; kb < KB; ++kb)
+  for (int ks = 0; ks < D / 16; ++ks) asm volatile("" : "+v"(kf[ks]), "+v"(vf[ks]));
+  float16v dk_acc[D / 32], dv_acc[D / 32];
 #pragma unroll
-    for (int ks = 0; ks < D / 16; ++ks) asm volatile("" : "+v"(kf[kb][ks]), "+v"(vf[kb][ks]));
-  float16v dk_acc[KB][D / 32], dv_acc[KB][D / 32];
-#pragma unroll
-  for (int kb = 0; kb < KB; ++kb)
-#pragma unroll
-    for (int i = 0; i < D / 32; ++i) { dk_acc[kb][i] = float16v{0}; dv_acc[kb][i] = float16v{0}; }
+  for (int i = 0; i < D / 32; ++i) { dk_acc[i] = float16v{0}; dv_acc[i] = float16v{0}; }
 
-  // query tiles that can see keys [kvb0, kvb0 + kKeys)
+  // query tiles that can see keys [kvb0, kvb0 + 128)
   int q_lo = 0, q_hi = p.sq;
-  if (p.wr >= 0) q_lo = max(0, kvb0 - off - p.wr);              // hi(q) = q+1+off+wr > kvb0
-  if (p.wl >= 0) q_hi = min(p.sq, kvb0 + kKeys - off + p.wl);   // lo(q) = q+off-wl < kvb0+kKeys
+  if (p.wr >= 0) q_lo = max(0, kvb0 - off - p.wr);                 // hi(q) = q+1+off+wr > kvb0
+  if (p.wl >= 0) q_hi = min(p.sq, kvb0 + kKvBlock - off + p.wl);   // lo(q) = q+off-wl < kvb0+128
   const int m_min = q_lo / kQTile;
   const int m_max = q_hi > 0 ? (q_hi + kQTile - 1) / kQTile : 0;
   const float c = p.scale_log2;
@@ -172,18 +176,19 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) dkdv_kernel(const Params
   const int win_lo = p.wl >= 0 ? -p.wl : -(1 << 30);
   const unsigned win_span = (unsigned)((p.wr >= 0 ? p.wr : (1 << 30)) - win_lo);
 
-  TileLoader<T, D, kQTile> lq, ldo;
+  TileLoader<T, D, kQTile> lq, ldo;  // tiles are fetched in order, m_min first
   lq.start(qg, p.q_rs, m_min * kQTile, p.sq);
   ldo.start(dog, p.o_rs, m_min * kQTile, p.sq);
   float lse_r = 0.f, dsm_r = 0.f;
-  auto gload = [&](int m) {  // tiles are fetched in order, m_min first
+  int q_next = m_min * kQTile + tid;  // the row whose LSE and D this thread stages next
+  auto gload = [&]() {
     lq.gload();
     ldo.gload();
     if (tid < kQTile) {
-      const int q = m * kQTile + tid;
-      lse_r = q < p.sq ? lse_g[q] : INFINITY;  // +inf: the row contributes P = 0
-      dsm_r = q < p.sq ? dsm_g[q] : 0.f;
+      lse_r = q_next < p.sq ? lse_g[q_next] : INFINITY;  // +inf: the row contributes P = 0
+      dsm_r = q_next < p.sq ? dsm_g[q_next] : 0.f;
     }
+    q_next += kQTile;
   };
   auto lstore = [&](int buf) {
     lq.lstore(Qs[buf], QS);
@@ -191,124 +196,130 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) dkdv_kernel(const Params
     if (tid < kQTile) { lse_s[buf][tid] = lse_r * kLog2e; dsm_s[buf][tid] = dsm_r; }
   };
 
-  // double-buffered tiles, one barrier per tile: tile m is read from buffer b while tile m+1
-  // is written to the other one (free since the barrier that closed tile m-1) and tile m+2 is
-  // in flight from global memory
-  if (m_min < m_max) {
-    gload(m_min);
+  struct Unit { float16v s, dp; };
+  const int frag_rd = r32 * QS + g * 8;  // this lane's plain fragment inside a 32-row unit
+
+  // A: S = Q K^T, dP = dO V^T for the 32 query rows of unit `qs` of a tile
+  auto part_a = [&](const T *Qt, const T *dOt, int qs, Unit &u) {
+    u.s = float16v{0};
+    u.dp = float16v{0};
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ++ks) {
+      const vec8 aq = lds_read8<T>(&Qt[qs * 32 * QS + frag_rd + ks * 16]);
+      const vec8 ad = lds_read8<T>(&dOt[qs * 32 * QS + frag_rd + ks * 16]);
+      u.s = Traits<T>::mfma(aq, kf[ks], u.s);
+      u.dp = Traits<T>::mfma(ad, vf[ks], u.dp);
+    }
+  };
+  // scores outside the window become -inf (P = 0): key - (query + sk - sq) must lie in
+  // [-wl, wr], one unsigned compare per element
+  auto mask = [&](Unit &u, int q0) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const unsigned rel = (unsigned)(kvcol - off - q0 - g * 4 - ((i >> 2) * 8 + (i & 3)) - win_lo);
+      if (rel > win_span) u.s[i] = -INFINITY;
+    }
+  };
+  // B: P and dS of the unit, rounded and packed as B operands [16-query window]
+  auto part_b = [&](Unit &u, int buf, int qs, vec8 (&pb)[2], vec8 (&dsb)[2]) {
+    float pv[16], dsv[16];
+#pragma unroll
+    for (int i4 = 0; i4 < 4; ++i4) {
+      const int ql = qs * 32 + i4 * 8 + g * 4;  // 4 consecutive rows of the LDS tile
+      const float4 l4 = *reinterpret_cast<const float4 *>(&lse_s[buf][ql]);
+      const float4 d4 = *reinterpret_cast<const float4 *>(&dsm_s[buf][ql]);
+      const float lq4[4] = {l4.x, l4.y, l4.z, l4.w}, dq4[4] = {d4.x, d4.y, d4.z, d4.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int i = i4 * 4 + j;
+        const float pe = exp2_fast(fmaf(u.s[i], c, -lq4[j]));
+        pv[i] = pe;
+        dsv[i] = pe * (u.dp[i] - dq4[j]);
+      }
+    }
+#pragma unroll
+    for (int w = 0; w < 2; ++w) {
+      pb[w] = pack8<T>(&pv[w * 8]);
+      dsb[w] = pack8<T>(&dsv[w * 8]);
+    }
+  };
+  // C: dV^T += dO^T P, dK^T += Q^T dS
+  auto part_c = [&](const T *Qt, const T *dOt, int qs, const vec8 (&pb)[2], const vec8 (&dsb)[2]) {
+#pragma unroll
+    for (int w = 0; w < 2; ++w)
+#pragma unroll
+      for (int db = 0; db < D / 32; ++db) {
+        const vec8 a_do = lds_read_operand_tr<T>(dOt, QS, qs * 32 + w * 16, db * 32);
+        const vec8 a_q = lds_read_operand_tr<T>(Qt, QS, qs * 32 + w * 16, db * 32);
+        dv_acc[db] = Traits<T>::mfma(a_do, pb[w], dv_acc[db]);
+        dk_acc[db] = Traits<T>::mfma(a_q, dsb[w], dk_acc[db]);
+      }
+  };
+  // does the window keep every (query, key) pair of the 32 rows from q0 and the wave's keys?
+  auto all_kept = [&](int q0) {
+    int lo_first, hi_first, lo_last, hi_last;
+    row_limits(p, q0, lo_first, hi_first);
+    row_limits(p, q0 + 31, lo_last, hi_last);
+    return wkv0 + 32 <= hi_first && wkv0 >= lo_last;
+  };
+  vec8 pb[2], dsb[2];  // packed P and dS of the previous unit, still to be accumulated
+#pragma unroll
+  for (int w = 0; w < 2; ++w) { pb[w] = vec8{0}; dsb[w] = vec8{0}; }
+  auto step = [&](int buf, int qs, int q0, int pbuf, int pqs) {
+    Unit u;
+    part_a(Qs[buf], dOs[buf], qs, u);
+    if (!all_kept(q0)) mask(u, q0);
+    vec8 pb_new[2], dsb_new[2];
+    part_c(Qs[pbuf], dOs[pbuf], pqs, pb, dsb);
+    part_b(u, buf, qs, pb_new, dsb_new);
+#pragma unroll
+    for (int w = 0; w < 2; ++w) { pb[w] = pb_new[w]; dsb[w] = dsb_new[w]; }
+  };
+
+  // prologue: tiles m_min and m_min+1 into the ring, tile m_min+2 into registers
+  const int n_tiles = m_max > m_min ? m_max - m_min : 0;
+  if (n_tiles > 0) {
+    gload();
     lstore(0);
-    if (m_min + 1 < m_max) gload(m_min + 1);
+    if (n_tiles > 1) { gload(); lstore(1); }
+    if (n_tiles > 2) gload();
     __syncthreads();
   }
+  int buf = 0, pbuf = 0;  // ring slots of tile m and of the tile of the pending unit
   for (int m = m_min; m < m_max; ++m) {
-    const int buf = (m - m_min) & 1;
-    if (m + 1 < m_max) lstore(buf ^ 1);
-    if (m + 2 < m_max) gload(m + 2);
-    const T *Qt = Qs[buf];
-    const T *dOt = dOs[buf];
-    // S = Q K^T and dP = dO V^T of one 32-query sub-tile (the zero accumulators stay next to
-    // their first MFMA, which then takes the constant 0 as its C operand)
-    auto scores = [&](int qs, float16v (&s)[KB], float16v (&dp)[KB]) {
-#pragma unroll
-      for (int kb = 0; kb < KB; ++kb) { s[kb] = float16v{0}; dp[kb] = float16v{0}; }
-#pragma unroll
-      for (int ks = 0; ks < D / 16; ++ks) {
-        const vec8 aq = lds_read8<T>(&Qt[(qs * 32 + r32) * QS + ks * 16 + g * 8]);
-        const vec8 ad = lds_read8<T>(&dOt[(qs * 32 + r32) * QS + ks * 16 + g * 8]);
-#pragma unroll
-        for (int kb = 0; kb < KB; ++kb) {
-          s[kb] = Traits<T>::mfma(aq, kf[kb][ks], s[kb]);
-          dp[kb] = Traits<T>::mfma(ad, vf[kb][ks], dp[kb]);
-        }
-      }
-    };
-    // P and dS of the sub-tile as packed B operands [key block][16-query window]; kMask: the
-    // window edge crosses it.  Only this vector part exists twice: the accumulating MFMAs
-    // follow after the two variants have joined, so that dK / dV keep one set of registers.
-    auto softmax_grad = [&](auto mask_tag, int qs, int q0, float16v (&s)[KB], float16v (&dp)[KB],
-                            vec8 (&pb)[KB][2], vec8 (&dsb)[KB][2]) {
-      constexpr bool kMask = decltype(mask_tag)::value;
-      float lse_q[16], dsm_q[16];
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int ql = qs * 32 + (i >> 2) * 8 + g * 4 + (i & 3);  // row inside the LDS tile
-        lse_q[i] = lse_s[buf][ql];
-        dsm_q[i] = dsm_s[buf][ql];
-      }
-#pragma unroll
-      for (int kb = 0; kb < KB; ++kb) {
-        float pv[16], dsv[16];
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          float pe = exp2_fast(fmaf(s[kb][i], c, -lse_q[i]));
-          if constexpr (kMask) {
-            // key - (query + sk - sq) must lie in [-wl, wr]: one unsigned compare
-            const unsigned rel = (unsigned)(kvcol[kb] - off - q0 - g * 4 - ((i >> 2) * 8 + (i & 3)) - win_lo);
-            if (rel > win_span) pe = 0.f;
-          }
-          pv[i] = pe;
-          dsv[i] = pe * (dp[kb][i] - dsm_q[i]);
-        }
-#pragma unroll
-        for (int w = 0; w < 2; ++w) {
-          pb[kb][w] = pack8<T>(&pv[w * 8]);
-          dsb[kb][w] = pack8<T>(&dsv[w * 8]);
-        }
-      }
-    };
-    // dV^T += dO^T P, dK^T += Q^T dS
-    auto accumulate = [&](int qs, const vec8 (&pb)[KB][2], const vec8 (&dsb)[KB][2]) {
-#pragma unroll
-      for (int w = 0; w < 2; ++w)
-#pragma unroll
-        for (int db = 0; db < D / 32; ++db) {
-          const vec8 a_do = lds_read_operand_tr<T>(dOt, QS, qs * 32 + w * 16, db * 32);
-          const vec8 a_q = lds_read_operand_tr<T>(Qt, QS, qs * 32 + w * 16, db * 32);
-#pragma unroll
-          for (int kb = 0; kb < KB; ++kb) {
-            dv_acc[kb][db] = Traits<T>::mfma(a_do, pb[kb][w], dv_acc[kb][db]);
-            dk_acc[kb][db] = Traits<T>::mfma(a_q, dsb[kb][w], dk_acc[kb][db]);
-          }
-        }
-    };
-#pragma unroll
-    for (int qs = 0; qs < kQTile / 32; ++qs) {
-      const int q0 = m * kQTile + qs * 32;  // first query row of this 32-row sub-tile
-      // wave-uniform visibility of the sub-tile against the wave's keys
-      int lo_first, hi_first, lo_last, hi_last;
-      row_limits(p, q0, lo_first, hi_first);
-      row_limits(p, q0 + 31, lo_last, hi_last);
-      if (wkv0 >= hi_last || wkv0 + 32 * KB <= lo_first) continue;  // nothing kept
-      float16v s[KB], dp[KB];
-      scores(qs, s, dp);
-      vec8 pb[KB][2], dsb[KB][2];
-      if (wkv0 + 32 * KB > hi_first || wkv0 < lo_last) softmax_grad(std::true_type{}, qs, q0, s, dp, pb, dsb);
-      else softmax_grad(std::false_type{}, qs, q0, s, dp, pb, dsb);
-      accumulate(qs, pb, dsb);
-    }
-    __syncthreads();  // tile m is consumed, tile m+1 is visible
+    const int buf1 = buf + 1 == kRing ? 0 : buf + 1;
+    const int buf2 = buf1 + 1 == kRing ? 0 : buf1 + 1;
+    const int q0 = m * kQTile;
+    // unit 0 of tile m; C of unit 1 of tile m-1 (still in its ring slot) rides along
+    step(buf, 0, q0, pbuf, 1);
+    __syncthreads();  // tile m+1 is visible; every wave has left tile m-1
+    // tile m+2: registers -> the ring slot tile m-1 occupied; tile m+3 in flight
+    if (m + 2 < m_max) lstore(buf2);
+    if (m + 3 < m_max) gload();
+    // unit 1 of tile m; C of unit 0 rides along
+    step(buf, 1, q0 + 32, buf, 0);
+    pbuf = buf;
+    buf = buf1;
   }
+  if (n_tiles > 0) part_c(Qs[pbuf], dOs[pbuf], 1, pb, dsb);
 
+  if (kvcol < p.sk) {
+    T *dkg = static_cast<T *>(p.dk) + bi * p.k_bs + (int64_t)kvcol * p.k_rs + hi * p.k_hs;
+    T *dvg = static_cast<T *>(p.dv) + bi * p.v_bs + (int64_t)kvcol * p.v_rs + hi * p.v_hs;
+    typedef T vec4 __attribute__((ext_vector_type(4)));
 #pragma unroll
-  for (int kb = 0; kb < KB; ++kb) {
-    if (kvcol[kb] < p.sk) {
-      T *dkg = static_cast<T *>(p.dk) + bi * p.k_bs + (int64_t)kvcol[kb] * p.k_rs + hi * p.k_hs;
-      T *dvg = static_cast<T *>(p.dv) + bi * p.v_bs + (int64_t)kvcol[kb] * p.v_rs + hi * p.v_hs;
-      typedef T vec4 __attribute__((ext_vector_type(4)));
+    for (int db = 0; db < D / 32; ++db)
 #pragma unroll
-      for (int db = 0; db < D / 32; ++db)
+      for (int i4 = 0; i4 < 4; ++i4) {
+        vec4 a, b;
 #pragma unroll
-        for (int i4 = 0; i4 < 4; ++i4) {
-          vec4 a, b;
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            a[j] = (T)(dk_acc[kb][db][i4 * 4 + j] * p.scale);
-            b[j] = (T)(dv_acc[kb][db][i4 * 4 + j]);
-          }
-          *reinterpret_cast<vec4 *>(dkg + db * 32 + i4 * 8 + g * 4) = a;
-          *reinterpret_cast<vec4 *>(dvg + db * 32 + i4 * 8 + g * 4) = b;
+        for (int j = 0; j < 4; ++j) {
+          a[j] = (T)(dk_acc[db][i4 * 4 + j] * p.scale);
+          b[j] = (T)(dv_acc[db][i4 * 4 + j]);
         }
-    }
+        *reinterpret_cast<vec4 *>(dkg + db * 32 + i4 * 8 + g * 4) = a;
+        *reinterpret_cast<vec4 *>(dvg + db * 32 + i4 * 8 + g * 4) = b;
+      }
   }
 }
 
@@ -507,7 +518,6 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) dq_kernel(const Params p
   }
 }
 
-template <int D> struct DkdvGeom { static constexpr int KB = 1; };
 template <typename T, int D>
 hipError_t launch_bwd_td(const Params &p, hipStream_t stream) {
   const int64_t rows = (int64_t)p.b * p.h * p.sq;
@@ -515,11 +525,10 @@ hipError_t launch_bwd_td(const Params &p, hipStream_t stream) {
     constexpr int RPB = 256 / (D / 8);
     dot_do_o_kernel<T, D><<<dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(256), 0, stream>>>(p);
   }
-  constexpr int KB = DkdvGeom<D>::KB;
   Params pk = p;
-  pk.n_nblocks = (p.sk + kKvBlock * KB - 1) / (kKvBlock * KB);
+  pk.n_nblocks = (p.sk + kKvBlock - 1) / kKvBlock;
   if (pk.n_nblocks > 0)
-    dkdv_kernel<T, D, KB><<<dim3((unsigned)(pk.n_nblocks * p.b * p.h)), dim3(256), 0, stream>>>(pk);
+    dkdv_kernel<T, D><<<dim3((unsigned)(pk.n_nblocks * p.b * p.h)), dim3(256), 0, stream>>>(pk);
   Params pq = p;
   pq.n_mblocks = (p.sq + kQBlock - 1) / kQBlock;
   if (pq.n_mblocks > 0)
