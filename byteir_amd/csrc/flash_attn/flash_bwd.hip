@@ -104,8 +104,10 @@ struct TileLoader {
 // The step has a single instance: window edges are applied as -inf scores between A and B, a
 // unit that the wave's keys do not see at all is treated like an edge unit (it adds zeros),
 // and the first step accumulates a zero P / dS.
-template <typename T, int D>
-__global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) dkdv_kernel(const Params p) {
+// KB: 32-key blocks per wave; the workgroup covers 128*KB keys and every Q / dO fragment read
+// from LDS feeds KB MFMAs.
+template <typename T, int D, int KB>
+__global__ void __launch_bounds__(256, (D <= 64 && KB == 1) ? 2 : 1) dkdv_kernel(const Params p) {
   using vec8 = typename Traits<T>::vec8;
   constexpr int QS = D + 16;  // tiles are read both plainly and transposed
   constexpr int kRing = 3;
@@ -132,8 +134,9 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) dkdv_kernel(const Params
     }
   }
   const int bi = bh / p.h, hi = bh % p.h;
-  const int kvb0 = n_block * kKvBlock;
-  const int wkv0 = kvb0 + wave * 32;  // first key of the wave
+  constexpr int kKeys = kKvBlock * KB;
+  const int kvb0 = n_block * kKeys;
+  const int wkv0 = kvb0 + wave * 32 * KB;  // first key of the wave
   const int off = p.sk - p.sq;
 
   const T *qg = static_cast<const T *>(p.q) + bi * p.q_bs + hi * p.q_hs;
@@ -141,33 +144,39 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) dkdv_kernel(const Params
   const float *lse_g = p.lse + ((int64_t)bi * p.h + hi) * p.sq;
   const float *dsm_g = p.dsoftmax + ((int64_t)bi * p.h + hi) * p.sq_rounded;
 
-  const int kvcol = wkv0 + r32;  // the key this lane owns
-  vec8 kf[D / 16], vf[D / 16];
-  {
-    const T *kg = static_cast<const T *>(p.k) + bi * p.k_bs + (int64_t)kvcol * p.k_rs + hi * p.k_hs;
-    const T *vg = static_cast<const T *>(p.v) + bi * p.v_bs + (int64_t)kvcol * p.v_rs + hi * p.v_hs;
+  int kvcol[KB];  // the keys this lane owns
+  vec8 kf[KB][D / 16], vf[KB][D / 16];
+#pragma unroll
+  for (int kb = 0; kb < KB; ++kb) {
+    kvcol[kb] = wkv0 + kb * 32 + r32;
+    const T *kg = static_cast<const T *>(p.k) + bi * p.k_bs + (int64_t)kvcol[kb] * p.k_rs + hi * p.k_hs;
+    const T *vg = static_cast<const T *>(p.v) + bi * p.v_bs + (int64_t)kvcol[kb] * p.v_rs + hi * p.v_hs;
 #pragma unroll
     for (int ks = 0; ks < D / 16; ++ks) {
-      if (kvcol < p.sk) {
-        kf[ks] = *reinterpret_cast<const vec8 *>(kg + ks * 16 + g * 8);
-        vf[ks] = *reinterpret_cast<const vec8 *>(vg + ks * 16 + g * 8);
+      if (kvcol[kb] < p.sk) {
+        kf[kb][ks] = *reinterpret_cast<const vec8 *>(kg + ks * 16 + g * 8);
+        vf[kb][ks] = *reinterpret_cast<const vec8 *>(vg + ks * 16 + g * 8);
       } else {
-        kf[ks] = vec8{0};
-        vf[ks] = vec8{0};
+        kf[kb][ks] = vec8{0};
+        vf[kb][ks] = vec8{0};
       }
     }
   }
   // consume the fragments once so that the wait for their loads sits here, not inside the loop
 #pragma unroll
-  for (int ks = 0; ks < D / 16; ++ks) asm volatile("" : "+v"(kf[ks]), "+v"(vf[ks]));
-  float16v dk_acc[D / 32], dv_acc[D / 32];
+  for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
-  for (int i = 0; i < D / 32; ++i) { dk_acc[i] = float16v{0}; dv_acc[i] = float16v{0}; }
+    for (int ks = 0; ks < D / 16; ++ks) asm volatile("" : "+v"(kf[kb][ks]), "+v"(vf[kb][ks]));
+  float16v dk_acc[KB][D / 32], dv_acc[KB][D / 32];
+#pragma unroll
+  for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+    for (int i = 0; i < D / 32; ++i) { dk_acc[kb][i] = float16v{0}; dv_acc[kb][i] = float16v{0}; }
 
-  // query tiles that can see keys [kvb0, kvb0 + 128)
+  // query tiles that can see keys [kvb0, kvb0 + kKeys)
   int q_lo = 0, q_hi = p.sq;
   if (p.wr >= 0) q_lo = max(0, kvb0 - off - p.wr);                 // hi(q) = q+1+off+wr > kvb0
-  if (p.wl >= 0) q_hi = min(p.sq, kvb0 + kKvBlock - off + p.wl);   // lo(q) = q+off-wl < kvb0+128
+  if (p.wl >= 0) q_hi = min(p.sq, kvb0 + kKeys - off + p.wl);      // lo(q) = q+off-wl < kvb0+kKeys
   const int m_min = q_lo / kQTile;
   const int m_max = q_hi > 0 ? (q_hi + kQTile - 1) / kQTile : 0;
   const float c = p.scale_log2;
@@ -196,33 +205,38 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) dkdv_kernel(const Params
     if (tid < kQTile) { lse_s[buf][tid] = lse_r * kLog2e; dsm_s[buf][tid] = dsm_r; }
   };
 
-  struct Unit { float16v s, dp; };
+  struct Unit { float16v s[KB], dp[KB]; };
   const int frag_rd = r32 * QS + g * 8;  // this lane's plain fragment inside a 32-row unit
 
   // A: S = Q K^T, dP = dO V^T for the 32 query rows of unit `qs` of a tile
   auto part_a = [&](const T *Qt, const T *dOt, int qs, Unit &u) {
-    u.s = float16v{0};
-    u.dp = float16v{0};
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb) { u.s[kb] = float16v{0}; u.dp[kb] = float16v{0}; }
 #pragma unroll
     for (int ks = 0; ks < D / 16; ++ks) {
       const vec8 aq = lds_read8<T>(&Qt[qs * 32 * QS + frag_rd + ks * 16]);
       const vec8 ad = lds_read8<T>(&dOt[qs * 32 * QS + frag_rd + ks * 16]);
-      u.s = Traits<T>::mfma(aq, kf[ks], u.s);
-      u.dp = Traits<T>::mfma(ad, vf[ks], u.dp);
+#pragma unroll
+      for (int kb = 0; kb < KB; ++kb) {
+        u.s[kb] = Traits<T>::mfma(aq, kf[kb][ks], u.s[kb]);
+        u.dp[kb] = Traits<T>::mfma(ad, vf[kb][ks], u.dp[kb]);
+      }
     }
   };
   // scores outside the window become -inf (P = 0): key - (query + sk - sq) must lie in
   // [-wl, wr], one unsigned compare per element
   auto mask = [&](Unit &u, int q0) {
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const unsigned rel = (unsigned)(kvcol - off - q0 - g * 4 - ((i >> 2) * 8 + (i & 3)) - win_lo);
-      if (rel > win_span) u.s[i] = -INFINITY;
-    }
+    for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const unsigned rel = (unsigned)(kvcol[kb] - off - q0 - g * 4 - ((i >> 2) * 8 + (i & 3)) - win_lo);
+        if (rel > win_span) u.s[kb][i] = -INFINITY;
+      }
   };
   // B: P and dS of the unit, rounded and packed as B operands [16-query window]
-  auto part_b = [&](Unit &u, int buf, int qs, vec8 (&pb)[2], vec8 (&dsb)[2]) {
-    float pv[16], dsv[16];
+  auto part_b = [&](Unit &u, int buf, int qs, vec8 (&pb)[KB][2], vec8 (&dsb)[KB][2]) {
+    float pv[KB][16], dsv[KB][16];
 #pragma unroll
     for (int i4 = 0; i4 < 4; ++i4) {
       const int ql = qs * 32 + i4 * 8 + g * 4;  // 4 consecutive rows of the LDS tile
@@ -230,29 +244,36 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) dkdv_kernel(const Params
       const float4 d4 = *reinterpret_cast<const float4 *>(&dsm_s[buf][ql]);
       const float lq4[4] = {l4.x, l4.y, l4.z, l4.w}, dq4[4] = {d4.x, d4.y, d4.z, d4.w};
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int i = i4 * 4 + j;
-        const float pe = exp2_fast(fmaf(u.s[i], c, -lq4[j]));
-        pv[i] = pe;
-        dsv[i] = pe * (u.dp[i] - dq4[j]);
-      }
+      for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int i = i4 * 4 + j;
+          const float pe = exp2_fast(fmaf(u.s[kb][i], c, -lq4[j]));
+          pv[kb][i] = pe;
+          dsv[kb][i] = pe * (u.dp[kb][i] - dq4[j]);
+        }
     }
 #pragma unroll
-    for (int w = 0; w < 2; ++w) {
-      pb[w] = pack8<T>(&pv[w * 8]);
-      dsb[w] = pack8<T>(&dsv[w * 8]);
-    }
+    for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+      for (int w = 0; w < 2; ++w) {
+        pb[kb][w] = pack8<T>(&pv[kb][w * 8]);
+        dsb[kb][w] = pack8<T>(&dsv[kb][w * 8]);
+      }
   };
   // C: dV^T += dO^T P, dK^T += Q^T dS
-  auto part_c = [&](const T *Qt, const T *dOt, int qs, const vec8 (&pb)[2], const vec8 (&dsb)[2]) {
+  auto part_c = [&](const T *Qt, const T *dOt, int qs, const vec8 (&pb)[KB][2], const vec8 (&dsb)[KB][2]) {
 #pragma unroll
     for (int w = 0; w < 2; ++w)
 #pragma unroll
       for (int db = 0; db < D / 32; ++db) {
         const vec8 a_do = lds_read_operand_tr<T>(dOt, QS, qs * 32 + w * 16, db * 32);
         const vec8 a_q = lds_read_operand_tr<T>(Qt, QS, qs * 32 + w * 16, db * 32);
-        dv_acc[db] = Traits<T>::mfma(a_do, pb[w], dv_acc[db]);
-        dk_acc[db] = Traits<T>::mfma(a_q, dsb[w], dk_acc[db]);
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb) {
+          dv_acc[kb][db] = Traits<T>::mfma(a_do, pb[kb][w], dv_acc[kb][db]);
+          dk_acc[kb][db] = Traits<T>::mfma(a_q, dsb[kb][w], dk_acc[kb][db]);
+        }
       }
   };
   // does the window keep every (query, key) pair of the 32 rows from q0 and the wave's keys?
@@ -260,20 +281,24 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) dkdv_kernel(const Params
     int lo_first, hi_first, lo_last, hi_last;
     row_limits(p, q0, lo_first, hi_first);
     row_limits(p, q0 + 31, lo_last, hi_last);
-    return wkv0 + 32 <= hi_first && wkv0 >= lo_last;
+    return wkv0 + 32 * KB <= hi_first && wkv0 >= lo_last;
   };
-  vec8 pb[2], dsb[2];  // packed P and dS of the previous unit, still to be accumulated
+  vec8 pb[KB][2], dsb[KB][2];  // packed P and dS of the previous unit, still to be accumulated
 #pragma unroll
-  for (int w = 0; w < 2; ++w) { pb[w] = vec8{0}; dsb[w] = vec8{0}; }
+  for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+    for (int w = 0; w < 2; ++w) { pb[kb][w] = vec8{0}; dsb[kb][w] = vec8{0}; }
   auto step = [&](int buf, int qs, int q0, int pbuf, int pqs) {
     Unit u;
     part_a(Qs[buf], dOs[buf], qs, u);
     if (!all_kept(q0)) mask(u, q0);
-    vec8 pb_new[2], dsb_new[2];
+    vec8 pb_new[KB][2], dsb_new[KB][2];
     part_c(Qs[pbuf], dOs[pbuf], pqs, pb, dsb);
     part_b(u, buf, qs, pb_new, dsb_new);
 #pragma unroll
-    for (int w = 0; w < 2; ++w) { pb[w] = pb_new[w]; dsb[w] = dsb_new[w]; }
+    for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+      for (int w = 0; w < 2; ++w) { pb[kb][w] = pb_new[kb][w]; dsb[kb][w] = dsb_new[kb][w]; }
   };
 
   // prologue: tiles m_min and m_min+1 into the ring, tile m_min+2 into registers
@@ -303,23 +328,26 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) dkdv_kernel(const Params
   }
   if (n_tiles > 0) part_c(Qs[pbuf], dOs[pbuf], 1, pb, dsb);
 
-  if (kvcol < p.sk) {
-    T *dkg = static_cast<T *>(p.dk) + bi * p.k_bs + (int64_t)kvcol * p.k_rs + hi * p.k_hs;
-    T *dvg = static_cast<T *>(p.dv) + bi * p.v_bs + (int64_t)kvcol * p.v_rs + hi * p.v_hs;
-    typedef T vec4 __attribute__((ext_vector_type(4)));
 #pragma unroll
-    for (int db = 0; db < D / 32; ++db)
+  for (int kb = 0; kb < KB; ++kb) {
+    if (kvcol[kb] < p.sk) {
+      T *dkg = static_cast<T *>(p.dk) + bi * p.k_bs + (int64_t)kvcol[kb] * p.k_rs + hi * p.k_hs;
+      T *dvg = static_cast<T *>(p.dv) + bi * p.v_bs + (int64_t)kvcol[kb] * p.v_rs + hi * p.v_hs;
+      typedef T vec4 __attribute__((ext_vector_type(4)));
 #pragma unroll
-      for (int i4 = 0; i4 < 4; ++i4) {
-        vec4 a, b;
+      for (int db = 0; db < D / 32; ++db)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          a[j] = (T)(dk_acc[db][i4 * 4 + j] * p.scale);
-          b[j] = (T)(dv_acc[db][i4 * 4 + j]);
+        for (int i4 = 0; i4 < 4; ++i4) {
+          vec4 a, b;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            a[j] = (T)(dk_acc[kb][db][i4 * 4 + j] * p.scale);
+            b[j] = (T)(dv_acc[kb][db][i4 * 4 + j]);
+          }
+          *reinterpret_cast<vec4 *>(dkg + db * 32 + i4 * 8 + g * 4) = a;
+          *reinterpret_cast<vec4 *>(dvg + db * 32 + i4 * 8 + g * 4) = b;
         }
-        *reinterpret_cast<vec4 *>(dkg + db * 32 + i4 * 8 + g * 4) = a;
-        *reinterpret_cast<vec4 *>(dvg + db * 32 + i4 * 8 + g * 4) = b;
-      }
+    }
   }
 }
 
@@ -525,10 +553,15 @@ hipError_t launch_bwd_td(const Params &p, hipStream_t stream) {
     constexpr int RPB = 256 / (D / 8);
     dot_do_o_kernel<T, D><<<dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(256), 0, stream>>>(p);
   }
+  // One 32-key block per wave.  Two blocks halve the LDS reads per MFMA (LDS bandwidth is
+  // what bounds this kernel) but need about 450 registers: one wave per SIMD and accumulators
+  // in AccVGPRs, whose results reach the vector ALU through a v_accvgpr_read per value;
+  // measured 1.43 ms against 1.31 ms on the bf16 head_dim-64 benchmark.
+  constexpr int KB = 1;
   Params pk = p;
-  pk.n_nblocks = (p.sk + kKvBlock - 1) / kKvBlock;
+  pk.n_nblocks = (p.sk + kKvBlock * KB - 1) / (kKvBlock * KB);
   if (pk.n_nblocks > 0)
-    dkdv_kernel<T, D><<<dim3((unsigned)(pk.n_nblocks * p.b * p.h)), dim3(256), 0, stream>>>(pk);
+    dkdv_kernel<T, D, KB><<<dim3((unsigned)(pk.n_nblocks * p.b * p.h)), dim3(256), 0, stream>>>(pk);
   Params pq = p;
   pq.n_mblocks = (p.sq + kQBlock - 1) / kQBlock;
   if (pq.n_mblocks > 0)
