@@ -109,7 +109,10 @@ struct TileLoader {
 template <typename T, int D, int KB>
 __global__ void __launch_bounds__(256, (D <= 64 && KB == 1) ? 2 : 1) dkdv_kernel(const Params p) {
   using vec8 = typename Traits<T>::vec8;
-  constexpr int QS = D + 16;  // tiles are read both plainly and transposed
+  // Tiles are read both plainly and transposed.  A stride of 4*odd banks keeps the plain reads
+  // free of bank conflicts; the transposed ones then conflict in about a fifth of the LDS
+  // cycles (a third with D + 16, nearly half with D + 32) -- with < 3 % effect on the time.
+  constexpr int QS = Pad<D>::kPlain;
   constexpr int kRing = 3;
   __shared__ __attribute__((aligned(16))) T Qs[kRing][kQTile * QS];
   __shared__ __attribute__((aligned(16))) T dOs[kRing][kQTile * QS];
@@ -359,12 +362,13 @@ __global__ void __launch_bounds__(256, (D <= 64 && KB == 1) ? 2 : 1) dkdv_kernel
 // ALU); C: dQ^T += K^T dS^T (MFMA, K^T through the transposing LDS read).  The loop is
 // software pipelined like the forward kernel: one step holds A of the next unit together
 // with B and C of the current one in a single basic block, so that matrix instructions run
-// under the exponentials.  Window edges are applied beforehand, by setting the masked scores
+// under the exponentials, and the K / V fragments of a unit are fetched from LDS a step before
+// that.  Window edges are applied beforehand, by setting the masked scores
 // of an edge unit to -inf in a block of their own, which keeps B free of branches.
 template <typename T, int D>
 __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) dq_kernel(const Params p) {
   using vec8 = typename Traits<T>::vec8;
-  constexpr int KS = D + 16;          // K tile: plain and transposed reads
+  constexpr int KS = Pad<D>::kPlain;  // K tile: plain and transposed reads (see dkdv_kernel)
   constexpr int VS = Pad<D>::kPlain;  // V tile: plain reads only
   constexpr int kRing = 3;
   __shared__ __attribute__((aligned(16))) T Ks[kRing][kKvTile * KS];
@@ -445,16 +449,24 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) dq_kernel(const Params p
     if (kv0 >= w_hi_last || kv0 + 32 <= w_lo_first) return 0;
     return (kv0 + 32 > w_hi_first || kv0 < w_lo_last) ? 2 : 1;
   };
-  // A: S^T = K Q^T, dP^T = V dO^T for 32-key unit `kvb` of a tile
-  auto part_a = [&](const T *Kt, const T *Vt, int kvb, Unit &u) {
+  // K and V fragments of one 32-key unit, fetched from LDS one step before the MFMAs that
+  // use them, so that the LDS latency is not on the path of the step that consumes them
+  vec8 fk[D / 16], fv[D / 16];
+  auto fetch = [&](const T *Kt, const T *Vt, int kvb) {
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ++ks) {
+      fk[ks] = lds_read8<T>(&Kt[kvb * 32 * KS + frag_k + ks * 16]);
+      fv[ks] = lds_read8<T>(&Vt[kvb * 32 * VS + frag_v + ks * 16]);
+    }
+  };
+  // A: S^T = K Q^T, dP^T = V dO^T for the unit whose fragments are in fk / fv
+  auto part_a = [&](Unit &u) {
     u.s = float16v{0};
     u.dp = float16v{0};
 #pragma unroll
     for (int ks = 0; ks < D / 16; ++ks) {
-      const vec8 ak = lds_read8<T>(&Kt[kvb * 32 * KS + frag_k + ks * 16]);
-      const vec8 av = lds_read8<T>(&Vt[kvb * 32 * VS + frag_v + ks * 16]);
-      u.s = Traits<T>::mfma(ak, qf[ks], u.s);
-      u.dp = Traits<T>::mfma(av, dof[ks], u.dp);
+      u.s = Traits<T>::mfma(fk[ks], qf[ks], u.s);
+      u.dp = Traits<T>::mfma(fv[ks], dof[ks], u.dp);
     }
   };
   // the scores of an edge unit that fall outside the row's window become -inf (P = 0)
@@ -496,10 +508,11 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) dq_kernel(const Params p
   // last tile reads a stale ring slot whose result is never used.  Variants of the step would
   // each accumulate into dQ, and the register allocator then reconciles their assignments
   // with 16 moves (and a drain of the matrix pipe) at the end of every step.
-  auto step = [&](int vis, Unit &cur, int kv0, int buf, int kvb, Unit &nxt, int nbuf, int nkvb) {
+  auto step = [&](int vis, Unit &cur, int kv0, int buf, int kvb, Unit &nxt, int fbuf, int fkvb) {
     if (vis != 1) mask(cur, kv0);
     vec8 dsb[2];
-    part_a(Ks[nbuf], Vs[nbuf], nkvb, nxt);
+    part_a(nxt);                        // the next unit, from the fragments fetched a step ago
+    fetch(Ks[fbuf], Vs[fbuf], fkvb);    // fragments of the unit after next
     part_b(cur, dsb);
     part_c(Ks[buf], kvb, dsb);
   };
@@ -513,21 +526,23 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) dq_kernel(const Params p
     if (n_tiles > 1) { gload(); lstore(1); }
     if (n_tiles > 2) gload();
     __syncthreads();
-    part_a(Ks[0], Vs[0], 0, ua);
+    fetch(Ks[0], Vs[0], 0);
+    part_a(ua);
+    fetch(Ks[0], Vs[0], 1);
   }
   int buf = 0;  // ring slot of tile t
   for (int t = n_min; t < n_max; ++t) {
     const int buf1 = buf + 1 == kRing ? 0 : buf + 1;
     const int buf2 = buf1 + 1 == kRing ? 0 : buf1 + 1;
     const int kv0 = t * kKvTile;
-    // unit 0 of tile t (in ua) while unit 1 is produced into ub
-    step(visibility(kv0), ua, kv0, buf, 0, ub, buf, 1);
-    __syncthreads();  // tile t+1 is visible; every wave has left tile t-1
+    if (t > n_min) __syncthreads();  // tile t+1 is visible; every wave has left tile t-1
     // tile t+2: registers -> the ring slot tile t-1 occupied; tile t+3 in flight
     if (t + 2 < n_max) lstore(buf2);
     if (t + 3 < n_max) gload();
-    // unit 1 of tile t (in ub) while unit 0 of tile t+1 is produced into ua
-    step(visibility(kv0 + 32), ub, kv0 + 32, buf, 1, ua, buf1, 0);
+    // unit 0 of tile t (in ua); unit 1 is produced into ub; fragments of unit 0 of tile t+1
+    step(visibility(kv0), ua, kv0, buf, 0, ub, buf1, 0);
+    // unit 1 of tile t (in ub); unit 0 of tile t+1 into ua; fragments of its unit 1
+    step(visibility(kv0 + 32), ub, kv0 + 32, buf, 1, ua, buf1, 1);
     buf = buf1;
   }
 
