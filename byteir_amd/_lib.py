@@ -114,6 +114,8 @@ def brt():
         L.brt_session_load_text.argtypes = [vp, cp]
         L.brt_register_kernels_from_dynlib.argtypes = [cp]
         L.brt_session_has_kernel.argtypes = [vp, cp]
+        L.brt_session_intermediate_bytes.argtypes = [vp, cp]
+        L.brt_session_intermediate_bytes.restype = ctypes.c_size_t
         L.brt_session_arg_num.argtypes = [vp]
         L.brt_session_arg_num.restype = sz
         L.brt_session_arg_offset.argtypes = [vp, cp]

@@ -99,6 +99,10 @@ class Session:
     def get_space(self, offset):
         return _brt().brt_session_arg_space(self._h, offset).decode()
 
+    def get_intermediate_bytes(self, space):
+        """size of the per-frame arena for the memref.alloc intermediates of a memory space"""
+        return _brt().brt_session_intermediate_bytes(self._h, space.encode())
+
     def get_op_keys(self):
         B = _brt()
         return [B.brt_session_op_key(self._h, i).decode() for i in range(B.brt_session_op_num(self._h))]

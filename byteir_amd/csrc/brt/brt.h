@@ -185,6 +185,7 @@ private:
   std::vector<void *> base_;        // per value: bound/allocated pointer (aliases resolved lazily)
   std::vector<bool> owned_;         // allocated by the frame
   std::vector<void *> state_;       // per op
+  std::vector<std::pair<std::string, void *>> arenas_;  // one block per memory space for the intermediates
   const ir::ByREHandle *ir_ = nullptr;
   bool prologue_done_ = false;
   bool io_bound_ = false;
@@ -358,6 +359,11 @@ public:
   size_t GetArgNum() const;
   int GetGraphArgOffset(const std::string &name) const;
   const std::vector<size_t> &GetInputArgOffsets() const { return in_offsets_; }
+  // bytes of the per-frame arena that holds the intermediates of memory space `space`
+  size_t GetIntermediateBytes(const std::string &space) const {
+    auto it = arena_bytes_.find(space);
+    return it == arena_bytes_.end() ? 0 : it->second;
+  }
   const std::vector<size_t> &GetOutputArgOffsets() const { return out_offsets_; }
   const std::vector<size_t> &GetWeightArgOffsets() const { return weight_offsets_; }
   std::string GetArgName(size_t offset) const;
@@ -380,6 +386,11 @@ private:
   std::vector<std::shared_ptr<OpKernel>> kernels_;
   std::vector<std::unique_ptr<OpKernelInfo>> infos_;
   std::vector<size_t> in_offsets_, out_offsets_, weight_offsets_;
+  // static memory plan of the memref.alloc intermediates: byte offset of each value inside the
+  // arena of its memory space (SIZE_MAX: not an intermediate, or never used by an op), and
+  // the arena sizes
+  std::vector<size_t> intermediate_offset_;
+  std::unordered_map<std::string, size_t> arena_bytes_;
   std::function<WorkQueue *()> wq_factory_;
 };
 

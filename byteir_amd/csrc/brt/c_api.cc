@@ -75,6 +75,9 @@ int brt_session_has_kernel(brt_session *, const char *key) {
 }
 
 size_t brt_session_arg_num(brt_session *s) { return s->session.GetArgNum(); }
+size_t brt_session_intermediate_bytes(brt_session *s, const char *space) {
+  return s->session.GetIntermediateBytes(space ? space : "");
+}
 int brt_session_arg_offset(brt_session *s, const char *name) { return s->session.GetGraphArgOffset(name); }
 const char *brt_session_arg_name(brt_session *s, size_t offset) {
   try { s->scratch = s->session.GetArgName(offset); } catch (...) { s->scratch.clear(); }

@@ -261,6 +261,23 @@ common::Status Session::BuildPlan() {
     if ((v.arg_index >= 0 || v.is_alloc) && !allocators_.count(v.type.space))
       return common::Status::Fail("no allocator for memory space \"" + v.type.space + "\" (value " + v.name + ")");
   }
+  // Static memory plan (execution_plan.cc:473-578): walking the ops in order, every
+  // memref.alloc intermediate gets, at its first use, the next kAllocAlignment-rounded offset
+  // in the arena of its memory space; aliases resolve through their source.  No reuse of
+  // dead ranges, as in the reference.
+  intermediate_offset_.assign(ir_->values.size(), SIZE_MAX);
+  arena_bytes_.clear();
+  for (const ir::Op &op : ir_->ops) {
+    for (int operand : op.operands) {
+      int v = operand;
+      while (ir_->values[(size_t)v].alias_of >= 0) v = ir_->values[(size_t)v].alias_of;
+      const ir::Value &val = ir_->values[(size_t)v];
+      if (!val.is_alloc || intermediate_offset_[(size_t)v] != SIZE_MAX) continue;
+      size_t &total = arena_bytes_[val.type.space];
+      intermediate_offset_[(size_t)v] = total;
+      total += (val.type.Bytes() + kAllocAlignment - 1) / kAllocAlignment * kAllocAlignment;
+    }
+  }
   for (size_t i = 0; i < ir_->ops.size(); ++i) {
     const std::string &key = ir_->ops[i].key;
     ExecutionProvider *chosen = nullptr;
@@ -344,6 +361,10 @@ void Session::Cleanup(RequestContext &request) noexcept {
       f.owned_[i] = false;
     }
   }
+  for (auto &arena : f.arenas_) {
+    if (IAllocator *a = GetAllocator(arena.first)) a->Free(arena.second);
+  }
+  f.arenas_.clear();
 }
 
 // ---- request context --------------------------------------------------------------------------------------
@@ -365,10 +386,28 @@ common::Status RequestContext::BindArg(size_t offset, const void *value, BrtOwne
 // from the allocator named by the memref's memory space (execution_frame.cc:160-184)
 void RequestContext::FinishIOBinding() {
   const ir::ByREHandle &ir = *session_.ir_;
+  // intermediates: one arena per memory space, laid out by the session's static plan
+  // (BRTInferenceExecutionFrame, execution_frame.cc:60-120)
+  if (frame_->arenas_.empty()) {
+    for (const auto &kv : session_.arena_bytes_) {
+      if (kv.second == 0) continue;
+      IAllocator *a = session_.GetAllocator(kv.first);
+      BRT_ENFORCE(a != nullptr, "no allocator for space " + kv.first);
+      void *block = a->Alloc(kv.second);
+      BRT_ENFORCE(block != nullptr, "allocation of the intermediate arena failed");
+      frame_->arenas_.emplace_back(kv.first, block);
+    }
+    for (size_t i = 0; i < ir.values.size(); ++i) {
+      const size_t off = session_.intermediate_offset_[i];
+      if (off == SIZE_MAX) continue;
+      for (const auto &arena : frame_->arenas_)
+        if (arena.first == ir.values[i].type.space) frame_->base_[i] = static_cast<char *>(arena.second) + off;
+    }
+  }
   for (size_t i = 0; i < ir.values.size(); ++i) {
     const ir::Value &v = ir.values[i];
     if (frame_->base_[i] || v.alias_of >= 0) continue;
-    if (v.arg_index < 0 && !v.is_alloc) continue;
+    if (v.arg_index < 0) continue;  // an intermediate no op uses needs no memory
     IAllocator *a = session_.GetAllocator(v.type.space);
     BRT_ENFORCE(a != nullptr, "no allocator for space " + v.type.space);
     const size_t bytes = (v.type.Bytes() + kAllocAlignment - 1) / kAllocAlignment * kAllocAlignment;

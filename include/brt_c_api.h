@@ -51,6 +51,10 @@ size_t brt_session_arg_rank(brt_session *s, size_t offset);
 void brt_session_arg_shape(brt_session *s, size_t offset, int64_t *shape_out);
 const char *brt_session_arg_dtype(brt_session *s, size_t offset);   /* "f32", "f16", "bf16", "i64", ... */
 const char *brt_session_arg_space(brt_session *s, size_t offset);
+/* bytes of the per-frame arena that holds all memref.alloc intermediates of memory space
+ * `space`, laid out by the static memory plan (bump allocation in order of first use, every
+ * tensor rounded up to 256 bytes; execution_plan.cc:473-578) */
+size_t brt_session_intermediate_bytes(brt_session *s, const char *space);
 size_t brt_session_op_num(brt_session *s);
 const char *brt_session_op_key(brt_session *s, size_t op_index);
 /* OpAccessor::GetAttrAsVoidPtr (op_accessor.cc:212-242) for op `op_index`: copies the packed

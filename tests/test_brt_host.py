@@ -254,3 +254,24 @@ def test_reference_kvcache_module_loads_unchanged(session, golden_dir):
     assert session.get_static_shape(1) == [2, 128, 3, 32]
     blob = session.get_op_attr_blob(0, "extra_args")
     assert blob == oracle.fa_kvcache_pack_args(2, 1, 128, 3, 3, 32, 1, 0.5, (-1, -1)).tobytes()
+
+
+def test_static_memory_plan_of_intermediates(session):
+    """memref.alloc intermediates share one arena per memory space: offsets in order of first
+    use, every tensor rounded up to 256 bytes, an alias adds nothing, an alloc no op uses gets
+    no room (StaticBRTExecutionPlan, execution_plan.cc:473-578)."""
+    text = """func.func @t(%h : memref<1000xf32, "cpu"> {byre.argname = "h", byre.argtype = 1: i32},
+                      %o : memref<1000xf32, "cpu"> {byre.argname = "o", byre.argtype = 2: i32}) attributes {byre.entry_point} {
+      %unused = memref.alloc() : memref<77xf32, "cuda">
+      %d0 = memref.alloc() : memref<1000xf32, "cuda">
+      %d1 = memref.alloc() : memref<4000xi8, "cuda">
+      %v1 = "byre.alias"(%d1) {offset = 0 : i64} : (memref<4000xi8, "cuda">) -> memref<1000xf32, "cuda">
+      %s0 = memref.alloc() : memref<3xf32, "cpu">
+      byre.compute @cpu2cuda(%h, %d0) : memref<1000xf32, "cpu">, memref<1000xf32, "cuda">
+      byre.compute @cuda2cuda(%d0, %v1) : memref<1000xf32, "cuda">, memref<1000xf32, "cuda">
+      byre.compute @cuda2cpu(%v1, %o) : memref<1000xf32, "cuda">, memref<1000xf32, "cpu">
+      return }"""
+    session.load_from_memory(text)
+    assert session.get_intermediate_bytes("cuda") == 4096 + 4096   # 4000 B -> 4096, twice
+    assert session.get_intermediate_bytes("cpu") == 0              # %s0 is never used
+    assert session.get_intermediate_bytes("nowhere") == 0

@@ -358,3 +358,47 @@ def test_flash_attn_kvcache_module_unchanged(session, golden_dir):
     got, want = host(o).astype(np.float32), g["out"].astype(np.float32)
     assert np.all(np.abs(got - want) <= 2.0 ** -10 * np.abs(want) + 1e-7)  # one fp16 ulp
     assert np.array_equal(host(kc), g["kcache_out"]) and np.array_equal(host(vc), g["vcache_out"])
+
+
+def test_intermediates_live_in_one_arena_per_frame():
+    """The memref.alloc intermediates of a module come out of ONE allocation per frame and
+    memory space (the static plan's arena), not one allocation each; data still flows through
+    them correctly, an alias included."""
+    from byteir_amd import brt
+    allocs = []
+
+    def alloc(n):
+        allocs.append(n)
+        return torch.cuda.caching_allocator_alloc(n)
+
+    s = brt.Session(device="ROCM", alloc_func=alloc, free_func=torch.cuda.caching_allocator_delete)
+    text = """func.func @t(%x : memref<64x4096xf32, "cuda"> {byre.argname = "x", byre.argtype = 1: i32},
+                      %y : memref<64xf32, "cuda"> {byre.argname = "y", byre.argtype = 2: i32}) attributes {byre.entry_point} {
+      %a = memref.alloc() : memref<64x4096xf32, "cuda">
+      %b = memref.alloc() : memref<1048576xi8, "cuda">
+      %bv = "byre.alias"(%b) {offset = 0 : i64} : (memref<1048576xi8, "cuda">) -> memref<64x4096xf32, "cuda">
+      %m = memref.alloc() : memref<64xf32, "cuda">
+      byre.compute @cuda2cuda(%x, %a) : memref<64x4096xf32, "cuda">, memref<64x4096xf32, "cuda">
+      byre.compute @cuda2cuda(%a, %bv) : memref<64x4096xf32, "cuda">, memref<64x4096xf32, "cuda">
+      byre.compute @ReduceMaxOp_f32_f32(%bv, %m) {dimensions = dense<[1]> : tensor<1xi64>} : memref<64x4096xf32, "cuda">, memref<64xf32, "cuda">
+      byre.compute @cuda2cuda(%m, %y) : memref<64xf32, "cuda">, memref<64xf32, "cuda">
+      return }"""
+    s.load_from_memory(text)
+    arena = 2 * 64 * 4096 * 4 + 256
+    assert s.get_intermediate_bytes("cuda") == arena
+    x = torch.randn((64, 4096), device="cuda")
+    y = torch.zeros(64, device="cuda")
+    req = s.new_request_context(torch.cuda.current_stream().cuda_stream)
+    req.bind_arg(0, x.data_ptr())
+    req.bind_arg(1, y.data_ptr())
+    req.finish_io_binding()
+    assert allocs == [arena]
+    for _ in range(2):
+        req.run()
+    req.sync()
+    from byteir_amd import ops
+    ws = ops.reduce_workspace_bytes(torch.float32, 64, 4096, 1)  # the reduce op's own per-frame workspace
+    assert allocs == ([arena, ws] if ws else [arena])
+    assert torch.equal(y, x.amax(dim=1))
+    req.close()
+    s.close()
