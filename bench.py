@@ -3,11 +3,11 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2] [--no-extras] [--pmc-probe]
 
-Prints ONE JSON line.  The headline workload (`config.workload`) is BASELINE.json configs[1]:
+Prints ONE JSON line.  The headline workload (`config.workload`) is the second of the benchmark configurations the repository's BASELINE.json lists:
 ReduceMaxOp_f32_f32 and ReduceSumOp_f32_f32 over axis 0 (column / two-pass split case) and over
 axis 1 of one [16384, 8192] float tensor; a "step" is those four op-kernel launches, `value` is
 the algorithmic bytes of a step divided by the step time, inputs resident in HBM.  The other
-BASELINE configurations (row sum, fused softmax, flash-attention forward and backward) are
+listed configurations (row sum, fused softmax, flash-attention forward and backward) are
 timed in the same run and reported under `all_configs`, each with its own roofline fraction and
 a CPU figure.
 
@@ -100,7 +100,7 @@ def main():
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c2", choices=["c2"])
-    ap.add_argument("--no-extras", action="store_true", help="skip the other BASELINE configs")
+    ap.add_argument("--no-extras", action="store_true", help="skip the other benchmark configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="counter-collection mode: one copy kernel of known size, then two steps")
@@ -246,7 +246,7 @@ def main():
 
 
 def extras(all_cfg, ev, ops, _lib, gen, args, np, torch):
-    """The remaining BASELINE configurations, timed with the same event machinery."""
+    """The remaining benchmark configurations, timed with the same event machinery."""
     import oracle
     steps, warm = max(5, args.steps // 2), max(2, args.warmup // 2)
     do_cpu = not args.no_cpu

@@ -14,7 +14,7 @@
  * What pins each function (see tests/test_oracle_*.py):
  *   shape canonicalisation / workspace rule : the reference test's shape list
  *       (runtime/test/backends/cuda/providers/default/kernel/reduction_test.cc:171-180),
- *       brute force by index decode, closed forms for the workspace of BASELINE's shapes.
+ *       brute force by index decode, closed forms for the workspace of the benchmark shapes.
  *   reduce sum / max                         : numpy (pairwise / exact), fp64, NaN cases.
  *   softmax                                  : scipy.special.softmax in fp64, shift
  *       invariance, rows summing to one, one-hot limit.

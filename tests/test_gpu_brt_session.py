@@ -17,7 +17,7 @@ pytestmark = pytest.mark.gpu
 REF_CASES = [
     ((1, 16, 32), (0,)), ((1, 16, 32), (1,)), ((1, 16, 32), (2,)), ((1, 16, 32), (0, 1)),
     ((1, 16, 32), (0, 2)), ((1, 128, 128), (0, 1)), ((2, 128, 256), (0, 1)), ((2, 16, 8, 64), (1, 2)),
-    ((16384, 8192), (0,)),  # BASELINE configs[1]: needs the per-frame workspace
+    ((16384, 8192), (0,)),  # the headline benchmark shape: needs the per-frame workspace
 ]
 
 

@@ -4,7 +4,7 @@
 Mirrors the reference's SM80CUDATestFlashAttnFwd.Basic / SM80CUDATestFlashAttnBwd.Basic
 (runtime/test/backends/cuda/providers/default/kernel/flash_attn_{fwd,bwd}_test.cc) on the
 reference's golden vectors, then widens to seeded random cases against the CPU oracle and to
-BASELINE's full-size configurations."""
+the full-size benchmark configurations."""
 import os
 
 import numpy as np

@@ -2,7 +2,7 @@
 
 Mirrors the reference's CUDATestReductionOp tests
 (runtime/test/backends/cuda/providers/default/kernel/reduction_test.cc:94-230): the same shape
-list, two runs on the same buffers, NaN propagation; plus BASELINE's full-size shapes."""
+list, two runs on the same buffers, NaN propagation; plus the full-size benchmark shapes."""
 import numpy as np
 import pytest
 import torch
@@ -112,7 +112,7 @@ def test_workspace_too_small_is_an_error():
 
 
 def test_baseline_config1_row_sum():
-    """[4096, 1024] f32 ~ N(0,1), reduce axis 1 (BASELINE configs[0])."""
+    """[4096, 1024] f32 ~ N(0,1), reduce axis 1 (the first benchmark configuration)."""
     from byteir_amd import ops
     x = np.random.default_rng(0xC1).standard_normal((4096, 1024)).astype(np.float32)
     got = host(ops.reduce(oracle.SUM, dev(x), (1,)))

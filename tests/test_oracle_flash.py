@@ -182,7 +182,7 @@ def test_extra_args_blob_known_answer():
     assert blob.tobytes() == want
     back = oracle.fa_unpack_args(blob)
     assert (back.seqlen_q, back.window_size_left, back.window_size_right, back.softmax_scale) == (128, -1, 0, 0.5)
-    # BASELINE config 4 strides
+    # strides of the causal fp16 benchmark configuration
     c4 = oracle.fa_args(4, 2048, 2048, 32, 32, 128, 1 / np.sqrt(128), window=(-1, 0))
     assert (c4.q_batch_stride, c4.q_row_stride, c4.q_head_stride) == (8388608, 4096, 128)
 

@@ -68,7 +68,7 @@ def test_canonicalize_rules():
     assert oracle.reduce_canonicalize((1, 7, 1), (7,), (0, 2)) == (0, 0, 0, 7)
     # out-of-range dimension
     assert oracle.reduce_canonicalize((4, 8), (4,), (2,))[0] == 3
-    # BASELINE shapes
+    # benchmark shapes
     assert oracle.reduce_canonicalize((4096, 1024), (4096,), (1,)) == (0, 4096, 1024, 1)
     assert oracle.reduce_canonicalize((16384, 8192), (8192,), (0,)) == (0, 1, 16384, 8192)
     assert oracle.reduce_canonicalize((16384, 8192), (16384,), (1,)) == (0, 16384, 8192, 1)
