@@ -29,8 +29,8 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E, published
 MFMA_PEAK_TFLOPS = 2500.0  # dense bf16 / fp16 MFMA, published
 
-# measured HBM bytes of one first-pass launch: 536 873 984 fetched + 2 097 152 written
-TRAFFIC_COL_FIRST_PASS = 538971136
+# measured HBM bytes of one first-pass launch: 536 894 846 fetched + 4 194 304 written
+TRAFFIC_COL_FIRST_PASS = 541089150
 
 METRIC = "reduce HBM GB/s + flash-attn fwd/bwd TFLOP/s, % of MI355X roofline, 1 GPU"
 
@@ -165,7 +165,7 @@ def main():
     # The axis-0 op is two launches: the split first pass (the dominant kernel) and a small
     # combine over the [S, 8192] partials.  A second timed region records an event between the
     # two (brt_rocm_reduce_ex), so `avg_launch_us` is the first pass alone (compare with
-    # rocprofv3's figure for reduce_col_kernel<..., 256>).
+    # rocprofv3's figure for reduce_colwide_kernel).
     n_mid = max(args.steps, 10)
     triples = [(ev.new(), ev.new(), ev.new()) for _ in range(2 * n_mid)]
     for i, (e0, e1, e2) in enumerate(triples):
@@ -180,7 +180,7 @@ def main():
         ev.free(t)
     col_gbs = bytes_col / (pass1_ms * 1e-3) / 1e9
     roofline = {
-        "bound": "hbm", "kernel": "reduce_col_kernel<float, float, OP, 4, 256> (first pass of the axis-0 split reduction)",
+        "bound": "hbm", "kernel": "reduce_colwide_kernel<float, float, OP, 4, 2, 2> (first pass of the axis-0 split reduction)",
         "achieved": round(col_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": round(col_gbs / HBM_PEAK_GBS, 4),
         "algorithmic_bytes_per_launch": bytes_col, "avg_launch_us": round(pass1_ms * 1e3, 2),

@@ -21,6 +21,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
+#include <type_traits>
 
 #include "brt_rocm_kernels.h"
 
@@ -31,6 +32,7 @@ namespace {
 // HBM efficiency (79 us against 82 us with eight for the [16384, 8192] column fold).
 constexpr int kRowU = 4;
 constexpr int kColU = 4;
+constexpr int kColWideW = 2, kColWideU = 2;  // column groups per lane and rows in flight, wide kernel
 constexpr int kBlock = 256;            // threads per workgroup (4 waves)
 constexpr uint64_t kFillThreads = 256ull * 1024;  // threads wanted in flight chip-wide
 
@@ -196,9 +198,78 @@ reduce_col_kernel(const T *__restrict__ in, TO *__restrict__ out, uint64_t B, ui
   }
 }
 
+// Wide tensors: a block of 256 lanes spans W * 4 KiB of a row, every lane owns W groups of
+// VEC adjacent columns 256 * VEC apart and keeps U rows in flight (W * U 128-bit loads per
+// lane).  No LDS: every lane stores its own columns.  Two groups with two rows in flight
+// measured fastest for the [16384, 8192] fold (77 us against 79.6 us with one group and
+// four rows), at the price of twice as many segments for the same 512 workgroups.
+template <typename T, typename TO, int OP, int VEC, int W, int U>
+__global__ void __launch_bounds__(kBlock)
+reduce_colwide_kernel(const T *__restrict__ in, TO *__restrict__ out, uint64_t B, uint64_t C,
+                      uint32_t S, uint64_t seg_rows, uint32_t col_tiles) {
+  uint64_t bid = blockIdx.x;
+  const uint32_t tile = bid % col_tiles; bid /= col_tiles;
+  const uint32_t s = bid % S;
+  const uint64_t a = bid / S;
+  const uint64_t c0 = ((uint64_t)tile * W * kBlock + threadIdx.x) * VEC;  // first group of this lane
+  constexpr uint64_t kGroupStep = (uint64_t)kBlock * VEC;
+  const uint64_t r0 = (uint64_t)s * seg_rows;
+  uint64_t r1 = r0 + seg_rows;
+  if (r1 > B) r1 = B;
+  const T *p = in + a * B * C + c0;
+  TO *o = out + (a * S + s) * C + c0;
+  // full: the whole tile lies inside the row (block-uniform), so the loads need no predicate
+  auto fold = [&](auto full_tag) {
+    constexpr bool kFull = decltype(full_tag)::value;
+    bool ok[W];
+#pragma unroll
+    for (int w = 0; w < W; ++w) ok[w] = kFull || c0 + w * kGroupStep < C;
+    float acc[W][VEC];
+#pragma unroll
+    for (int w = 0; w < W; ++w)
+#pragma unroll
+      for (int k = 0; k < VEC; ++k) acc[w][k] = Fold<OP>::init();
+    uint64_t r = r0;
+    for (; r + (U - 1) < r1; r += U) {
+      float v[U][W][VEC];
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int w = 0; w < W; ++w)
+          if (kFull || ok[w]) Loader<T, VEC>::load(p + (r + u) * C + w * kGroupStep, v[u][w]);
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int w = 0; w < W; ++w)
+          if (kFull || ok[w]) {
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) acc[w][k] = Fold<OP>::apply(acc[w][k], v[u][w][k]);
+          }
+    }
+    for (; r < r1; ++r) {
+#pragma unroll
+      for (int w = 0; w < W; ++w)
+        if (kFull || ok[w]) {
+          float v[VEC];
+          Loader<T, VEC>::load(p + r * C + w * kGroupStep, v);
+#pragma unroll
+          for (int k = 0; k < VEC; ++k) acc[w][k] = Fold<OP>::apply(acc[w][k], v[k]);
+        }
+    }
+#pragma unroll
+    for (int w = 0; w < W; ++w)
+      if (kFull || ok[w]) {
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) o[w * kGroupStep + k] = to_out<TO>(acc[w][k]);
+      }
+  };
+  if (((uint64_t)tile + 1) * W * kGroupStep <= C) fold(std::true_type{});
+  else fold(std::false_type{});
+}
+
 // ---- host-side planning -------------------------------------------------------------------
 struct Plan {
-  int kind;       // 0 copy, 1 row, 2 col
+  int kind;       // 0 copy, 1 row, 2 col, 3 wide col (reduce_colwide_kernel)
   int vec;        // elements per load when pointers are 16-byte aligned
   int g;          // row: lanes per unit; col: TX
   uint32_t S;     // segments of the fold axis
@@ -233,7 +304,10 @@ Plan make_plan(int dtype, uint64_t A, uint64_t B, uint64_t C, bool allow_split) 
   p.kind = 2;
   p.vec = (C % vec_full == 0) ? vec_full : 1;
   const uint64_t ncolv = ceil_div(C, p.vec);
-  if (allow_split) {
+  if (allow_split && p.vec > 1 && ncolv >= 2 * kBlock) {
+    p.kind = 3;  // 8 KiB of a row per block
+    p.g = kColWideW * kBlock;
+  } else if (allow_split) {
     // first (or only) pass: a block spans up to 256 lanes x 128 bits = 4 KiB of one row
     p.g = ncolv >= 256 ? 256 : ncolv > 32 ? 64 : ncolv > 8 ? 32 : 8;
   } else {
@@ -242,7 +316,7 @@ Plan make_plan(int dtype, uint64_t A, uint64_t B, uint64_t C, bool allow_split) 
     if (A * ceil_div(ncolv, 64) < 256) p.g = 32;
     if (A * ceil_div(ncolv, 32) < 256) p.g = 8;
   }
-  const int ty = kBlock / p.g;
+  const int ty = p.kind == 3 ? 1 : kBlock / p.g;
   p.col_tiles = (uint32_t)ceil_div(ncolv, p.g);
   const uint64_t blocks0 = A * p.col_tiles;
   uint64_t S = 1;
@@ -284,13 +358,22 @@ hipError_t launch(const Plan &p, const T *in, TO *out, uint64_t A, uint64_t B, u
 #undef ROW
     return hipGetLastError();
   }
-  const uint64_t blocks = A * p.S * p.col_tiles;
+  // The plan counts column tiles in 128-bit groups; a pointer that is not 16-byte aligned
+  // forces scalar loads at launch time, and the same segments are then covered by four (f32)
+  // or eight (f16) times as many tiles of the 256-lane kernel.
+  const int tx = (p.kind == 3 && !vec) ? kBlock : p.g;
+  const uint32_t col_tiles = vec ? p.col_tiles : (uint32_t)ceil_div(C, (uint64_t)tx);
+  const uint64_t blocks = A * p.S * col_tiles;
   if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
   const dim3 grid((unsigned)blocks), block(kBlock);
+  if (p.kind == 3 && vec) {
+    reduce_colwide_kernel<T, TO, OP, VF, kColWideW, kColWideU><<<grid, block, 0, stream>>>(in, out, B, C, p.S, p.seg, col_tiles);
+    return hipGetLastError();
+  }
 #define COL(TX)                                                                                  \
-  if (vec) reduce_col_kernel<T, TO, OP, VF, TX><<<grid, block, 0, stream>>>(in, out, B, C, p.S, p.seg, p.col_tiles); \
-  else reduce_col_kernel<T, TO, OP, 1, TX><<<grid, block, 0, stream>>>(in, out, B, C, p.S, p.seg, p.col_tiles)
-  switch (p.g) {
+  if (vec) reduce_col_kernel<T, TO, OP, VF, TX><<<grid, block, 0, stream>>>(in, out, B, C, p.S, p.seg, col_tiles); \
+  else reduce_col_kernel<T, TO, OP, 1, TX><<<grid, block, 0, stream>>>(in, out, B, C, p.S, p.seg, col_tiles)
+  switch (tx) {
   case 8: COL(8); break;
   case 32: COL(32); break;
   case 256: COL(256); break;

@@ -21,6 +21,8 @@ EXTRA_CASES = [
     ((7, 13), (1,)), ((7, 13), (0,)), ((3, 1000003), (1,)), ((1000003, 3), (0,)), ((5, 333, 7), (1,)),
     ((1, 1 << 20), (1,)), ((1 << 20,), (0,)), ((64, 4096), (1,)), ((4096, 64), (0,)), ((2, 5000, 36), (1,)),
     ((129, 1024), (1,)), ((1, 70000, 8), (1,)), ((300, 40), (1,)), ((16, 2049, 260), (1,)),
+    # wide rows (8 KiB of a row per block): whole tiles, a ragged last tile, few rows
+    ((4096, 8192), (0,)), ((300, 2600), (0,)), ((5, 40, 4104), (1,)), ((3, 2048), (0,)),
 ]
 
 
@@ -84,7 +86,7 @@ def test_max_of_all_minus_inf_and_inf():
 
 
 @pytest.mark.parametrize("shape,dims", [((64, 4096), (1,)), ((4096, 64), (0,)), ((3, 1001, 5), (1,)), ((1, 200000), (1,)),
-                                        ((2, 16, 8, 64), (1, 2))])
+                                        ((2, 16, 8, 64), (1, 2)), ((2000, 4104), (0,)), ((7, 8192), (0,))])
 @pytest.mark.parametrize("op", [oracle.SUM, oracle.MAX])
 def test_reduce_f16(shape, dims, op):
     from byteir_amd import ops
@@ -97,6 +99,29 @@ def test_reduce_f16(shape, dims, op):
         want = x.astype(np.float64).sum(axis=dims)
         sabs = np.abs(x.astype(np.float64)).sum(axis=dims)
         assert np.all(np.abs(got.astype(np.float64) - want) <= 2.0 ** -10 * np.abs(want) + 1e-6 * sabs + 1e-7)
+
+
+@pytest.mark.parametrize("shape,dims", [((1000, 4096), (0,)), ((1000, 4096), (1,)), ((3000, 64), (0,)), ((2, 500, 2048), (1,)),
+                                        ((40000, 8), (0,))])
+@pytest.mark.parametrize("op", [oracle.SUM, oracle.MAX])
+def test_input_that_is_not_16_byte_aligned(shape, dims, op):
+    """Extents that allow 128-bit loads but a pointer that does not: the launch falls back to
+    scalar loads and must still cover every column."""
+    from byteir_amd import ops
+    n = int(np.prod(shape))
+    x = np.random.default_rng(9).standard_normal(n).astype(np.float32)
+    buf = torch.zeros(n + 1, device="cuda")
+    buf[1:] = dev(x)
+    view = buf[1:].view(shape)
+    assert view.data_ptr() % 16 == 4
+    got = host(ops.reduce(op, view, dims))
+    xs = x.reshape(shape)
+    if op == oracle.MAX:
+        assert np.array_equal(got, xs.max(axis=dims[0]))
+    else:
+        out_shape = oracle.deduce_output_shape(shape, dims)
+        st, A, B, C = oracle.reduce_canonicalize(shape, out_shape, dims)
+        check_sum(got, xs, A, B, C)
 
 
 def test_workspace_too_small_is_an_error():
