@@ -62,22 +62,35 @@ class Events:
 
 def time_ops(ev, fns, steps, warmup):
     """Run `fns` (a list of launch closures = one step) `warmup` + `steps` times.
-    -> (ms per step by events, [ms per launch of fns[i]], ms per step by host clock)."""
+    -> (ms per step by events, [ms per launch of fns[i]], ms per step by host clock).
+    The step time comes from ONE pair of events around all `steps` steps (an event between every
+    two launches costs a few microseconds of idle GPU each); the per-launch breakdown is taken
+    in a second pass of the same length with an event after every launch."""
     import torch
     for _ in range(warmup):
         for f in fns:
             f()
     torch.cuda.synchronize()
-    marks = [[ev.new() for _ in range(len(fns) + 1)] for _ in range(steps)]
+    e0, e1 = ev.new(), ev.new()
     t0 = time.perf_counter()
+    ev.record(e0)
+    for _ in range(steps):
+        for f in fns:
+            f()
+    ev.record(e1)
+    torch.cuda.synchronize()
+    host_ms = (time.perf_counter() - t0) * 1e3 / steps
+    total = ev.elapsed_ms(e0, e1) / steps
+    ev.free([e0, e1])
+    if len(fns) == 1:
+        return total, [total], host_ms
+    marks = [[ev.new() for _ in range(len(fns) + 1)] for _ in range(steps)]
     for s in range(steps):
         ev.record(marks[s][0])
         for i, f in enumerate(fns):
             f()
             ev.record(marks[s][i + 1])
     torch.cuda.synchronize()
-    host_ms = (time.perf_counter() - t0) * 1e3 / steps
-    total = ev.elapsed_ms(marks[0][0], marks[-1][-1]) / steps
     per = [sum(ev.elapsed_ms(marks[s][i], marks[s][i + 1]) for s in range(steps)) / steps
            for i in range(len(fns))]
     for m in marks:
@@ -319,7 +332,8 @@ def extras(all_cfg, ev, ops, _lib, gen, args, np, torch):
     q, k, v = (torch.randn((4, 2048, 32, 128), generator=gen, device="cuda").half() for _ in range(3))
     sc4 = 1.0 / np.sqrt(128.0)
     fl4 = 4 * 4 * 32 * 2048 * 2048 * 128 // 2  # 137 438 953 472
-    ms4, _, _ = time_ops(ev, [lambda: ops.flash_attn_fwd(q, k, v, sc4, (-1, 0))], steps, warm)
+    fwd_out = (torch.empty_like(q), torch.empty((4, 32, 2048), device="cuda"), torch.zeros(2, dtype=torch.int64, device="cuda"))
+    ms4, _, _ = time_ops(ev, [lambda: ops.flash_attn_fwd(q, k, v, sc4, (-1, 0), out=fwd_out)], steps, warm)
     c4 = {"value": round(fl4 / (ms4 * 1e-3) / 1e12, 1), "unit": "TFLOP/s", "us_per_op": round(ms4 * 1e3, 1),
           "frac_of_mfma_peak": round(fl4 / (ms4 * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, 4), "flop": fl4}
     if do_cpu:
@@ -337,9 +351,11 @@ def extras(all_cfg, ev, ops, _lib, gen, args, np, torch):
     gen.manual_seed(0xC5)
     q, k, v, do = (torch.randn((2, 8192, 16, 64), generator=gen, device="cuda").bfloat16() for _ in range(4))
     fl5 = 4 * 2 * 16 * 8192 * 8192 * 64  # 549 755 813 888
-    msf, _, _ = time_ops(ev, [lambda: ops.flash_attn_fwd(q, k, v, 0.125, (-1, -1))], steps, warm)
+    fwd_out = (torch.empty_like(q), torch.empty((2, 16, 8192), device="cuda"), torch.zeros(2, dtype=torch.int64, device="cuda"))
+    msf, _, _ = time_ops(ev, [lambda: ops.flash_attn_fwd(q, k, v, 0.125, (-1, -1), out=fwd_out)], steps, warm)
     o, lse = ops.flash_attn_fwd(q, k, v, 0.125, (-1, -1))
-    msb, _, _ = time_ops(ev, [lambda: ops.flash_attn_bwd(do, q, k, v, o, lse, 0.125, (-1, -1))], max(3, steps // 3), 2)
+    bwd_out = ops.flash_attn_bwd_buffers(q, k, v)
+    msb, _, _ = time_ops(ev, [lambda: ops.flash_attn_bwd(do, q, k, v, o, lse, 0.125, (-1, -1), out=bwd_out)], max(3, steps // 3), 2)
     all_cfg["c5_flash_fwd_bf16"] = {
         "value": round(fl5 / (msf * 1e-3) / 1e12, 1), "unit": "TFLOP/s", "us_per_op": round(msf * 1e3, 1),
         "frac_of_mfma_peak": round(fl5 / (msf * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, 4), "flop": fl5}

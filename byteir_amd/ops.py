@@ -121,29 +121,40 @@ def _call_custom(fn, tensors, blob, stream):
     fn(arr, ctypes.cast(buf, ctypes.c_void_p), _stream(stream))
 
 
-def flash_attn_fwd(q, k, v, scale, window=(-1, -1), stream=None):
+def flash_attn_fwd(q, k, v, scale, window=(-1, -1), stream=None, out=None):
     """run_flash_attn_fwd: tensors {q, k, v, rng_state, o, softmax_lse, softmax_P}
-    (external_libs/runtime/flash_attn/lib/flash_api.cu:586-654). -> (o, lse[b,h,sq] f32)."""
+    (external_libs/runtime/flash_attn/lib/flash_api.cu:586-654). -> (o, lse[b,h,sq] f32).
+    out: optional (o, lse, rng_state) to write into instead of allocating."""
     L = _lib.flash_attn()
     b, sq, h, d = q.shape
-    o = torch.empty_like(q)
-    lse = torch.empty((b, h, sq), dtype=torch.float32, device=q.device)
-    rng = torch.zeros(2, dtype=torch.int64, device=q.device)
+    if out is not None:
+        o, lse, rng = out
+    else:
+        o = torch.empty_like(q)
+        lse = torch.empty((b, h, sq), dtype=torch.float32, device=q.device)
+        rng = torch.zeros(2, dtype=torch.int64, device=q.device)
     fn = L.run_flash_attn_fwd if q.dtype == torch.float16 else L.run_flash_attn_fwd_bf16
     _call_custom(fn, [q, k, v, rng, o, lse, None], pack_flash_args(q, k, v, o, scale, window), stream)
     return o, lse
 
 
-def flash_attn_bwd(dout, q, k, v, o, lse, scale, window=(-1, -1), stream=None):
-    """run_flash_attn_bwd: tensors {dout, q, k, v, out, softmax_lse, rng_state, dq, dk, dv,
-    d_softmax, dq_accum} (flash_api.cu:656-725). -> (dq, dk, dv)."""
-    L = _lib.flash_attn()
+def flash_attn_bwd_buffers(q, k, v):
+    """The output and scratch tensors of run_flash_attn_bwd for these shapes:
+    (dq, dk, dv, d_softmax, dq_accum, rng_state)."""
     b, sq, h, d = q.shape
-    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     sq_r, d_r = round_up(sq, 128), round_up(d, 32)
-    dsm = torch.empty((b, h, sq_r), dtype=torch.float32, device=q.device)
-    dq_accum = torch.empty((b, sq_r, h, d_r), dtype=torch.float32, device=q.device)
-    rng = torch.zeros(2, dtype=torch.int64, device=q.device)
+    return (torch.empty_like(q), torch.empty_like(k), torch.empty_like(v),
+            torch.empty((b, h, sq_r), dtype=torch.float32, device=q.device),
+            torch.empty((b, sq_r, h, d_r), dtype=torch.float32, device=q.device),
+            torch.zeros(2, dtype=torch.int64, device=q.device))
+
+
+def flash_attn_bwd(dout, q, k, v, o, lse, scale, window=(-1, -1), stream=None, out=None):
+    """run_flash_attn_bwd: tensors {dout, q, k, v, out, softmax_lse, rng_state, dq, dk, dv,
+    d_softmax, dq_accum} (flash_api.cu:656-725). -> (dq, dk, dv).
+    out: optional result of flash_attn_bwd_buffers to write into instead of allocating."""
+    L = _lib.flash_attn()
+    dq, dk, dv, dsm, dq_accum, rng = out if out is not None else flash_attn_bwd_buffers(q, k, v)
     fn = L.run_flash_attn_bwd if q.dtype == torch.float16 else L.run_flash_attn_bwd_bf16
     _call_custom(fn, [dout, q, k, v, o, lse, rng, dq, dk, dv, dsm, dq_accum],
                  pack_flash_args(q, k, v, o, scale, window), stream)
