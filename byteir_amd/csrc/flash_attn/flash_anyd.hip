@@ -1,0 +1,573 @@
+// Flash-attention forward and backward for every head dimension the reference accepts
+// (a multiple of 8 up to 256; external_libs/runtime/flash_attn/lib/flash_api.cu:163-225
+// dispatches on head_dim <= 32, 64, ... 256) other than the three that have tuned kernels
+// (32, 64, 128).
+//
+// The head dimension d is rounded up to DR (32, 64, 96, 128, 192 or 256): tiles and operand
+// fragments are DR wide, columns d..DR-1 are filled with zeros on the way in (they add nothing
+// to Q K^T or dO V^T and give zero output columns) and are not written on the way out.  The
+// structure is the plain one: one workgroup of four waves owns 128 rows (queries in forward
+// and dQ, keys in dK/dV), each wave 32 of them; the other operand streams through one LDS tile
+// of 64 rows, prefetched into registers during the math of the previous tile when DR <= 128
+// and loaded between the two barriers otherwise (the wide kernels have no registers to spare).
+// The arithmetic, the masks and the operand orientation are those of flash_fwd.hip and
+// flash_bwd.hip: S^T = K Q^T with one query per lane, P rounded to the storage type before
+// P V, exp2 with scale*log2(e) folded in, LSE = max*scale + ln(sum); backward recomputes P
+// from the forward's LSE, dS = P * (dP - D), no atomics, one launch each for D, dK/dV and dQ.
+#include "flash_common.h"
+
+namespace fa {
+namespace {
+
+constexpr int kRows = 128;  // rows per workgroup, 32 per wave
+constexpr int kTile = 64;   // rows per LDS tile
+
+// Copies a [ROWS x DR] tile (rows row0.. of a strided [n_rows, d] matrix) through registers
+// into LDS; rows >= n_rows and columns >= d arrive as zeros.  DR / 8 chunks of 16 bytes per
+// row need not divide the workgroup: the threads left over after the last whole row idle.
+template <typename T, int DR, int ROWS>
+struct AnyTileLoader {
+  static constexpr int CPR = DR / 8;
+  static constexpr int RPP = 256 / CPR;
+  static constexpr int NP = (ROWS + RPP - 1) / RPP;
+  uint4 reg[NP];
+  __device__ __forceinline__ void gload(const T *base, int64_t row_stride, int row0, int n_rows, int d) {
+    const int c = threadIdx.x % CPR, r = threadIdx.x / CPR;
+#pragma unroll
+    for (int s = 0; s < NP; ++s) {
+      const int row = row0 + s * RPP + r;
+      if (r < RPP && s * RPP + r < ROWS && row < n_rows && c * 8 < d)
+        reg[s] = *reinterpret_cast<const uint4 *>(base + (int64_t)row * row_stride + c * 8);
+      else
+        reg[s] = uint4{0, 0, 0, 0};
+    }
+  }
+  __device__ __forceinline__ void lstore(T *tile, int stride) const {
+    const int c = threadIdx.x % CPR, r = threadIdx.x / CPR;
+#pragma unroll
+    for (int s = 0; s < NP; ++s)
+      if (r < RPP && s * RPP + r < ROWS)
+        *reinterpret_cast<uint4 *>(&tile[(s * RPP + r) * stride + c * 8]) = reg[s];
+  }
+};
+
+// the 8 elements at column ks*16 + g*8 of a global row, zero beyond d or for a row that does not exist
+template <typename T>
+__device__ __forceinline__ typename Traits<T>::vec8 load_frag(const T *row, bool row_ok, int col, int d) {
+  using vec8 = typename Traits<T>::vec8;
+  if (row_ok && col < d) return *reinterpret_cast<const vec8 *>(row + col);
+  return vec8{0};
+}
+
+// 16 accumulator values of a lane -> 4 stores of 4 elements at columns db*32 + i4*8 + g*4
+template <typename T>
+__device__ __forceinline__ void store_acc(T *row, const float16v &acc, int db, int g, float mul, int d) {
+  typedef T vec4 __attribute__((ext_vector_type(4)));
+#pragma unroll
+  for (int i4 = 0; i4 < 4; ++i4) {
+    const int col = db * 32 + i4 * 8 + g * 4;
+    if (col < d) {
+      vec4 v;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) v[j] = (T)(acc[i4 * 4 + j] * mul);
+      *reinterpret_cast<vec4 *>(row + col) = v;
+    }
+  }
+}
+
+__device__ __forceinline__ void block_of(const Params &p, int n_blocks, bool reversed, int &blk, int &bh) {
+  const int L = blockIdx.x;
+  if (p.xcd_remap) {  // consecutive workgroup ids go round-robin over the 8 XCDs
+    const int xcd = L & 7, slot = L >> 3;
+    bh = (slot / n_blocks) * 8 + xcd;
+    blk = slot % n_blocks;
+  } else {
+    bh = L / n_blocks;
+    blk = L % n_blocks;
+  }
+  if (reversed) blk = n_blocks - 1 - blk;  // longest (causal) blocks first
+}
+
+// ---- forward ----------------------------------------------------------------------------------
+template <typename T, int DR>
+__global__ void __launch_bounds__(256, DR <= 128 ? 2 : 1) fwd_anyd_kernel(const Params p) {
+  using vec8 = typename Traits<T>::vec8;
+  constexpr int KS = Pad<DR>::kPlain, VS = Pad<DR>::kTr;
+  constexpr bool kPrefetch = DR <= 128;
+  __shared__ __attribute__((aligned(16))) T Ks[kTile * KS];
+  __shared__ __attribute__((aligned(16))) T Vs[kTile * VS];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r32 = lane & 31, g = lane >> 5;
+  int m_block, bh;
+  block_of(p, p.n_mblocks, true, m_block, bh);
+  const int bi = bh / p.h, hi = bh % p.h, hk = hi / (p.h / p.h_k);
+  int sk = p.sk;
+  if (p.seqlens_k) sk = min(p.sk, p.seqlens_k[bi] + p.seqlen_knew);
+  const int m0 = m_block * kRows, wq0 = m0 + wave * 32, qrow = wq0 + r32;
+
+  int lo_lim, hi_lim, w_lo_first, w_hi_first, w_lo_last, w_hi_last, b_lo, b_hi, t0, t1;
+  row_limits_sk(p, sk, qrow, lo_lim, hi_lim);
+  row_limits_sk(p, sk, wq0, w_lo_first, w_hi_first);
+  row_limits_sk(p, sk, wq0 + 31, w_lo_last, w_hi_last);
+  row_limits_sk(p, sk, m0, b_lo, t0);
+  row_limits_sk(p, sk, m0 + kRows - 1, t1, b_hi);
+  const int n_min = b_lo / kTile;
+  const int n_max = b_hi > 0 ? (b_hi + kTile - 1) / kTile : 0;
+
+  const T *qg = static_cast<const T *>(p.q) + bi * p.q_bs + (int64_t)qrow * p.q_rs + hi * p.q_hs;
+  const T *kg = static_cast<const T *>(p.k) + bi * p.k_bs + hk * p.k_hs;
+  const T *vg = static_cast<const T *>(p.v) + bi * p.v_bs + hk * p.v_hs;
+
+  vec8 qf[DR / 16];
+#pragma unroll
+  for (int ks = 0; ks < DR / 16; ++ks) qf[ks] = load_frag<T>(qg, qrow < p.sq, ks * 16 + g * 8, p.d);
+
+  AnyTileLoader<T, DR, kTile> lk, lv;
+  auto gload = [&](int t) {
+    lk.gload(kg, p.k_rs, t * kTile, sk, p.d);
+    lv.gload(vg, p.v_rs, t * kTile, sk, p.d);  // zero rows: 0 * finite stays finite in P V
+  };
+  auto lstore = [&]() { lk.lstore(Ks, KS); lv.lstore(Vs, VS); };
+
+  float16v o_acc[DR / 32];
+#pragma unroll
+  for (int i = 0; i < DR / 32; ++i) o_acc[i] = float16v{0};
+  float m_run = -INFINITY, l_run = 0.f;
+  const float c = p.scale_log2;
+
+  if (kPrefetch && n_min < n_max) {
+    gload(n_min);
+    lstore();
+    __syncthreads();
+  }
+  for (int t = n_min; t < n_max; ++t) {
+    const int kv0 = t * kTile;
+    if constexpr (kPrefetch) {
+      if (t + 1 < n_max) gload(t + 1);
+    } else {
+      gload(t);
+      lstore();
+      __syncthreads();
+    }
+    // the wave sees nothing of this tile when it lies wholly outside the widest row window
+    const bool skip = kv0 >= w_hi_last || kv0 + kTile <= w_lo_first;
+    if (!skip) {
+      float16v s[2];
+#pragma unroll
+      for (int kvb = 0; kvb < 2; ++kvb) {
+        s[kvb] = float16v{0};
+#pragma unroll
+        for (int ks = 0; ks < DR / 16; ++ks) {
+          const vec8 a = lds_read8<T>(&Ks[(kvb * 32 + r32) * KS + ks * 16 + g * 8]);
+          s[kvb] = Traits<T>::mfma(a, qf[ks], s[kvb]);
+        }
+      }
+      if (kv0 + kTile > w_hi_first || kv0 < w_lo_last) {  // a tile on the edge of the window
+#pragma unroll
+        for (int kvb = 0; kvb < 2; ++kvb)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            const int kv = kv0 + kvb * 32 + (i >> 2) * 8 + g * 4 + (i & 3);
+            if (kv >= hi_lim || kv < lo_lim) s[kvb][i] = -INFINITY;
+          }
+      }
+      float mx = -INFINITY;
+#pragma unroll
+      for (int kvb = 0; kvb < 2; ++kvb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[kvb][i]);
+      mx = fmaxf(mx, partner32(mx));
+      const float m_new = fmaxf(m_run, mx);
+      const float m_use = m_new == -INFINITY ? 0.f : m_new;
+      const float alpha = exp2_fast((m_run - m_use) * c);
+      const float m_scaled = m_use * c;
+      float rs = 0.f;
+#pragma unroll
+      for (int kvb = 0; kvb < 2; ++kvb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const float e = exp2_fast(fmaf(s[kvb][i], c, -m_scaled));
+          s[kvb][i] = e;
+          rs += e;
+        }
+      l_run = l_run * alpha + rs;
+      m_run = m_new;
+#pragma unroll
+      for (int db = 0; db < DR / 32; ++db)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o_acc[db][i] *= alpha;
+      // O^T += V^T P^T, 16 keys per step
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        float pf[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) pf[j] = s[w >> 1][(w & 1) * 8 + j];
+        const vec8 pb = pack8<T>(pf);
+#pragma unroll
+        for (int db = 0; db < DR / 32; ++db) {
+          const vec8 a = lds_read_operand_tr<T>(Vs, VS, w * 16, db * 32);
+          o_acc[db] = Traits<T>::mfma(a, pb, o_acc[db]);
+        }
+      }
+    }
+    __syncthreads();  // every wave is done with the tile in LDS
+    if constexpr (kPrefetch) {
+      if (t + 1 < n_max) lstore();
+      __syncthreads();
+    }
+  }
+
+  // epilogue: normalise, write O and LSE
+  const float l_tot = l_run + partner32(l_run);
+  const bool empty = l_tot == 0.f || l_tot != l_tot;
+  const float inv = empty ? 1.f : 1.f / l_tot;
+  if (qrow < p.sq) {
+    T *og = static_cast<T *>(p.o_w) + bi * p.o_bs + (int64_t)qrow * p.o_rs + hi * p.o_hs;
+#pragma unroll
+    for (int db = 0; db < DR / 32; ++db) store_acc<T>(og, o_acc[db], db, g, inv, p.d);
+    if (g == 0)
+      p.lse[((int64_t)bi * p.h + hi) * p.sq + qrow] =
+          empty ? INFINITY : m_run * p.scale + log2_fast(l_tot) * kLn2;
+  }
+}
+
+// ---- backward 1: D = rowsum(dO * O), half a wave per row ------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(256) dot_do_o_anyd_kernel(const Params p) {
+  const int sub = threadIdx.x & 31;
+  const int64_t row = (int64_t)blockIdx.x * 8 + (threadIdx.x >> 5);  // over b * h * sq
+  const int64_t total = (int64_t)p.b * p.h * p.sq;
+  const bool ok = row < total;
+  const int64_t rr = ok ? row : total - 1;
+  const int i = (int)(rr % p.sq);
+  const int hi = (int)((rr / p.sq) % p.h);
+  const int bi = (int)(rr / ((int64_t)p.sq * p.h));
+  const int64_t off = bi * p.o_bs + (int64_t)i * p.o_rs + hi * p.o_hs + sub * 8;
+  typedef T vec8 __attribute__((ext_vector_type(8)));
+  float s = 0.f;
+  if (sub * 8 < p.d) {
+    const vec8 a = *reinterpret_cast<const vec8 *>(static_cast<const T *>(p.dout) + off);
+    const vec8 o = *reinterpret_cast<const vec8 *>(static_cast<const T *>(p.o) + off);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) s += (float)a[j] * (float)o[j];
+  }
+#pragma unroll
+  for (int m = 16; m > 0; m >>= 1) s += __shfl_xor(s, m, 64);
+  if (ok && sub == 0) p.dsoftmax[((int64_t)bi * p.h + hi) * p.sq_rounded + i] = s;
+}
+
+// ---- backward 2: dK, dV -----------------------------------------------------------------------------
+template <typename T, int DR>
+__global__ void __launch_bounds__(256) dkdv_anyd_kernel(const Params p) {
+  using vec8 = typename Traits<T>::vec8;
+  constexpr int QS = Pad<DR>::kPlain;  // tiles are read both plainly and transposed
+  constexpr bool kPrefetch = DR <= 128;
+  __shared__ __attribute__((aligned(16))) T Qs[kTile * QS];
+  __shared__ __attribute__((aligned(16))) T dOs[kTile * QS];
+  __shared__ float lse_s[kTile];
+  __shared__ float dsm_s[kTile];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r32 = lane & 31, g = lane >> 5;
+  int n_block, bh;
+  block_of(p, p.n_nblocks, false, n_block, bh);
+  const int bi = bh / p.h, hi = bh % p.h;
+  const int kvb0 = n_block * kRows;
+  const int kvcol = kvb0 + wave * 32 + r32;  // the key this lane owns
+  const int off = p.sk - p.sq;
+
+  const T *qg = static_cast<const T *>(p.q) + bi * p.q_bs + hi * p.q_hs;
+  const T *dog = static_cast<const T *>(p.dout) + bi * p.o_bs + hi * p.o_hs;
+  const T *kg = static_cast<const T *>(p.k) + bi * p.k_bs + (int64_t)kvcol * p.k_rs + hi * p.k_hs;
+  const T *vg = static_cast<const T *>(p.v) + bi * p.v_bs + (int64_t)kvcol * p.v_rs + hi * p.v_hs;
+  const float *lse_g = p.lse + ((int64_t)bi * p.h + hi) * p.sq;
+  const float *dsm_g = p.dsoftmax + ((int64_t)bi * p.h + hi) * p.sq_rounded;
+
+  vec8 kf[DR / 16], vf[DR / 16];
+#pragma unroll
+  for (int ks = 0; ks < DR / 16; ++ks) {
+    kf[ks] = load_frag<T>(kg, kvcol < p.sk, ks * 16 + g * 8, p.d);
+    vf[ks] = load_frag<T>(vg, kvcol < p.sk, ks * 16 + g * 8, p.d);
+  }
+  float16v dk_acc[DR / 32], dv_acc[DR / 32];
+#pragma unroll
+  for (int i = 0; i < DR / 32; ++i) { dk_acc[i] = float16v{0}; dv_acc[i] = float16v{0}; }
+
+  // query tiles that can see keys [kvb0, kvb0 + 128)
+  int q_lo = 0, q_hi = p.sq;
+  if (p.wr >= 0) q_lo = max(0, kvb0 - off - p.wr);              // hi(q) = q+1+off+wr > kvb0
+  if (p.wl >= 0) q_hi = min(p.sq, kvb0 + kRows - off + p.wl);   // lo(q) = q+off-wl < kvb0+128
+  const int m_min = q_lo / kTile;
+  const int m_max = q_hi > 0 ? (q_hi + kTile - 1) / kTile : 0;
+  const float c = p.scale_log2;
+
+  AnyTileLoader<T, DR, kTile> lq, ldo;
+  float lse_r = 0.f, dsm_r = 0.f;
+  auto gload = [&](int m) {
+    lq.gload(qg, p.q_rs, m * kTile, p.sq, p.d);
+    ldo.gload(dog, p.o_rs, m * kTile, p.sq, p.d);
+    if (tid < kTile) {
+      const int q = m * kTile + tid;
+      lse_r = q < p.sq ? lse_g[q] : INFINITY;  // +inf: the row contributes P = 0
+      dsm_r = q < p.sq ? dsm_g[q] : 0.f;
+    }
+  };
+  auto lstore = [&]() {
+    lq.lstore(Qs, QS);
+    ldo.lstore(dOs, QS);
+    if (tid < kTile) { lse_s[tid] = lse_r * kLog2e; dsm_s[tid] = dsm_r; }
+  };
+
+  if (kPrefetch && m_min < m_max) {
+    gload(m_min);
+    lstore();
+    __syncthreads();
+  }
+  for (int m = m_min; m < m_max; ++m) {
+    if constexpr (kPrefetch) {
+      if (m + 1 < m_max) gload(m + 1);
+    } else {
+      gload(m);
+      lstore();
+      __syncthreads();
+    }
+#pragma unroll
+    for (int qs = 0; qs < kTile / 32; ++qs) {
+      const int q0 = m * kTile + qs * 32;  // first query row of this 32-row sub-tile
+      // wave-uniform visibility of the sub-tile against the wave's 32 keys
+      const int wkv0 = kvb0 + wave * 32;
+      int lo_first, hi_first, lo_last, hi_last;
+      row_limits(p, q0, lo_first, hi_first);
+      row_limits(p, q0 + 31, lo_last, hi_last);
+      if (wkv0 >= hi_last || wkv0 + 32 <= lo_first) continue;  // nothing kept
+      const bool need_mask = wkv0 + 32 > hi_first || wkv0 < lo_last || q0 + 32 > p.sq;
+
+      float16v s = float16v{0}, dp = float16v{0};
+#pragma unroll
+      for (int ks = 0; ks < DR / 16; ++ks) {
+        const vec8 aq = lds_read8<T>(&Qs[(qs * 32 + r32) * QS + ks * 16 + g * 8]);
+        s = Traits<T>::mfma(aq, kf[ks], s);
+        const vec8 ad = lds_read8<T>(&dOs[(qs * 32 + r32) * QS + ks * 16 + g * 8]);
+        dp = Traits<T>::mfma(ad, vf[ks], dp);
+      }
+      float pv[16], dsv[16];
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int ql = qs * 32 + (i >> 2) * 8 + g * 4 + (i & 3);  // row inside the LDS tile
+        float pe = exp2_fast(fmaf(s[i], c, -lse_s[ql]));
+        if (need_mask) {
+          int lo, hi_;
+          row_limits(p, m * kTile + ql, lo, hi_);
+          if (kvcol >= hi_ || kvcol < lo) pe = 0.f;
+        }
+        pv[i] = pe;
+        dsv[i] = pe * (dp[i] - dsm_s[ql]);
+      }
+#pragma unroll
+      for (int w = 0; w < 2; ++w) {
+        const vec8 pb = pack8<T>(&pv[w * 8]);
+        const vec8 dsb = pack8<T>(&dsv[w * 8]);
+#pragma unroll
+        for (int db = 0; db < DR / 32; ++db) {
+          const vec8 a_do = lds_read_operand_tr<T>(dOs, QS, qs * 32 + w * 16, db * 32);
+          dv_acc[db] = Traits<T>::mfma(a_do, pb, dv_acc[db]);
+          const vec8 a_q = lds_read_operand_tr<T>(Qs, QS, qs * 32 + w * 16, db * 32);
+          dk_acc[db] = Traits<T>::mfma(a_q, dsb, dk_acc[db]);
+        }
+      }
+    }
+    __syncthreads();
+    if constexpr (kPrefetch) {
+      if (m + 1 < m_max) lstore();
+      __syncthreads();
+    }
+  }
+
+  if (kvcol < p.sk) {
+    T *dkg = static_cast<T *>(p.dk) + bi * p.k_bs + (int64_t)kvcol * p.k_rs + hi * p.k_hs;
+    T *dvg = static_cast<T *>(p.dv) + bi * p.v_bs + (int64_t)kvcol * p.v_rs + hi * p.v_hs;
+#pragma unroll
+    for (int db = 0; db < DR / 32; ++db) {
+      store_acc<T>(dkg, dk_acc[db], db, g, p.scale, p.d);
+      store_acc<T>(dvg, dv_acc[db], db, g, 1.f, p.d);
+    }
+  }
+}
+
+// ---- backward 3: dQ ---------------------------------------------------------------------------------
+template <typename T, int DR>
+__global__ void __launch_bounds__(256) dq_anyd_kernel(const Params p) {
+  using vec8 = typename Traits<T>::vec8;
+  constexpr int KS = Pad<DR>::kPlain;  // K tile: plain and transposed reads
+  constexpr int VS = Pad<DR>::kPlain;  // V tile: plain reads only
+  constexpr bool kPrefetch = DR <= 128;
+  __shared__ __attribute__((aligned(16))) T Ks[kTile * KS];
+  __shared__ __attribute__((aligned(16))) T Vs[kTile * VS];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r32 = lane & 31, g = lane >> 5;
+  int m_block, bh;
+  block_of(p, p.n_mblocks, true, m_block, bh);
+  const int bi = bh / p.h, hi = bh % p.h;
+  const int m0 = m_block * kRows, wq0 = m0 + wave * 32, qrow = wq0 + r32;
+
+  int lo_lim, hi_lim, w_lo_first, w_hi_first, w_lo_last, w_hi_last, b_lo, b_hi, t0, t1;
+  row_limits(p, qrow, lo_lim, hi_lim);
+  row_limits(p, wq0, w_lo_first, w_hi_first);
+  row_limits(p, wq0 + 31, w_lo_last, w_hi_last);
+  row_limits(p, m0, b_lo, t0);
+  row_limits(p, m0 + kRows - 1, t1, b_hi);
+  const int n_min = b_lo / kTile;
+  const int n_max = b_hi > 0 ? (b_hi + kTile - 1) / kTile : 0;
+
+  const T *qg = static_cast<const T *>(p.q) + bi * p.q_bs + (int64_t)qrow * p.q_rs + hi * p.q_hs;
+  const T *dog = static_cast<const T *>(p.dout) + bi * p.o_bs + (int64_t)qrow * p.o_rs + hi * p.o_hs;
+  const T *kg = static_cast<const T *>(p.k) + bi * p.k_bs + hi * p.k_hs;
+  const T *vg = static_cast<const T *>(p.v) + bi * p.v_bs + hi * p.v_hs;
+
+  vec8 qf[DR / 16], dof[DR / 16];
+#pragma unroll
+  for (int ks = 0; ks < DR / 16; ++ks) {
+    qf[ks] = load_frag<T>(qg, qrow < p.sq, ks * 16 + g * 8, p.d);
+    dof[ks] = load_frag<T>(dog, qrow < p.sq, ks * 16 + g * 8, p.d);
+  }
+  float lse_l = INFINITY, dsm_l = 0.f;
+  if (qrow < p.sq) {
+    lse_l = p.lse[((int64_t)bi * p.h + hi) * p.sq + qrow] * kLog2e;
+    dsm_l = p.dsoftmax[((int64_t)bi * p.h + hi) * p.sq_rounded + qrow];
+  }
+  float16v dq_acc[DR / 32];
+#pragma unroll
+  for (int i = 0; i < DR / 32; ++i) dq_acc[i] = float16v{0};
+  const float c = p.scale_log2;
+
+  AnyTileLoader<T, DR, kTile> lk, lv;
+  auto gload = [&](int t) {
+    lk.gload(kg, p.k_rs, t * kTile, p.sk, p.d);
+    lv.gload(vg, p.v_rs, t * kTile, p.sk, p.d);
+  };
+  auto lstore = [&]() { lk.lstore(Ks, KS); lv.lstore(Vs, VS); };
+
+  if (kPrefetch && n_min < n_max) {
+    gload(n_min);
+    lstore();
+    __syncthreads();
+  }
+  for (int t = n_min; t < n_max; ++t) {
+    const int kv0 = t * kTile;
+    if constexpr (kPrefetch) {
+      if (t + 1 < n_max) gload(t + 1);
+    } else {
+      gload(t);
+      lstore();
+      __syncthreads();
+    }
+    const bool skip = kv0 >= w_hi_last || kv0 + kTile <= w_lo_first;
+    if (!skip) {
+      const bool need_mask = kv0 + kTile > w_hi_first || kv0 < w_lo_last;
+      float16v s[2], dp[2];
+#pragma unroll
+      for (int kvb = 0; kvb < 2; ++kvb) {
+        s[kvb] = float16v{0};
+        dp[kvb] = float16v{0};
+#pragma unroll
+        for (int ks = 0; ks < DR / 16; ++ks) {
+          const vec8 ak = lds_read8<T>(&Ks[(kvb * 32 + r32) * KS + ks * 16 + g * 8]);
+          s[kvb] = Traits<T>::mfma(ak, qf[ks], s[kvb]);
+          const vec8 av = lds_read8<T>(&Vs[(kvb * 32 + r32) * VS + ks * 16 + g * 8]);
+          dp[kvb] = Traits<T>::mfma(av, dof[ks], dp[kvb]);
+        }
+      }
+#pragma unroll
+      for (int kvb = 0; kvb < 2; ++kvb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          float pe = exp2_fast(fmaf(s[kvb][i], c, -lse_l));
+          if (need_mask) {
+            const int kv = kv0 + kvb * 32 + (i >> 2) * 8 + g * 4 + (i & 3);
+            if (kv >= hi_lim || kv < lo_lim) pe = 0.f;
+          }
+          s[kvb][i] = pe * (dp[kvb][i] - dsm_l);  // dS^T
+        }
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        float f[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) f[j] = s[w >> 1][(w & 1) * 8 + j];
+        const vec8 dsb = pack8<T>(f);
+#pragma unroll
+        for (int db = 0; db < DR / 32; ++db) {
+          const vec8 a = lds_read_operand_tr<T>(Ks, KS, w * 16, db * 32);
+          dq_acc[db] = Traits<T>::mfma(a, dsb, dq_acc[db]);
+        }
+      }
+    }
+    __syncthreads();
+    if constexpr (kPrefetch) {
+      if (t + 1 < n_max) lstore();
+      __syncthreads();
+    }
+  }
+
+  if (qrow < p.sq) {
+    T *dqg = static_cast<T *>(p.dq) + bi * p.q_bs + (int64_t)qrow * p.q_rs + hi * p.q_hs;
+#pragma unroll
+    for (int db = 0; db < DR / 32; ++db) store_acc<T>(dqg, dq_acc[db], db, g, p.scale, p.d);
+  }
+}
+
+template <typename T, int DR>
+hipError_t fwd_anyd_d(const Params &p, hipStream_t stream) {
+  fwd_anyd_kernel<T, DR><<<dim3((unsigned)(p.n_mblocks * p.b * p.h)), dim3(256), 0, stream>>>(p);
+  return hipGetLastError();
+}
+
+template <typename T, int DR>
+hipError_t bwd_anyd_d(const Params &p, hipStream_t stream) {
+  if (p.n_nblocks > 0)
+    dkdv_anyd_kernel<T, DR><<<dim3((unsigned)(p.n_nblocks * p.b * p.h)), dim3(256), 0, stream>>>(p);
+  if (p.n_mblocks > 0)
+    dq_anyd_kernel<T, DR><<<dim3((unsigned)(p.n_mblocks * p.b * p.h)), dim3(256), 0, stream>>>(p);
+  return hipGetLastError();
+}
+
+template <typename T>
+hipError_t fwd_anyd_t(const Params &p, hipStream_t stream) {
+  if (p.d <= 32) return fwd_anyd_d<T, 32>(p, stream);
+  if (p.d <= 64) return fwd_anyd_d<T, 64>(p, stream);
+  if (p.d <= 96) return fwd_anyd_d<T, 96>(p, stream);
+  if (p.d <= 128) return fwd_anyd_d<T, 128>(p, stream);
+  if (p.d <= 192) return fwd_anyd_d<T, 192>(p, stream);
+  return fwd_anyd_d<T, 256>(p, stream);
+}
+
+template <typename T>
+hipError_t bwd_anyd_t(const Params &p, hipStream_t stream) {
+  const int64_t rows = (int64_t)p.b * p.h * p.sq;
+  if (rows > 0) dot_do_o_anyd_kernel<T><<<dim3((unsigned)((rows + 7) / 8)), dim3(256), 0, stream>>>(p);
+  if (p.d <= 32) return bwd_anyd_d<T, 32>(p, stream);
+  if (p.d <= 64) return bwd_anyd_d<T, 64>(p, stream);
+  if (p.d <= 96) return bwd_anyd_d<T, 96>(p, stream);
+  if (p.d <= 128) return bwd_anyd_d<T, 128>(p, stream);
+  if (p.d <= 192) return bwd_anyd_d<T, 192>(p, stream);
+  return bwd_anyd_d<T, 256>(p, stream);
+}
+
+}  // namespace
+
+hipError_t launch_fwd_anyd(Params &p, int dtype, hipStream_t stream) {
+  if (p.d <= 0 || p.d > 256 || p.d % 8 != 0) return hipErrorInvalidValue;
+  p.n_mblocks = (p.sq + kRows - 1) / kRows;
+  if (p.n_mblocks == 0) return hipSuccess;
+  return dtype == 1 ? fwd_anyd_t<_Float16>(p, stream) : fwd_anyd_t<__bf16>(p, stream);
+}
+
+hipError_t launch_bwd_anyd(Params &p, int dtype, hipStream_t stream) {
+  if (p.d <= 0 || p.d > 256 || p.d % 8 != 0) return hipErrorInvalidValue;
+  p.n_mblocks = (p.sq + kRows - 1) / kRows;
+  p.n_nblocks = (p.sk + kRows - 1) / kRows;
+  return dtype == 1 ? bwd_anyd_t<_Float16>(p, stream) : bwd_anyd_t<__bf16>(p, stream);
+}
+
+}  // namespace fa

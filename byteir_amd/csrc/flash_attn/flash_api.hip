@@ -67,8 +67,8 @@ int fill(const Blob &a, fa::Params &p) {
   if (a.b < 0 || a.h <= 0 || a.h_k <= 0 || a.seqlen_q < 0 || a.seqlen_k < 0)
     return fail("negative or zero dimension (b=%ld h=%ld h_k=%ld sq=%ld sk=%ld)", (long)a.b,
                 (long)a.h, (long)a.h_k, (long)a.seqlen_q, (long)a.seqlen_k);
-  if (a.d != 32 && a.d != 64 && a.d != 128)
-    return fail("head_dim %ld is not supported (32, 64 or 128)", (long)a.d);
+  if (a.d <= 0 || a.d > 256 || a.d % 8 != 0)
+    return fail("head_dim %ld is not supported (a multiple of 8 up to 256)", (long)a.d);
   if (a.h % a.h_k != 0) return fail("h (%ld) must be a multiple of h_k (%ld)", (long)a.h, (long)a.h_k);
   if (a.p_dropout != 0.f) return fail("p_dropout %g is not supported (0 only)", a.p_dropout);
   const int64_t strides[] = {a.q_bs, a.k_bs, a.v_bs, a.o_bs, a.q_rs, a.k_rs,

@@ -96,10 +96,10 @@ __device__ __forceinline__ typename Traits<T>::vec8 lds_read_operand_tr(const T 
 
 // LDS row strides (elements).  Rows read with plain 128-bit loads (32 rows x 16 B at a time)
 // want a stride of 4*odd banks; rows read with the transposing load (4 rows x 64 B per
-// half-wave) want a stride of 16 (mod 64) banks.
+// half-wave) want a stride of 16 (mod 32) banks.
 template <int D> struct Pad {
   static constexpr int kPlain = D + 8;
-  static constexpr int kTr = D == 32 ? 32 : D + 32;
+  static constexpr int kTr = D % 64 == 32 ? D : D + 32;
 };
 
 struct Params {
@@ -136,5 +136,10 @@ __device__ __forceinline__ void row_limits_sk(const Params &p, int sk, int q, in
 __device__ __forceinline__ void row_limits(const Params &p, int q, int &lo, int &hi) {
   row_limits_sk(p, p.sk, q, lo, hi);
 }
+
+// Kernels for the head dimensions without a tuned instantiation (flash_anyd.hip); the callers
+// have set everything in `p` but the block counts.
+hipError_t launch_fwd_anyd(Params &p, int dtype, hipStream_t stream);
+hipError_t launch_bwd_anyd(Params &p, int dtype, hipStream_t stream);
 
 }  // namespace fa

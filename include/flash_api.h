@@ -23,7 +23,8 @@
  * Tensors are [batch, seqlen, heads, head_dim] with a contiguous head_dim; softmax_lse is
  * [batch, heads, seqlen_q] float.
  *
- * Supported here: head_dim 32, 64 or 128, p_dropout == 0, any seqlen, h % h_k == 0
+ * Supported here: head_dim a multiple of 8 up to 256 (the reference's range; 32, 64 and 128
+ * have tuned kernels), p_dropout == 0, any seqlen, h % h_k == 0
  * (backward: h == h_k).  Anything else is reported on stderr and the process aborts, since
  * the ABI has no error channel; the *_checked variants return an error code instead.
  */

@@ -74,6 +74,21 @@ CASES = [
     (1, 300, 300, 2, 2, 64, (64, 0)),      # sliding window, left-bounded causal
     (1, 300, 260, 2, 2, 128, (40, 30)),    # local window both sides
     (3, 1, 50, 1, 1, 32, (-1, -1)),        # single query row
+    # head dimensions without a tuned kernel: every multiple of 8 up to 256 is accepted
+    (1, 150, 150, 2, 2, 8, (-1, 0)),
+    (1, 1, 40, 2, 2, 16, (-1, -1)),
+    (1, 40, 40, 1, 1, 24, (-1, 0)),
+    (1, 129, 65, 1, 1, 40, (-1, -1)),
+    (1, 96, 96, 2, 2, 48, (-1, 0)),
+    (1, 200, 200, 2, 2, 72, (30, 0)),
+    (1, 130, 190, 2, 2, 96, (-1, 0)),
+    (2, 100, 100, 2, 1, 96, (-1, -1)),     # grouped-query heads (forward only)
+    (1, 64, 64, 1, 1, 104, (-1, -1)),
+    (1, 140, 260, 2, 2, 160, (-1, 0)),
+    (1, 257, 129, 1, 1, 192, (-1, -1)),
+    (1, 131, 131, 2, 2, 224, (-1, 0)),
+    (2, 128, 192, 2, 2, 256, (-1, 0)),
+    (1, 70, 300, 1, 1, 256, (20, 10)),
 ]
 
 
@@ -135,7 +150,7 @@ def test_unsupported_arguments_are_reported_not_run():
     L = _lib.flash_attn()
     L.flash_attn_fwd_checked.argtypes = [ctypes.POINTER(ctypes.c_void_p), ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p]
     L.flash_attn_last_error.restype = ctypes.c_char_p
-    q = torch.zeros((1, 16, 1, 48), dtype=torch.float16, device="cuda")  # head_dim 48
+    q = torch.zeros((1, 16, 1, 264), dtype=torch.float16, device="cuda")  # head_dim 264 > 256
     blob = ops.pack_flash_args(q, q, q, q, 1.0, (-1, -1))
     arr = (ctypes.c_void_p * 7)(*[q.data_ptr()] * 7)
     buf = ctypes.create_string_buffer(blob, len(blob))
@@ -240,6 +255,9 @@ KV_CASES = [
     (4, 16, 2, 2, 32, 1024, 16, [1000, 3, 500, 64], (-1, 0), True),
     (2, 3, 4, 4, 64, 130, 0, [130, 1], (-1, -1), False),        # no append: read-only cache
     (2, 2, 4, 1, 64, 520, 2, [518, 300], (64, 0), True),        # sliding window, MQA
+    (2, 3, 4, 2, 96, 260, 3, [250, 17], (-1, 0), True),         # head dimensions without a tuned kernel
+    (1, 1, 2, 2, 256, 300, 1, [299], (-1, -1), True),
+    (2, 4, 2, 2, 80, 128, 0, [128, 5], (-1, -1), False),
 ]
 
 
