@@ -14,6 +14,12 @@
 // flash_bwd.hip: S^T = K Q^T with one query per lane, P rounded to the storage type before
 // P V, exp2 with scale*log2(e) folded in, LSE = max*scale + ln(sum); backward recomputes P
 // from the forward's LSE, dS = P * (dP - D), no atomics, one launch each for D, dK/dV and dQ.
+//
+// These kernels also carry dropout for every head dimension (the tuned kernels do not): the
+// keep-mask is the reference's function of (seed, offset, batch, head, row, column)
+// (lib/dropout.h, lib/philox.cuh), evaluated here for the elements a lane holds in the MFMA
+// accumulator layout; the scalings follow the reference (forward: row sums of the undropped P,
+// O / p_keep; backward: D * p_keep, dS = P * (keep ? dP - D : -D), dQ and dK / p_keep, dV / p_keep).
 #include "flash_common.h"
 
 namespace fa {
@@ -75,6 +81,73 @@ __device__ __forceinline__ void store_acc(T *row, const float16v &acc, int db, i
   }
 }
 
+// Philox4x32 with 7 rounds (lib/philox.cuh:22-52): key = seed, counter = (offset, subsequence).
+__device__ __forceinline__ uint4 philox7(uint32_t k0, uint32_t k1, uint64_t offset, uint32_t sub_lo, uint32_t sub_hi) {
+  uint32_t c0 = (uint32_t)offset, c1 = (uint32_t)(offset >> 32), c2 = sub_lo, c3 = sub_hi;
+#pragma unroll
+  for (int r = 0; r < 7; ++r) {
+    if (r > 0) { k0 += 0x9E3779B9u; k1 += 0xBB67AE85u; }
+    const uint32_t hi0 = __umulhi(0xD2511F53u, c0), lo0 = 0xD2511F53u * c0;
+    const uint32_t hi1 = __umulhi(0xCD9E8D57u, c2), lo1 = 0xCD9E8D57u * c2;
+    const uint32_t n0 = hi1 ^ c1 ^ k0, n2 = hi0 ^ c3 ^ k1;
+    c0 = n0; c1 = lo1; c2 = n2; c3 = lo0;
+  }
+  return uint4{c0, c1, c2, c3};
+}
+
+// The reference draws one Philox value per (16-row x 32-column block of the attention matrix,
+// lane of a 32-lane warp): 16 bytes, one per element that lane holds in the m16n8 accumulator
+// layout: row = lane/4 (+8), column = 8*tile + 2*(lane%4) (+1) for four 8-column tiles, byte =
+// 4*tile + 2*(row half) + (column & 1); subsequence = (row block, column block), offset =
+// rng_state[1] + (batch*heads + head)*32 + lane; an element is kept iff its byte <= threshold
+// (lib/dropout.h:19-23,38-84; call sites flash_fwd_kernel.h:321-334, flash_bwd_kernel.h:524-533).
+struct DropCtx {
+  uint32_t k0, k1;
+  uint64_t off;   // rng_state[1] + (batch*heads + head)*32
+  uint32_t thr;
+  __device__ __forceinline__ void init(const Params &p, int bh) {
+    const uint64_t seed = p.rng_state[0];
+    k0 = (uint32_t)seed; k1 = (uint32_t)(seed >> 32);
+    off = p.rng_state[1] + (uint64_t)(bh * 32);
+    thr = p.keep_thr;
+  }
+  // Scores held with the query on the lane (column of S^T): bit i of the result is set when
+  // key kv32 + 8*(i/4) + 4*g + i%4 is kept for query q; kv32 is a multiple of 32.
+  __device__ __forceinline__ uint32_t keep_q_on_lane(int q, int kv32, int g) const {
+    uint32_t m = 0;
+    const int sh = ((q >> 3) & 1) * 16;
+#pragma unroll
+    for (int c2 = 0; c2 < 2; ++c2) {
+      const uint4 r = philox7(k0, k1, off + (uint32_t)((q & 7) * 4 + g * 2 + c2), (uint32_t)(q >> 4), (uint32_t)(kv32 >> 5));
+      const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int e = 0; e < 2; ++e)
+          if (((w[t] >> (sh + 8 * e)) & 0xffu) <= thr) m |= 1u << (t * 4 + c2 * 2 + e);
+    }
+    return m;
+  }
+  // Scores held with the key on the lane (column of S): bit i is set when query
+  // q32 + 8*(i/4) + 4*g + i%4 is kept for key kv; q32 is a multiple of 32.
+  __device__ __forceinline__ uint32_t keep_k_on_lane(int q32, int kv, int g) const {
+    uint32_t m = 0;
+    const int tile = (kv & 31) >> 3, e = kv & 1;
+#pragma unroll
+    for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+      for (int c4 = 0; c4 < 4; ++c4) {
+        const uint4 r = philox7(k0, k1, off + (uint32_t)((g * 4 + c4) * 4 + ((kv & 7) >> 1)),
+                                (uint32_t)((q32 >> 4) + rb), (uint32_t)(kv >> 5));
+        const uint32_t w = tile == 0 ? r.x : tile == 1 ? r.y : tile == 2 ? r.z : r.w;
+#pragma unroll
+        for (int rh = 0; rh < 2; ++rh)
+          if (((w >> (8 * (2 * rh + e))) & 0xffu) <= thr) m |= 1u << (rb * 8 + rh * 4 + c4);
+      }
+    return m;
+  }
+};
+
 __device__ __forceinline__ void block_of(const Params &p, int n_blocks, bool reversed, int &blk, int &bh) {
   const int L = blockIdx.x;
   if (p.xcd_remap) {  // consecutive workgroup ids go round-robin over the 8 XCDs
@@ -89,7 +162,7 @@ __device__ __forceinline__ void block_of(const Params &p, int n_blocks, bool rev
 }
 
 // ---- forward ----------------------------------------------------------------------------------
-template <typename T, int DR>
+template <typename T, int DR, bool Drop>
 __global__ void __launch_bounds__(256, DR <= 128 ? 2 : 1) fwd_anyd_kernel(const Params p) {
   using vec8 = typename Traits<T>::vec8;
   constexpr int KS = Pad<DR>::kPlain, VS = Pad<DR>::kTr;
@@ -135,6 +208,8 @@ __global__ void __launch_bounds__(256, DR <= 128 ? 2 : 1) fwd_anyd_kernel(const 
   for (int i = 0; i < DR / 32; ++i) o_acc[i] = float16v{0};
   float m_run = -INFINITY, l_run = 0.f;
   const float c = p.scale_log2;
+  DropCtx drop;
+  if constexpr (Drop) drop.init(p, bh);
 
   if (kPrefetch && n_min < n_max) {
     gload(n_min);
@@ -193,6 +268,15 @@ __global__ void __launch_bounds__(256, DR <= 128 ? 2 : 1) fwd_anyd_kernel(const 
         }
       l_run = l_run * alpha + rs;
       m_run = m_new;
+      if constexpr (Drop) {  // the row sum above is that of the undropped P
+#pragma unroll
+        for (int kvb = 0; kvb < 2; ++kvb) {
+          const uint32_t keep = drop.keep_q_on_lane(qrow, kv0 + kvb * 32, g);
+#pragma unroll
+          for (int i = 0; i < 16; ++i)
+            if (!((keep >> i) & 1u)) s[kvb][i] = 0.f;
+        }
+      }
 #pragma unroll
       for (int db = 0; db < DR / 32; ++db)
 #pragma unroll
@@ -221,7 +305,8 @@ __global__ void __launch_bounds__(256, DR <= 128 ? 2 : 1) fwd_anyd_kernel(const 
   // epilogue: normalise, write O and LSE
   const float l_tot = l_run + partner32(l_run);
   const bool empty = l_tot == 0.f || l_tot != l_tot;
-  const float inv = empty ? 1.f : 1.f / l_tot;
+  float inv = empty ? 1.f : 1.f / l_tot;
+  if constexpr (Drop) inv *= p.rp_keep;
   if (qrow < p.sq) {
     T *og = static_cast<T *>(p.o_w) + bi * p.o_bs + (int64_t)qrow * p.o_rs + hi * p.o_hs;
 #pragma unroll
@@ -254,11 +339,12 @@ __global__ void __launch_bounds__(256) dot_do_o_anyd_kernel(const Params p) {
   }
 #pragma unroll
   for (int m = 16; m > 0; m >>= 1) s += __shfl_xor(s, m, 64);
+  if (p.drop) s *= p.p_keep;  // flash_bwd_preprocess_kernel.h:124-128
   if (ok && sub == 0) p.dsoftmax[((int64_t)bi * p.h + hi) * p.sq_rounded + i] = s;
 }
 
 // ---- backward 2: dK, dV -----------------------------------------------------------------------------
-template <typename T, int DR>
+template <typename T, int DR, bool Drop>
 __global__ void __launch_bounds__(256) dkdv_anyd_kernel(const Params p) {
   using vec8 = typename Traits<T>::vec8;
   constexpr int QS = Pad<DR>::kPlain;  // tiles are read both plainly and transposed
@@ -301,6 +387,8 @@ __global__ void __launch_bounds__(256) dkdv_anyd_kernel(const Params p) {
   const int m_min = q_lo / kTile;
   const int m_max = q_hi > 0 ? (q_hi + kTile - 1) / kTile : 0;
   const float c = p.scale_log2;
+  DropCtx drop;
+  if constexpr (Drop) drop.init(p, bh);
 
   AnyTileLoader<T, DR, kTile> lq, ldo;
   float lse_r = 0.f, dsm_r = 0.f;
@@ -352,6 +440,8 @@ __global__ void __launch_bounds__(256) dkdv_anyd_kernel(const Params p) {
         dp = Traits<T>::mfma(ad, vf[ks], dp);
       }
       float pv[16], dsv[16];
+      uint32_t keep = 0xffffu;
+      if constexpr (Drop) keep = drop.keep_k_on_lane(q0, kvcol, g);
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         const int ql = qs * 32 + (i >> 2) * 8 + g * 4 + (i & 3);  // row inside the LDS tile
@@ -361,8 +451,9 @@ __global__ void __launch_bounds__(256) dkdv_anyd_kernel(const Params p) {
           row_limits(p, m * kTile + ql, lo, hi_);
           if (kvcol >= hi_ || kvcol < lo) pe = 0.f;
         }
-        pv[i] = pe;
-        dsv[i] = pe * (dp[i] - dsm_s[ql]);
+        const bool kept = !Drop || ((keep >> i) & 1u);
+        pv[i] = kept ? pe : 0.f;
+        dsv[i] = pe * ((kept ? dp[i] : 0.f) - dsm_s[ql]);
       }
 #pragma unroll
       for (int w = 0; w < 2; ++w) {
@@ -389,14 +480,14 @@ __global__ void __launch_bounds__(256) dkdv_anyd_kernel(const Params p) {
     T *dvg = static_cast<T *>(p.dv) + bi * p.v_bs + (int64_t)kvcol * p.v_rs + hi * p.v_hs;
 #pragma unroll
     for (int db = 0; db < DR / 32; ++db) {
-      store_acc<T>(dkg, dk_acc[db], db, g, p.scale, p.d);
-      store_acc<T>(dvg, dv_acc[db], db, g, 1.f, p.d);
+      store_acc<T>(dkg, dk_acc[db], db, g, Drop ? p.scale * p.rp_keep : p.scale, p.d);
+      store_acc<T>(dvg, dv_acc[db], db, g, Drop ? p.rp_keep : 1.f, p.d);
     }
   }
 }
 
 // ---- backward 3: dQ ---------------------------------------------------------------------------------
-template <typename T, int DR>
+template <typename T, int DR, bool Drop>
 __global__ void __launch_bounds__(256) dq_anyd_kernel(const Params p) {
   using vec8 = typename Traits<T>::vec8;
   constexpr int KS = Pad<DR>::kPlain;  // K tile: plain and transposed reads
@@ -441,6 +532,8 @@ __global__ void __launch_bounds__(256) dq_anyd_kernel(const Params p) {
 #pragma unroll
   for (int i = 0; i < DR / 32; ++i) dq_acc[i] = float16v{0};
   const float c = p.scale_log2;
+  DropCtx drop;
+  if constexpr (Drop) drop.init(p, bh);
 
   AnyTileLoader<T, DR, kTile> lk, lv;
   auto gload = [&](int t) {
@@ -480,7 +573,9 @@ __global__ void __launch_bounds__(256) dq_anyd_kernel(const Params p) {
         }
       }
 #pragma unroll
-      for (int kvb = 0; kvb < 2; ++kvb)
+      for (int kvb = 0; kvb < 2; ++kvb) {
+        uint32_t keep = 0xffffu;
+        if constexpr (Drop) keep = drop.keep_q_on_lane(qrow, kv0 + kvb * 32, g);
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
           float pe = exp2_fast(fmaf(s[kvb][i], c, -lse_l));
@@ -488,8 +583,10 @@ __global__ void __launch_bounds__(256) dq_anyd_kernel(const Params p) {
             const int kv = kv0 + kvb * 32 + (i >> 2) * 8 + g * 4 + (i & 3);
             if (kv >= hi_lim || kv < lo_lim) pe = 0.f;
           }
-          s[kvb][i] = pe * (dp[kvb][i] - dsm_l);  // dS^T
+          const bool kept = !Drop || ((keep >> i) & 1u);
+          s[kvb][i] = pe * ((kept ? dp[kvb][i] : 0.f) - dsm_l);  // dS^T
         }
+      }
 #pragma unroll
       for (int w = 0; w < 4; ++w) {
         float f[8];
@@ -513,22 +610,30 @@ __global__ void __launch_bounds__(256) dq_anyd_kernel(const Params p) {
   if (qrow < p.sq) {
     T *dqg = static_cast<T *>(p.dq) + bi * p.q_bs + (int64_t)qrow * p.q_rs + hi * p.q_hs;
 #pragma unroll
-    for (int db = 0; db < DR / 32; ++db) store_acc<T>(dqg, dq_acc[db], db, g, p.scale, p.d);
+    for (int db = 0; db < DR / 32; ++db)
+      store_acc<T>(dqg, dq_acc[db], db, g, Drop ? p.scale * p.rp_keep : p.scale, p.d);
   }
 }
 
 template <typename T, int DR>
 hipError_t fwd_anyd_d(const Params &p, hipStream_t stream) {
-  fwd_anyd_kernel<T, DR><<<dim3((unsigned)(p.n_mblocks * p.b * p.h)), dim3(256), 0, stream>>>(p);
+  const dim3 grid((unsigned)(p.n_mblocks * p.b * p.h)), block(256);
+  if (p.drop) fwd_anyd_kernel<T, DR, true><<<grid, block, 0, stream>>>(p);
+  else fwd_anyd_kernel<T, DR, false><<<grid, block, 0, stream>>>(p);
   return hipGetLastError();
 }
 
 template <typename T, int DR>
 hipError_t bwd_anyd_d(const Params &p, hipStream_t stream) {
-  if (p.n_nblocks > 0)
-    dkdv_anyd_kernel<T, DR><<<dim3((unsigned)(p.n_nblocks * p.b * p.h)), dim3(256), 0, stream>>>(p);
-  if (p.n_mblocks > 0)
-    dq_anyd_kernel<T, DR><<<dim3((unsigned)(p.n_mblocks * p.b * p.h)), dim3(256), 0, stream>>>(p);
+  const dim3 gk((unsigned)(p.n_nblocks * p.b * p.h)), gq((unsigned)(p.n_mblocks * p.b * p.h)), block(256);
+  if (p.n_nblocks > 0) {
+    if (p.drop) dkdv_anyd_kernel<T, DR, true><<<gk, block, 0, stream>>>(p);
+    else dkdv_anyd_kernel<T, DR, false><<<gk, block, 0, stream>>>(p);
+  }
+  if (p.n_mblocks > 0) {
+    if (p.drop) dq_anyd_kernel<T, DR, true><<<gq, block, 0, stream>>>(p);
+    else dq_anyd_kernel<T, DR, false><<<gq, block, 0, stream>>>(p);
+  }
   return hipGetLastError();
 }
 

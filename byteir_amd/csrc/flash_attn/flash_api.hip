@@ -70,7 +70,7 @@ int fill(const Blob &a, fa::Params &p) {
   if (a.d <= 0 || a.d > 256 || a.d % 8 != 0)
     return fail("head_dim %ld is not supported (a multiple of 8 up to 256)", (long)a.d);
   if (a.h % a.h_k != 0) return fail("h (%ld) must be a multiple of h_k (%ld)", (long)a.h, (long)a.h_k);
-  if (a.p_dropout != 0.f) return fail("p_dropout %g is not supported (0 only)", a.p_dropout);
+  if (!(a.p_dropout >= 0.f && a.p_dropout < 1.f)) return fail("p_dropout %g is outside [0, 1)", a.p_dropout);
   const int64_t strides[] = {a.q_bs, a.k_bs, a.v_bs, a.o_bs, a.q_rs, a.k_rs,
                              a.v_rs, a.o_rs, a.q_hs, a.k_hs, a.v_hs, a.o_hs};
   for (int64_t s : strides)
@@ -89,6 +89,11 @@ int fill(const Blob &a, fa::Params &p) {
   // "unbounded" (< 0) is the same thing
   p.wl = a.window_size_left < 0 ? -1 : (int)a.window_size_left;
   p.wr = a.window_size_right < 0 ? -1 : (int)a.window_size_right;
+  // flash_api.cu:291-294
+  p.p_keep = 1.f - a.p_dropout;
+  p.keep_thr = (unsigned)(uint8_t)std::floor(p.p_keep * 255.0);
+  p.rp_keep = 1.f / p.p_keep;
+  p.drop = a.p_dropout > 0.f ? 1 : 0;
   return 0;
 }
 
@@ -137,9 +142,11 @@ int flash_attn_fwd_checked(void **tensors, const void *extra_args, int dtype, vo
   if (int r = fill(a, p)) return r;
   // tensors: q, k, v, rng_state, o, softmax_lse, softmax_P
   p.q = tensors[0]; p.k = tensors[1]; p.v = tensors[2];
+  p.rng_state = static_cast<const uint64_t *>(tensors[3]);
   p.o_w = tensors[4];
   p.lse = static_cast<float *>(tensors[5]);
   if (p.b == 0 || p.sq == 0) return 0;
+  if (p.drop && !p.rng_state) return fail("p_dropout > 0 needs the rng_state tensor {seed, offset}");
   if (!p.q || !p.o_w || !p.lse || (p.sk > 0 && (!p.k || !p.v))) return fail("null tensor pointer");
   if (!aligned16(p.q) || !aligned16(p.k) || !aligned16(p.v) || !aligned16(p.o_w))
     return fail("q, k, v and o must be 16-byte aligned");
@@ -157,9 +164,11 @@ int flash_attn_bwd_checked(void **tensors, const void *extra_args, int dtype, vo
   // tensors: dout, q, k, v, out, softmax_lse, rng_state, dq, dk, dv, d_softmax, dq_accum
   p.dout = tensors[0]; p.q = tensors[1]; p.k = tensors[2]; p.v = tensors[3]; p.o = tensors[4];
   p.lse = static_cast<float *>(tensors[5]);
+  p.rng_state = static_cast<const uint64_t *>(tensors[6]);
   p.dq = tensors[7]; p.dk = tensors[8]; p.dv = tensors[9];
   p.dsoftmax = static_cast<float *>(tensors[10]);
   if (p.b == 0) return 0;
+  if (p.drop && !p.rng_state) return fail("p_dropout > 0 needs the rng_state tensor {seed, offset}");
   const void *need[] = {p.dout, p.q, p.k, p.v, p.o, p.dq, p.dk, p.dv};
   for (const void *t : need) {
     if (!t) return fail("null tensor pointer");

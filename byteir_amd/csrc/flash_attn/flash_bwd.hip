@@ -599,7 +599,7 @@ hipError_t launch_bwd(Params &p, int dtype, hipStream_t stream) {
   p.n_nblocks = (p.sk + kKvBlock - 1) / kKvBlock;
   p.xcd_remap = ((p.b * p.h) % 8 == 0) ? 1 : 0;
   if (p.b * p.h == 0) return hipSuccess;
-  if (p.d != 32 && p.d != 64 && p.d != 128) return launch_bwd_anyd(p, dtype, stream);
+  if (p.drop || (p.d != 32 && p.d != 64 && p.d != 128)) return launch_bwd_anyd(p, dtype, stream);
   return dtype == 1 ? launch_bwd_t<_Float16>(p, stream) : launch_bwd_t<__bf16>(p, stream);
 }
 

@@ -123,6 +123,12 @@ struct Params {
   int seqlen_knew;
   const void *k_new, *v_new;
   int64_t knew_bs, vnew_bs, knew_rs, vnew_rs, knew_hs, vnew_hs;
+  // dropout (forward and backward calls): rng_state = {seed, offset} in device memory,
+  // keep probability, its reciprocal and its 8-bit threshold floor(p_keep * 255)
+  const uint64_t *rng_state;
+  float p_keep, rp_keep;
+  unsigned keep_thr;
+  int drop;                           // 1: p_dropout > 0
 };
 
 // Kept key range [lo, hi) for query row `q` when the sequence has `sk` keys

@@ -121,10 +121,18 @@ def _call_custom(fn, tensors, blob, stream):
     fn(arr, ctypes.cast(buf, ctypes.c_void_p), _stream(stream))
 
 
-def flash_attn_fwd(q, k, v, scale, window=(-1, -1), stream=None, out=None):
+def rng_state_tensor(seed, offset, device):
+    """The rng_state operand of the attention calls: {seed, offset} as two 64-bit words."""
+    to_i64 = lambda x: int(x) - (1 << 64) if int(x) >= (1 << 63) else int(x)
+    return torch.tensor([to_i64(seed), to_i64(offset)], dtype=torch.int64, device=device)
+
+
+def flash_attn_fwd(q, k, v, scale, window=(-1, -1), stream=None, out=None, p_dropout=0.0, rng_state=None):
     """run_flash_attn_fwd: tensors {q, k, v, rng_state, o, softmax_lse, softmax_P}
     (external_libs/runtime/flash_attn/lib/flash_api.cu:586-654). -> (o, lse[b,h,sq] f32).
-    out: optional (o, lse, rng_state) to write into instead of allocating."""
+    out: optional (o, lse, rng_state) to write into instead of allocating.
+    p_dropout > 0 reads {seed, offset} from rng_state (an int64[2] device tensor, see
+    rng_state_tensor), as the reference's kernel does (flash_fwd_kernel.h:46-47)."""
     L = _lib.flash_attn()
     b, sq, h, d = q.shape
     if out is not None:
@@ -132,9 +140,9 @@ def flash_attn_fwd(q, k, v, scale, window=(-1, -1), stream=None, out=None):
     else:
         o = torch.empty_like(q)
         lse = torch.empty((b, h, sq), dtype=torch.float32, device=q.device)
-        rng = torch.zeros(2, dtype=torch.int64, device=q.device)
+        rng = rng_state if rng_state is not None else torch.zeros(2, dtype=torch.int64, device=q.device)
     fn = L.run_flash_attn_fwd if q.dtype == torch.float16 else L.run_flash_attn_fwd_bf16
-    _call_custom(fn, [q, k, v, rng, o, lse, None], pack_flash_args(q, k, v, o, scale, window), stream)
+    _call_custom(fn, [q, k, v, rng, o, lse, None], pack_flash_args(q, k, v, o, scale, window, p_dropout), stream)
     return o, lse
 
 
@@ -149,15 +157,19 @@ def flash_attn_bwd_buffers(q, k, v):
             torch.zeros(2, dtype=torch.int64, device=q.device))
 
 
-def flash_attn_bwd(dout, q, k, v, o, lse, scale, window=(-1, -1), stream=None, out=None):
+def flash_attn_bwd(dout, q, k, v, o, lse, scale, window=(-1, -1), stream=None, out=None, p_dropout=0.0,
+                   rng_state=None):
     """run_flash_attn_bwd: tensors {dout, q, k, v, out, softmax_lse, rng_state, dq, dk, dv,
     d_softmax, dq_accum} (flash_api.cu:656-725). -> (dq, dk, dv).
-    out: optional result of flash_attn_bwd_buffers to write into instead of allocating."""
+    out: optional result of flash_attn_bwd_buffers to write into instead of allocating.
+    p_dropout > 0 needs the rng_state the forward call used."""
     L = _lib.flash_attn()
     dq, dk, dv, dsm, dq_accum, rng = out if out is not None else flash_attn_bwd_buffers(q, k, v)
+    if rng_state is not None:
+        rng = rng_state
     fn = L.run_flash_attn_bwd if q.dtype == torch.float16 else L.run_flash_attn_bwd_bf16
     _call_custom(fn, [dout, q, k, v, o, lse, rng, dq, dk, dv, dsm, dq_accum],
-                 pack_flash_args(q, k, v, o, scale, window), stream)
+                 pack_flash_args(q, k, v, o, scale, window, p_dropout), stream)
     return dq, dk, dv
 
 

@@ -24,7 +24,7 @@
  * [batch, heads, seqlen_q] float.
  *
  * Supported here: head_dim a multiple of 8 up to 256 (the reference's range; 32, 64 and 128
- * have tuned kernels), p_dropout == 0, any seqlen, h % h_k == 0
+ * have tuned kernels), 0 <= p_dropout < 1, any seqlen, h % h_k == 0
  * (backward: h == h_k).  Anything else is reported on stderr and the process aborts, since
  * the ABI has no error channel; the *_checked variants return an error code instead.
  */
@@ -39,12 +39,16 @@ extern "C" {
 extern const char *VERSION;
 
 /* tensors: {q, k, v, rng_state, o, softmax_lse, softmax_P}  (flash_api.cu:626-654).
- * fp16 storage.  rng_state and softmax_P are accepted and never touched (p_dropout == 0). */
+ * fp16 storage.  rng_state is two 64-bit words {seed, offset} in device memory, read by the
+ * kernel when p_dropout > 0 as in the reference (flash_fwd_kernel.h:46-47; the caller fills
+ * it) and not touched otherwise; the keep-mask is the reference's function of (seed, offset,
+ * batch, head, row, column) (lib/dropout.h, lib/philox.cuh).  softmax_P is never touched. */
 void run_flash_attn_fwd(void **tensors, void *extra_args, void *stream);
 
 /* tensors: {dout, q, k, v, out, softmax_lse, rng_state, dq, dk, dv, d_softmax, dq_accum}
  * (flash_api.cu:696-725).  fp16 storage.  d_softmax is [b, h, seqlen_q_rounded] float scratch
- * that receives rowsum(dout * out); dq_accum is accepted and left untouched (dQ is
+ * that receives rowsum(dout * out) (times 1 - p_dropout, as in the reference); rng_state must
+ * hold what the forward call used; dq_accum is accepted and left untouched (dQ is
  * accumulated without atomics by a pass that is parallel over query blocks). */
 void run_flash_attn_bwd(void **tensors, void *extra_args, void *stream);
 

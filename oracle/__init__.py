@@ -81,6 +81,11 @@ def lib():
         L.oracle_fa_unpack_args.restype = ctypes.c_size_t
         L.oracle_flash_fwd.argtypes = [ctypes.POINTER(FaArgs), i32, i32, vp, vp, vp, vp, vp, vp]
         L.oracle_flash_bwd.argtypes = [ctypes.POINTER(FaArgs), i32, i32] + [vp] * 10
+        L.oracle_flash_fwd_rng.argtypes = [ctypes.POINTER(FaArgs), i32, i32] + [vp] * 7
+        L.oracle_flash_bwd_rng.argtypes = [ctypes.POINTER(FaArgs), i32, i32] + [vp] * 11
+        L.oracle_philox4x32.argtypes = [u64, u64, u64, i32, vp]
+        L.oracle_dropout_keep.argtypes = [vp, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_uint8]
+        L.oracle_dropout_keep.restype = i32
         _lib = L
     return _lib
 
@@ -243,33 +248,64 @@ def fa_unpack_args(blob):
     return a
 
 
-def flash_fwd(q, k, v, scale, window=(-1, -1), round_p=True):
-    """q [b,sq,h,d], k/v [b,sk,h_k,d] in one storage dtype.
+def philox4x32(seed, subsequence, offset, rounds=7):
+    """-> the 4 output words (uint32) of Philox4x32-`rounds` with key = seed and
+    counter = (offset, subsequence)."""
+    out = np.zeros(4, dtype=np.uint32)
+    lib().oracle_philox4x32(int(seed), int(subsequence), int(offset), int(rounds), _p(out))
+    return out
+
+
+def dropout_threshold(p_dropout):
+    """floor(p_keep * 255) with p_keep = 1 - p_dropout in float32 (flash_api.cu:291-292)."""
+    return int(np.floor(np.float64(np.float32(1.0) - np.float32(p_dropout)) * 255.0))
+
+
+def dropout_keep_mask(rng_state, b, h, sq, sk, p_dropout):
+    """-> bool [b, h, sq, sk]: which attention entries survive dropout for rng_state = (seed, offset)."""
+    rs = np.asarray(rng_state, dtype=np.uint64)
+    thr = dropout_threshold(p_dropout)
+    m = np.empty((b, h, sq, sk), dtype=bool)
+    L = lib()
+    for bi in range(b):
+        for hi in range(h):
+            for i in range(sq):
+                for j in range(sk):
+                    m[bi, hi, i, j] = L.oracle_dropout_keep(_p(rs), bi * h + hi, i, j, thr)
+    return m
+
+
+def flash_fwd(q, k, v, scale, window=(-1, -1), round_p=True, p_dropout=0.0, rng_state=None):
+    """q [b,sq,h,d], k/v [b,sk,h_k,d] in one storage dtype; rng_state = (seed, offset) when
+    p_dropout > 0.
     -> (o storage dtype [b,sq,h,d], lse f32 [b,h,sq], o unrounded f32 [b,sq,h,d])."""
     q, k, v = (np.ascontiguousarray(t) for t in (q, k, v))
     b, sq, h, d = q.shape
     sk, h_k = k.shape[1], k.shape[2]
-    a = fa_args(b, sq, sk, h, h_k, d, scale, window)
+    a = fa_args(b, sq, sk, h, h_k, d, scale, window, p_dropout)
     o = np.empty_like(q)
     lse = np.empty((b, h, sq), dtype=np.float32)
     o32 = np.empty((b, sq, h, d), dtype=np.float32)
-    lib().oracle_flash_fwd(ctypes.byref(a), _code(q), int(round_p), _p(q), _p(k), _p(v), _p(o),
-                           _p(lse), _p(o32))
+    rs = np.asarray(rng_state, dtype=np.uint64) if p_dropout > 0 else None
+    lib().oracle_flash_fwd_rng(ctypes.byref(a), _code(q), int(round_p), _p(q), _p(k), _p(v),
+                               _p(rs) if rs is not None else None, _p(o), _p(lse), _p(o32))
     return o, lse, o32
 
 
-def flash_bwd(dout, q, k, v, o, lse, scale, window=(-1, -1), round_p=True):
-    """-> (dq, dk, dv in storage dtype, D = rowsum(dout*o) f32 [b,h,sq])."""
+def flash_bwd(dout, q, k, v, o, lse, scale, window=(-1, -1), round_p=True, p_dropout=0.0, rng_state=None):
+    """-> (dq, dk, dv in storage dtype, D = rowsum(dout*o) f32 [b,h,sq], times p_keep under dropout)."""
     dout, q, k, v, o = (np.ascontiguousarray(t) for t in (dout, q, k, v, o))
     lse = np.ascontiguousarray(lse, dtype=np.float32)
     b, sq, h, d = q.shape
     sk, h_k = k.shape[1], k.shape[2]
     assert h == h_k, "backward needs h == h_k"
-    a = fa_args(b, sq, sk, h, h_k, d, scale, window)
+    a = fa_args(b, sq, sk, h, h_k, d, scale, window, p_dropout)
     dq, dk, dv = np.empty_like(q), np.empty_like(k), np.empty_like(v)
     dsm = np.empty((b, h, sq), dtype=np.float32)
-    lib().oracle_flash_bwd(ctypes.byref(a), _code(q), int(round_p), _p(dout), _p(q), _p(k), _p(v),
-                           _p(o), _p(lse), _p(dq), _p(dk), _p(dv), _p(dsm))
+    rs = np.asarray(rng_state, dtype=np.uint64) if p_dropout > 0 else None
+    lib().oracle_flash_bwd_rng(ctypes.byref(a), _code(q), int(round_p), _p(dout), _p(q), _p(k), _p(v),
+                               _p(o), _p(lse), _p(rs) if rs is not None else None,
+                               _p(dq), _p(dk), _p(dv), _p(dsm))
     return dq, dk, dv, dsm
 
 

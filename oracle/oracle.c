@@ -26,6 +26,13 @@
  *   attention backward dQ,dK,dV              : the reference's golden vectors
  *       (flash_attn_bwd_outputs_{dq,dk,dv}.data), torch autograd through CPU SDPA and a
  *       finite-difference check.
+ *   Philox4x32                               : the published known-answer vectors of the
+ *       10-round generator (the library's 7-round call differs in the round count only).
+ *   attention dropout                        : the arithmetic around the mask by its closed form
+ *       on an explicit mask (tests build it element by element with oracle_dropout_keep) and by
+ *       finite differences; the keep rate against the 8-bit threshold.  PARITY UNPINNED for the
+ *       element-to-random-byte mapping of oracle_dropout_keep: no reference fixture exercises
+ *       dropout and the CUDA kernels cannot be run here.
  *   extra_args blob                          : byte-level known answer from the reference's
  *       fixture module runtime/test/test_files/flash_attn_fwd.mlir:9.
  */
@@ -373,17 +380,65 @@ static inline void window_bounds(int64_t i, int64_t sq, int64_t sk, int64_t wl, 
   *lo = l; *hi = h;
 }
 
+/* Philox4x32 with `rounds` rounds: key = seed, counter = (offset, subsequence)
+ * (lib/philox.cuh:22-52; the library runs 7 rounds: six with a key bump and a last one). */
+void oracle_philox4x32(uint64_t seed, uint64_t subsequence, uint64_t offset, int rounds, uint32_t out[4]) {
+  uint32_t k0 = (uint32_t)seed, k1 = (uint32_t)(seed >> 32);
+  uint32_t c[4] = {(uint32_t)offset, (uint32_t)(offset >> 32), (uint32_t)subsequence, (uint32_t)(subsequence >> 32)};
+  for (int r = 0; r < rounds; ++r) {
+    if (r > 0) { k0 += 0x9E3779B9u; k1 += 0xBB67AE85u; }
+    uint64_t p0 = (uint64_t)0xD2511F53u * c[0], p1 = (uint64_t)0xCD9E8D57u * c[2];
+    uint32_t n0 = (uint32_t)(p1 >> 32) ^ c[1] ^ k0, n1 = (uint32_t)p1;
+    uint32_t n2 = (uint32_t)(p0 >> 32) ^ c[3] ^ k1, n3 = (uint32_t)p0;
+    c[0] = n0; c[1] = n1; c[2] = n2; c[3] = n3;
+  }
+  memcpy(out, c, 16);
+}
+
+/* Dropout keep-mask of the attention matrix (lib/dropout.h:19-23,26-44,76-84 with the call sites
+ * flash_fwd_kernel.h:321-334 and flash_bwd_kernel.h:524-533).  The matrix is cut into blocks of
+ * 16 rows x 32 columns; one Philox call per (block, lane of a 32-lane warp) yields 16 bytes, one
+ * per element the lane holds in the m16n8 accumulator layout (row = lane/4 [+8], column =
+ * 8*tile + 2*(lane%4) [+1], four 8-column tiles): byte = 4*tile + 2*(row half) + (column & 1).
+ * subsequence = (row block, column block) as (low, high) words, offset = rng_state[1] +
+ * (batch*heads + head)*32 + lane, seed = rng_state[0]; kept iff byte <= floor(p_keep*255).
+ * parity unpinned: no reference fixture exercises dropout, so the element-to-byte mapping above
+ * is restated from the sources (and the accumulator layout of the m16n8k16 instruction) only. */
+int oracle_dropout_keep(const uint64_t *rng_state, int64_t bh, int64_t row, int64_t col, uint8_t threshold) {
+  const uint32_t lane = (uint32_t)((row % 8) * 4 + (col % 8) / 2);
+  const uint64_t subseq = (uint64_t)(uint32_t)(row / 16) | ((uint64_t)(uint32_t)(col / 32) << 32);
+  uint32_t r[4];
+  oracle_philox4x32(rng_state[0], subseq, rng_state[1] + (uint64_t)((int)bh * 32) + lane, 7, r);
+  const int tile = (int)((col % 32) / 8);
+  const int byte = 4 * tile + 2 * (int)((row % 16) / 8) + (int)(col & 1);
+  return (uint8_t)(r[byte >> 2] >> (8 * (byte & 3))) <= threshold;
+}
+
+/* p_keep, its 8-bit threshold and reciprocal as run_mha_fwd derives them (flash_api.cu:291-294) */
+static inline void dropout_consts(float p_dropout, float *p_keep, uint8_t *thr, float *rp) {
+  *p_keep = 1.f - p_dropout;
+  *thr = (uint8_t)floor(*p_keep * 255.0);
+  *rp = 1.f / *p_keep;
+}
+
 /* Forward, per (batch, head, query row): flash_fwd_kernel.h:276-469 with softmax.h:128-178.
  *   s_j = q_i . k_j in float; m = max_j s_j; p_j = exp2((s_j - m) * scale*log2e);
  *   l = sum_j p_j (float, unrounded p); o = (sum_j round16(p_j) v_j) / l, rounded to storage;
  *   lse = m*scale + ln(l); a row with nothing kept gives o = 0, lse = +inf (softmax.h:171-172).
  * round_p = 0 skips the rounding of P (plain float attention, the "fp32 reference").
  * dtype: 1 = f16, 2 = bf16, 0 = f32 storage.  lse layout [b, h, sq] float.
- * o_f32, when non-null, additionally receives the unrounded output [b, sq, h, d] dense. */
-void oracle_flash_fwd(const oracle_fa_args *a, int dtype, int round_p, const void *q,
-                      const void *k, const void *v, void *o, float *lse, float *o_f32) {
+ * o_f32, when non-null, additionally receives the unrounded output [b, sq, h, d] dense.
+ * With a->p_dropout > 0 (rng_state = {seed, offset} required): the row sum and LSE are those of
+ * the undropped P; dropped entries of the rounded P are zeroed before P V and O is multiplied
+ * by 1/p_keep (flash_fwd_kernel.h:333-335, softmax.h:173). */
+void oracle_flash_fwd_rng(const oracle_fa_args *a, int dtype, int round_p, const void *q,
+                          const void *k, const void *v, const uint64_t *rng_state, void *o,
+                          float *lse, float *o_f32) {
   const int64_t b = a->b, h = a->h, hk = a->h_k, d = a->d, sq = a->seqlen_q, sk = a->seqlen_k;
   const float scale = a->softmax_scale;
+  const int drop = a->p_dropout > 0.f && rng_state;
+  float p_keep, rp_keep; uint8_t thr;
+  dropout_consts(drop ? a->p_dropout : 0.f, &p_keep, &thr, &rp_keep);
   const float scale_log2 = (float)(scale * M_LOG2E); /* flash_api.cu:289 */
   const int64_t ratio = h / hk;
 #pragma omp parallel for num_threads(g_threads) schedule(dynamic, 8) collapse(3)
@@ -411,11 +466,13 @@ void oracle_flash_fwd(const oracle_fa_args *a, int dtype, int round_p, const voi
           float p = exp2f((s[j] - m) * scale_log2);
           l += p;
           float pr = round_p ? round_storage(p, dtype) : p;
+          if (drop && !oracle_dropout_keep(rng_state, bi * h + hi, i, j, thr)) continue;
           size_t voff = (size_t)(bi * a->v_batch_stride + j * a->v_row_stride + (hi / ratio) * a->v_head_stride);
           for (int64_t x = 0; x < d; ++x) acc[x] += pr * load_elem(v, voff + x, dtype);
         }
         int empty = (l == 0.f || l != l);
         float inv = empty ? 1.f : 1.f / l;
+        if (drop) inv *= rp_keep;
         for (int64_t x = 0; x < d; ++x) {
           float val = acc[x] * inv;
           store_elem(o, ooff + x, dtype, val);
@@ -426,6 +483,11 @@ void oracle_flash_fwd(const oracle_fa_args *a, int dtype, int round_p, const voi
       }
 }
 
+void oracle_flash_fwd(const oracle_fa_args *a, int dtype, int round_p, const void *q,
+                      const void *k, const void *v, void *o, float *lse, float *o_f32) {
+  oracle_flash_fwd_rng(a, dtype, round_p, q, k, v, NULL, o, lse, o_f32);
+}
+
 /* Backward: flash_bwd_preprocess_kernel.h:23-50 (D = rowsum(dO*O)) and
  * flash_bwd_kernel.h:455-718:
  *   p_ij = exp2(s_ij*scale*log2e - lse_i*log2e) (0 where masked); dp_ij = dO_i . v_j;
@@ -434,13 +496,21 @@ void oracle_flash_fwd(const oracle_fa_args *a, int dtype, int round_p, const voi
  * Accumulation in float; outputs rounded to storage.  round_p = 0 keeps p and ds unrounded.
  * dq/dk/dv use the strides of q/k/v (flash_api.cu:377-389).  h must equal h_k (the
  * reference's dK/dV addressing is only right in that case).  d_softmax [b, h, sq] float,
- * when non-null, receives D. */
-void oracle_flash_bwd(const oracle_fa_args *a, int dtype, int round_p, const void *dout,
-                      const void *q, const void *k, const void *v, const void *o,
-                      const float *lse, void *dq, void *dk, void *dv, float *d_softmax) {
+ * when non-null, receives D.
+ * With a->p_dropout > 0 (rng_state = {seed, offset} required), as the reference arranges it
+ * (flash_bwd_preprocess_kernel.h:124-128, flash_bwd_kernel.h:524-536,571-573,667,713-718):
+ * D is scaled by p_keep; a dropped entry contributes p = 0 to dV and ds = p * (-D); dQ and dK
+ * are scaled by scale/p_keep, dV by 1/p_keep. */
+void oracle_flash_bwd_rng(const oracle_fa_args *a, int dtype, int round_p, const void *dout,
+                          const void *q, const void *k, const void *v, const void *o,
+                          const float *lse, const uint64_t *rng_state, void *dq, void *dk, void *dv,
+                          float *d_softmax) {
   const int64_t b = a->b, h = a->h, d = a->d, sq = a->seqlen_q, sk = a->seqlen_k;
-  const float scale = a->softmax_scale;
-  const float scale_log2 = (float)(scale * M_LOG2E);
+  const int drop = a->p_dropout > 0.f && rng_state;
+  float p_keep, rp_keep; uint8_t thr;
+  dropout_consts(drop ? a->p_dropout : 0.f, &p_keep, &thr, &rp_keep);
+  const float scale = drop ? a->softmax_scale * rp_keep : a->softmax_scale;
+  const float scale_log2 = (float)(a->softmax_scale * M_LOG2E);
 #pragma omp parallel for num_threads(g_threads) schedule(dynamic, 1) collapse(2)
   for (int64_t bi = 0; bi < b; ++bi)
     for (int64_t hi = 0; hi < h; ++hi) {
@@ -459,6 +529,7 @@ void oracle_flash_bwd(const oracle_fa_args *a, int dtype, int round_p, const voi
           D += dof[x] * load_elem(o, ooff + x, dtype);
           dqacc[x] = 0.f;
         }
+        if (drop) D *= p_keep;
         if (d_softmax) d_softmax[(size_t)(bi * h + hi) * sq + i] = D;
         float lse_i = lse[(size_t)(bi * h + hi) * sq + i];
         int64_t lo, hi_;
@@ -473,6 +544,7 @@ void oracle_flash_bwd(const oracle_fa_args *a, int dtype, int round_p, const voi
           }
           float p = exp2f(dot * scale_log2 - lse_i * (float)M_LOG2E);
           float ds = p * (dp - D);
+          if (drop && !oracle_dropout_keep(rng_state, bi * h + hi, i, j, thr)) { ds = p * -D; p = 0.f; }
           float pr = round_p ? round_storage(p, dtype) : p;
           float dsr = round_p ? round_storage(ds, dtype) : ds;
           for (int64_t x = 0; x < d; ++x) {
@@ -488,9 +560,15 @@ void oracle_flash_bwd(const oracle_fa_args *a, int dtype, int round_p, const voi
         size_t voff = (size_t)(bi * a->v_batch_stride + j * a->v_row_stride + hi * a->v_head_stride);
         for (int64_t x = 0; x < d; ++x) {
           store_elem(dk, koff + x, dtype, dkacc[j * d + x] * scale);
-          store_elem(dv, voff + x, dtype, dvacc[j * d + x]);
+          store_elem(dv, voff + x, dtype, drop ? dvacc[j * d + x] * rp_keep : dvacc[j * d + x]);
         }
       }
       free(dkacc); free(dvacc); free(dqacc); free(qf); free(dof);
     }
+}
+
+void oracle_flash_bwd(const oracle_fa_args *a, int dtype, int round_p, const void *dout,
+                      const void *q, const void *k, const void *v, const void *o,
+                      const float *lse, void *dq, void *dk, void *dv, float *d_softmax) {
+  oracle_flash_bwd_rng(a, dtype, round_p, dout, q, k, v, o, lse, NULL, dq, dk, dv, d_softmax);
 }

@@ -157,7 +157,7 @@ def test_unsupported_arguments_are_reported_not_run():
     assert L.flash_attn_fwd_checked(arr, ctypes.cast(buf, ctypes.c_void_p), 1, None) == -1
     assert b"head_dim" in L.flash_attn_last_error()
     q = torch.zeros((1, 16, 1, 64), dtype=torch.float16, device="cuda")
-    blob = ops.pack_flash_args(q, q, q, q, 1.0, (-1, -1), p_dropout=0.1)
+    blob = ops.pack_flash_args(q, q, q, q, 1.0, (-1, -1), p_dropout=-0.5)
     buf = ctypes.create_string_buffer(blob, len(blob))
     assert L.flash_attn_fwd_checked(arr, ctypes.cast(buf, ctypes.c_void_p), 1, None) == -1
     assert b"p_dropout" in L.flash_attn_last_error()
@@ -310,3 +310,80 @@ def test_kvcache_unsupported_arguments_are_reported_not_run():
                                 o.data_ptr(), lse.data_ptr())
     assert L.flash_attn_kvcache_checked(arr, ctypes.cast(buf, ctypes.c_void_p), 1, None) == -1
     torch.cuda.synchronize()
+
+
+# ---- dropout -----------------------------------------------------------------------------------
+RNG_STATE = (0x9E3779B97F4A7C15, 0x1_0000_0003)   # seed with the top bit set, offset above 2^32
+
+
+@pytest.mark.parametrize("code", [oracle.F16, oracle.BF16])
+def test_dropout_mask_is_the_reference_function_of_position(code):
+    """V = rows of the identity (head_dim = seqlen_k) makes O[i, :] = keep[i, :] * P[i, :] / p_keep,
+    dO = rows of the identity (head_dim = seqlen_q) makes dV[j, :] = the same matrix transposed:
+    the kept set of the forward and of the dK/dV kernel must equal the oracle's mask bit for bit."""
+    from byteir_amd import ops
+    b, h, n, p_drop = 2, 3, 256, 0.3
+    rng = np.random.default_rng(11)
+    q = oracle.from_f32((0.1 * rng.standard_normal((b, n, h, n))).astype(np.float32), code)
+    k = oracle.from_f32((0.1 * rng.standard_normal((b, n, h, n))).astype(np.float32), code)
+    eye = oracle.from_f32(np.broadcast_to(np.eye(n, dtype=np.float32)[None, :, None, :], (b, n, h, n)).copy(), code)
+    rs = ops.rng_state_tensor(*RNG_STATE, "cuda")
+    keep = oracle.dropout_keep_mask(RNG_STATE, b, h, n, n, p_drop)          # [b, h, i, j]
+    dq_, dk_, deye = dev(q), dev(k), dev(eye)
+    o, lse = ops.flash_attn_fwd(dq_, dk_, deye, 0.05, (-1, -1), p_dropout=p_drop, rng_state=rs)
+    got = oracle.to_f32(host(o)).transpose(0, 2, 1, 3) != 0                 # [b, h, i, j]
+    assert np.array_equal(got, keep)
+    _, _, dv = ops.flash_attn_bwd(deye, dq_, dk_, deye, o, lse, 0.05, (-1, -1), p_dropout=p_drop, rng_state=rs)
+    got_t = oracle.to_f32(host(dv)).transpose(0, 2, 3, 1) != 0              # dv[b, j, h, i] -> [b, h, i, j]
+    assert np.array_equal(got_t, keep)
+
+
+DROP_CASES = [
+    # b, sq, sk, h, d, window, p_dropout
+    (2, 128, 128, 2, 64, (-1, 0), 0.1),
+    (1, 200, 333, 2, 128, (-1, -1), 0.5),
+    (1, 150, 90, 3, 32, (-1, 0), 0.25),
+    (1, 130, 260, 2, 96, (40, 30), 0.2),
+    (1, 70, 70, 1, 256, (-1, 0), 0.1),
+]
+
+
+@pytest.mark.parametrize("code", [oracle.F16, oracle.BF16])
+@pytest.mark.parametrize("case", DROP_CASES)
+def test_dropout_forward_and_backward_match_oracle(case, code):
+    from byteir_amd import ops
+    b, sq, sk, h, d, window, p_drop = case
+    q, k, v, do = make_inputs((b, sq, sk, h, h, d, window), code, seed=sum(case[:5]) + 7)
+    scale = 1.0 / np.sqrt(d)
+    rs = ops.rng_state_tensor(*RNG_STATE, "cuda")
+    dq_, dk_, dv_, do_ = (dev(t) for t in (q, k, v, do))
+    o, lse = ops.flash_attn_fwd(dq_, dk_, dv_, scale, window, p_dropout=p_drop, rng_state=rs)
+    _, lse_ref, o32 = oracle.flash_fwd(q, k, v, scale, window, round_p=False, p_dropout=p_drop, rng_state=RNG_STATE)
+    assert np.abs(oracle.to_f32(host(o)) - o32).max() <= ATOL
+    inf = np.isposinf(lse_ref)
+    assert np.array_equal(np.isposinf(host(lse)), inf)
+    assert np.abs(host(lse)[~inf] - lse_ref[~inf]).max() <= ATOL
+    dq, dk, dv = ops.flash_attn_bwd(do_, dq_, dk_, dv_, o, lse, scale, window, p_dropout=p_drop, rng_state=rs)
+    rq, rk, rv, _ = oracle.flash_bwd(do, q, k, v, host(o), host(lse), scale, window, round_p=False,
+                                     p_dropout=p_drop, rng_state=RNG_STATE)
+    for name, got, want in (("dq", dq, rq), ("dk", dk, rk), ("dv", dv, rv)):
+        err = np.abs(oracle.to_f32(host(got)) - oracle.to_f32(want)).max()
+        assert err <= ATOL, (name, float(err))
+
+
+def test_dropout_without_rng_state_is_reported():
+    import ctypes
+    from byteir_amd import _lib, ops
+    L = _lib.flash_attn()
+    L.flash_attn_fwd_checked.argtypes = [ctypes.POINTER(ctypes.c_void_p), ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p]
+    L.flash_attn_last_error.restype = ctypes.c_char_p
+    q = torch.zeros((1, 16, 1, 64), dtype=torch.float16, device="cuda")
+    blob = ops.pack_flash_args(q, q, q, q, 1.0, (-1, -1), p_dropout=0.1)
+    arr = (ctypes.c_void_p * 7)(q.data_ptr(), q.data_ptr(), q.data_ptr(), None, q.data_ptr(), q.data_ptr(), None)
+    buf = ctypes.create_string_buffer(blob, len(blob))
+    assert L.flash_attn_fwd_checked(arr, ctypes.cast(buf, ctypes.c_void_p), 1, None) == -1
+    assert b"rng_state" in L.flash_attn_last_error()
+    blob = ops.pack_flash_args(q, q, q, q, 1.0, (-1, -1), p_dropout=1.0)
+    buf = ctypes.create_string_buffer(blob, len(blob))
+    assert L.flash_attn_fwd_checked(arr, ctypes.cast(buf, ctypes.c_void_p), 1, None) == -1
+    assert b"p_dropout" in L.flash_attn_last_error()

@@ -251,3 +251,103 @@ def test_kvcache_extra_args_blob_known_answer():
     want = b"".join(struct.pack("<f", f) if isinstance(f, float) else struct.pack("<q", f) for f in fields)
     assert len(want) == 244
     assert oracle.fa_kvcache_pack_args(2, 1, 128, 3, 3, 32, 1, 0.5, (-1, -1)).tobytes() == want
+
+
+# ---- dropout ---------------------------------------------------------------------------------
+def _philox_words(ctr, key, rounds):
+    off, sub, seed = ctr[0] | (ctr[1] << 32), ctr[2] | (ctr[3] << 32), key[0] | (key[1] << 32)
+    return [int(x) for x in oracle.philox4x32(seed, sub, off, rounds)]
+
+
+def test_philox4x32_known_answer_vectors():
+    """The published known-answer vectors of Philox4x32 (Random123 kat_vectors: counter words,
+    key words -> output words), for the standard 10 rounds and for 7 rounds, the count the
+    reference library runs (lib/philox.cuh:43-50)."""
+    zero, ones = [0] * 4, [0xFFFFFFFF] * 4
+    pi_ctr, pi_key = [0x243F6A88, 0x85A308D3, 0x13198A2E, 0x03707344], [0xA4093822, 0x299F31D0]
+    assert _philox_words(zero, [0, 0], 10) == [0x6627E8D5, 0xE169C58D, 0xBC57AC4C, 0x9B00DBD8]
+    assert _philox_words(ones, ones[:2], 10) == [0x408F276D, 0x41C83B0E, 0xA20BC7C6, 0x6D5451FD]
+    assert _philox_words(pi_ctr, pi_key, 10) == [0xD16CFE09, 0x94FDCCEB, 0x5001E420, 0x24126EA1]
+    assert _philox_words(zero, [0, 0], 7) == [0x5F6FB709, 0x0D893F64, 0x4F121F81, 0x4F730A48]
+    assert _philox_words(ones, ones[:2], 7) == [0x5207DDC2, 0x45165E59, 0x4D8EE751, 0x8C52F662]
+
+
+def test_dropout_mask_structure():
+    """One Philox value serves one lane of one 16 x 32 block: the 16 elements that share
+    (row % 8, (col % 8) / 2) inside a block are exactly the 16 bytes of that value, and
+    different (batch, head) pairs use offsets 32 apart."""
+    rs = np.array([0x1234567, 1000], dtype=np.uint64)
+    b, h, sq, sk = 1, 2, 32, 64
+    for thr_p in (0.0, 0.37, 0.9):
+        m = oracle.dropout_keep_mask(rs, b, h, sq, sk, thr_p)
+        thr = oracle.dropout_threshold(thr_p)
+        for hi, rb, cb, lane in ((0, 0, 0, 0), (1, 1, 1, 13), (0, 1, 0, 31)):
+            r = oracle.philox4x32(rs[0], rb | (cb << 32), int(rs[1]) + hi * 32 + lane)
+            by = r.view(np.uint8)
+            for tile in range(4):
+                for half in range(2):
+                    for e in range(2):
+                        row = rb * 16 + lane // 4 + 8 * half
+                        col = cb * 32 + tile * 8 + 2 * (lane % 4) + e
+                        assert m[0, hi, row, col] == (by[4 * tile + 2 * half + e] <= thr)
+    # p_dropout = 0 keeps everything (threshold 255)
+    assert oracle.dropout_threshold(0.0) == 255 and oracle.dropout_keep_mask(rs, 1, 1, 16, 32, 0.0).all()
+
+
+def test_dropout_keep_rate_matches_the_8_bit_threshold():
+    rs = np.array([42, 7], dtype=np.uint64)
+    for p in (0.1, 0.5):
+        m = oracle.dropout_keep_mask(rs, 1, 2, 64, 128, p)
+        want = (oracle.dropout_threshold(p) + 1) / 256.0
+        assert abs(m.mean() - want) < 4 * np.sqrt(want * (1 - want) / m.size)
+
+
+def _dropout_reference(q, k, v, keep, p_drop, scale, causal):
+    """float64 attention with an explicit keep-mask: O = ((keep * softmax(S)) / p_keep) V"""
+    b, sq, h, d = q.shape
+    sk = k.shape[1]
+    q64, k64, v64 = (t.astype(np.float64) for t in (q, k, v))
+    s = np.einsum("bihd,bjhd->bhij", q64, k64) * scale
+    if causal:
+        i, j = np.arange(sq)[:, None], np.arange(sk)[None, :]
+        s = np.where(j > i + sk - sq, -np.inf, s)
+    p = np.exp(s - s.max(-1, keepdims=True))
+    p /= p.sum(-1, keepdims=True)
+    z = np.where(keep, p, 0.0) / np.float64(np.float32(1.0) - np.float32(p_drop))
+    return np.einsum("bhij,bjhd->bihd", z, v64), z, p
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_dropout_forward_is_attention_with_the_explicit_mask(causal):
+    rng = np.random.default_rng(5)
+    b, sq, sk, h, d, p_drop = 2, 40, 72, 2, 16, 0.25
+    q, k, v = (rng.standard_normal((b, s, h, d)).astype(np.float32) for s in (sq, sk, sk))
+    rs = np.array([0xDEADBEEFCAFE, 12345], dtype=np.uint64)
+    keep = oracle.dropout_keep_mask(rs, b, h, sq, sk, p_drop)
+    window = (-1, 0) if causal else (-1, -1)
+    o, lse, o32 = oracle.flash_fwd(q, k, v, 0.3, window, round_p=False, p_dropout=p_drop, rng_state=rs)
+    want, _, _ = _dropout_reference(q, k, v, keep, p_drop, 0.3, causal)
+    np.testing.assert_allclose(o32, want, atol=2e-5, rtol=1e-4)
+    # LSE is that of the undropped scores
+    _, lse0, _ = oracle.flash_fwd(q, k, v, 0.3, window, round_p=False)
+    assert np.array_equal(lse, lse0)
+
+
+def test_dropout_backward_is_the_gradient_with_the_mask_held_fixed():
+    rng = np.random.default_rng(6)
+    b, sq, sk, h, d, p_drop, scale = 1, 24, 40, 2, 8, 0.4, 0.35
+    q, k, v, do = (rng.standard_normal((b, s, h, d)).astype(np.float32) for s in (sq, sk, sk, sq))
+    rs = np.array([99, 4], dtype=np.uint64)
+    keep = torch.from_numpy(oracle.dropout_keep_mask(rs, b, h, sq, sk, p_drop))
+    p_keep = float(np.float32(1.0) - np.float32(p_drop))
+    tq, tk, tv = (torch.from_numpy(t).double().requires_grad_(True) for t in (q, k, v))
+    s = torch.einsum("bihd,bjhd->bhij", tq, tk) * scale
+    z = torch.where(keep, torch.softmax(s, -1), torch.zeros((), dtype=torch.float64)) / p_keep
+    out = torch.einsum("bhij,bjhd->bihd", z, tv)
+    out.backward(torch.from_numpy(do).double())
+    o, lse, o32 = oracle.flash_fwd(q, k, v, scale, round_p=False, p_dropout=p_drop, rng_state=rs)
+    dq, dk, dv, dsm = oracle.flash_bwd(do, q, k, v, o32, lse, scale, round_p=False, p_dropout=p_drop, rng_state=rs)
+    for got, want in ((dq, tq.grad), (dk, tk.grad), (dv, tv.grad)):
+        np.testing.assert_allclose(got, want.numpy(), atol=3e-5, rtol=1e-4)
+    # D is kept scaled by p_keep (flash_bwd_preprocess_kernel.h:124-128)
+    np.testing.assert_allclose(dsm, np.einsum("bihd,bihd->bhi", do, o32) * p_keep, atol=1e-5, rtol=1e-5)
