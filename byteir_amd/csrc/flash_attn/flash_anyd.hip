@@ -150,7 +150,11 @@ struct DropCtx {
 
 __device__ __forceinline__ void block_of(const Params &p, int n_blocks, bool reversed, int &blk, int &bh) {
   const int L = blockIdx.x;
-  if (p.xcd_remap) {  // consecutive workgroup ids go round-robin over the 8 XCDs
+  if (p.xcd_remap == 2) {  // unequal blocks: the longest block of every (batch, head) first
+    const int xcd = L & 7, slot = L >> 3, per_xcd = (p.b * p.h) >> 3;
+    bh = (slot % per_xcd) * 8 + xcd;
+    blk = slot / per_xcd;
+  } else if (p.xcd_remap) {  // consecutive workgroup ids go round-robin over the 8 XCDs
     const int xcd = L & 7, slot = L >> 3;
     bh = (slot / n_blocks) * 8 + xcd;
     blk = slot % n_blocks;

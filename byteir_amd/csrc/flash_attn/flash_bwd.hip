@@ -127,7 +127,11 @@ __global__ void __launch_bounds__(256, (D <= 64 && KB == 1) ? 2 : 1) dkdv_kernel
   int n_block, bh;
   {
     const int L = blockIdx.x;
-    if (p.xcd_remap) {
+    if (p.xcd_remap == 2) {  // unequal blocks: the longest (first) key block of every head first
+      const int xcd = L & 7, slot = L >> 3, per_xcd = (p.b * p.h) >> 3;
+      bh = (slot % per_xcd) * 8 + xcd;
+      n_block = slot / per_xcd;
+    } else if (p.xcd_remap) {
       const int xcd = L & 7, slot = L >> 3;
       bh = (slot / p.n_nblocks) * 8 + xcd;
       n_block = slot % p.n_nblocks;
@@ -382,7 +386,11 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) dq_kernel(const Params p
   int m_block, bh;
   {
     const int L = blockIdx.x;
-    if (p.xcd_remap) {
+    if (p.xcd_remap == 2) {  // unequal blocks: the longest (last) query block of every head first
+      const int xcd = L & 7, slot = L >> 3, per_xcd = (p.b * p.h) >> 3;
+      bh = (slot % per_xcd) * 8 + xcd;
+      m_block = slot / per_xcd;
+    } else if (p.xcd_remap) {
       const int xcd = L & 7, slot = L >> 3;
       bh = (slot / p.n_mblocks) * 8 + xcd;
       m_block = slot % p.n_mblocks;
@@ -597,7 +605,7 @@ hipError_t launch_bwd_t(const Params &p, hipStream_t stream) {
 hipError_t launch_bwd(Params &p, int dtype, hipStream_t stream) {
   p.n_mblocks = (p.sq + kQBlock - 1) / kQBlock;
   p.n_nblocks = (p.sk + kKvBlock - 1) / kKvBlock;
-  p.xcd_remap = ((p.b * p.h) % 8 == 0) ? 1 : 0;
+  p.xcd_remap = ((p.b * p.h) % 8 == 0) ? (p.wr >= 0 ? 2 : 1) : 0;
   if (p.b * p.h == 0) return hipSuccess;
   if (p.drop || (p.d != 32 && p.d != 64 && p.d != 128)) return launch_bwd_anyd(p, dtype, stream);
   return dtype == 1 ? launch_bwd_t<_Float16>(p, stream) : launch_bwd_t<__bf16>(p, stream);

@@ -116,7 +116,7 @@ struct Params {
   float scale, scale_log2;
   int wl, wr;                         // window sizes after normalisation; < 0 = unbounded
   int n_mblocks, n_nblocks;
-  int xcd_remap;                      // 1: blocks of one (batch, head) share an XCD
+  int xcd_remap;                      // 1: blocks of one (batch, head) share an XCD; 2: also longest blocks of all heads first
   // key/value cache calls only: per-batch number of keys already in the cache (the cache
   // holds p.sk rows), rows appended from k_new / v_new before attending
   const int *seqlens_k;

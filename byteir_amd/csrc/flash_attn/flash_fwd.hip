@@ -52,7 +52,16 @@ __global__ void __launch_bounds__(NW * 64, NW * QB >= 16 ? 2 : (QB == 2 ? 1 : 2)
   int m_block, bh;
   {
     const int L = blockIdx.x;
-    if (p.xcd_remap) {  // consecutive workgroup ids go round-robin over the 8 XCDs
+    if (p.xcd_remap == 2) {
+      // Blocks of unequal length (a right window): within an XCD, the longest block of every
+      // (batch, head) first, then the second longest of every one, ...: longest-first list
+      // scheduling, which fills the CUs evenly over the causal triangle (measured 216 -> 178 us
+      // on fp16 causal b4 h32 s2048 d128) at the price of more (batch, head) pairs in flight
+      // per L2.
+      const int xcd = L & 7, slot = L >> 3, per_xcd = (p.b * p.h) >> 3;
+      bh = (slot % per_xcd) * 8 + xcd;
+      m_block = slot / per_xcd;
+    } else if (p.xcd_remap) {  // consecutive workgroup ids go round-robin over the 8 XCDs
       const int xcd = L & 7, slot = L >> 3;
       bh = (slot / p.n_mblocks) * 8 + xcd;
       m_block = slot % p.n_mblocks;
@@ -377,7 +386,7 @@ hipError_t launch_append_kv(const Params &p, int dtype, hipStream_t stream) {
 }
 
 hipError_t launch_fwd(Params &p, int dtype, hipStream_t stream) {
-  p.xcd_remap = ((p.b * p.h) % 8 == 0) ? 1 : 0;
+  p.xcd_remap = ((p.b * p.h) % 8 == 0) ? (p.wr >= 0 ? 2 : 1) : 0;
   if (p.b * p.h == 0 || p.sq == 0) return hipSuccess;
   if (p.drop || (p.d != 32 && p.d != 64 && p.d != 128)) return launch_fwd_anyd(p, dtype, stream);
   return dtype == 1 ? launch_fwd_t<_Float16>(p, stream) : launch_fwd_t<__bf16>(p, stream);
