@@ -209,16 +209,27 @@ __global__ void __launch_bounds__(256, (D <= 64 && KB == 1) ? 2 : 1) dkdv_kernel
   auto lstore = [&](int buf) {
     lq.lstore(Qs[buf], QS);
     ldo.lstore(dOs[buf], QS);
-    if (tid < kQTile) { lse_s[buf][tid] = lse_r * kLog2e; dsm_s[buf][tid] = dsm_r; }
+    if (tid < kQTile) { lse_s[buf][tid] = lse_r * kLog2e; dsm_s[buf][tid] = -dsm_r; }
   };
 
   struct Unit { float16v s[KB], dp[KB]; };
   const int frag_rd = r32 * QS + g * 8;  // this lane's plain fragment inside a 32-row unit
 
-  // A: S = Q K^T, dP = dO V^T for the 32 query rows of unit `qs` of a tile
-  auto part_a = [&](const T *Qt, const T *dOt, int qs, Unit &u) {
+  // A: S = Q K^T, dP - D = dO V^T - D for the 32 query rows of unit `qs` of a tile.  The
+  // accumulator of dP starts from -D (staged negated in LDS, four consecutive rows per read in
+  // the C layout), which takes the subtraction of dS = P (dP - D) off the vector ALU.
+  auto part_a = [&](const T *Qt, const T *dOt, const float *negD, int qs, Unit &u) {
 #pragma unroll
-    for (int kb = 0; kb < KB; ++kb) { u.s[kb] = float16v{0}; u.dp[kb] = float16v{0}; }
+    for (int i4 = 0; i4 < 4; ++i4) {
+      const float4 d4 = *reinterpret_cast<const float4 *>(&negD[qs * 32 + i4 * 8 + g * 4]);
+#pragma unroll
+      for (int kb = 0; kb < KB; ++kb) {
+        u.dp[kb][i4 * 4 + 0] = d4.x; u.dp[kb][i4 * 4 + 1] = d4.y;
+        u.dp[kb][i4 * 4 + 2] = d4.z; u.dp[kb][i4 * 4 + 3] = d4.w;
+      }
+    }
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb) u.s[kb] = float16v{0};
 #pragma unroll
     for (int ks = 0; ks < D / 16; ++ks) {
       const vec8 aq = lds_read8<T>(&Qt[qs * 32 * QS + frag_rd + ks * 16]);
@@ -248,8 +259,7 @@ __global__ void __launch_bounds__(256, (D <= 64 && KB == 1) ? 2 : 1) dkdv_kernel
     for (int i4 = 0; i4 < 4; ++i4) {
       const int ql = qs * 32 + i4 * 8 + g * 4;  // 4 consecutive rows of the LDS tile
       const float4 l4 = *reinterpret_cast<const float4 *>(&lse_s[buf][ql]);
-      const float4 d4 = *reinterpret_cast<const float4 *>(&dsm_s[buf][ql]);
-      const float lq4[4] = {l4.x, l4.y, l4.z, l4.w}, dq4[4] = {d4.x, d4.y, d4.z, d4.w};
+      const float lq4[4] = {l4.x, l4.y, l4.z, l4.w};
 #pragma unroll
       for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
@@ -257,7 +267,7 @@ __global__ void __launch_bounds__(256, (D <= 64 && KB == 1) ? 2 : 1) dkdv_kernel
           const int i = i4 * 4 + j;
           const float pe = exp2_fast(fmaf(u.s[kb][i], c, -lq4[j]));
           pv[kb][i] = pe;
-          dsv[kb][i] = pe * (u.dp[kb][i] - dq4[j]);
+          dsv[kb][i] = pe * u.dp[kb][i];  // dp already holds dP - D
         }
     }
 #pragma unroll
@@ -297,7 +307,7 @@ __global__ void __launch_bounds__(256, (D <= 64 && KB == 1) ? 2 : 1) dkdv_kernel
     for (int w = 0; w < 2; ++w) { pb[kb][w] = vec8{0}; dsb[kb][w] = vec8{0}; }
   auto step = [&](int buf, int qs, int q0, int pbuf, int pqs) {
     Unit u;
-    part_a(Qs[buf], dOs[buf], qs, u);
+    part_a(Qs[buf], dOs[buf], dsm_s[buf], qs, u);
     if (!all_kept(q0)) mask(u, q0);
     vec8 pb_new[KB][2], dsb_new[KB][2];
     part_c(Qs[pbuf], dOs[pbuf], pqs, pb, dsb);
@@ -438,6 +448,11 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) dq_kernel(const Params p
 #pragma unroll
   for (int ks = 0; ks < D / 16; ++ks) asm volatile("" : "+v"(qf[ks]), "+v"(dof[ks]));
   asm volatile("" : "+v"(lse_l), "+v"(dsm_l));
+  // -D of the lane's row in all 16 accumulator slots: dP^T starts from it (the MFMA's C
+  // operand), which takes the subtraction of dS = P (dP - D) off the vector ALU
+  float16v neg_d;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) neg_d[i] = -dsm_l;
   float16v dq_acc[D / 32];
 #pragma unroll
   for (int i = 0; i < D / 32; ++i) dq_acc[i] = float16v{0};
@@ -470,7 +485,7 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) dq_kernel(const Params p
   // A: S^T = K Q^T, dP^T = V dO^T for the unit whose fragments are in fk / fv
   auto part_a = [&](Unit &u) {
     u.s = float16v{0};
-    u.dp = float16v{0};
+    u.dp = neg_d;
 #pragma unroll
     for (int ks = 0; ks < D / 16; ++ks) {
       u.s = Traits<T>::mfma(fk[ks], qf[ks], u.s);
@@ -490,7 +505,7 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) dq_kernel(const Params p
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       const float pe = exp2_fast(fmaf(u.s[i], c, -lse_l));
-      u.s[i] = pe * (u.dp[i] - dsm_l);
+      u.s[i] = pe * u.dp[i];  // dp already holds dP - D
     }
 #pragma unroll
     for (int w = 0; w < 2; ++w) {
