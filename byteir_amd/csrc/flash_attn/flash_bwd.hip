@@ -88,6 +88,13 @@ struct TileLoader {
     for (int s = 0; s < NP; ++s)
       *reinterpret_cast<uint4 *>(&tile[(s * RPP + r) * stride + c * 8]) = reg[s];
   }
+  // the same into a tile laid out with Swz<D> (no padding, chunks permuted per row)
+  __device__ __forceinline__ void lstore_swz(T *tile) const {
+    const int c = threadIdx.x % CPR, r = threadIdx.x / CPR;
+#pragma unroll
+    for (int s = 0; s < NP; ++s)
+      *reinterpret_cast<uint4 *>(&tile[Swz<D>::off(s * RPP + r, c)]) = reg[s];
+  }
 };
 
 // ---- 2. dK, dV ------------------------------------------------------------------------------
@@ -112,7 +119,7 @@ __global__ void __launch_bounds__(256, (D <= 64 && KB == 1) ? 2 : 1) dkdv_kernel
   // Tiles are read both plainly and transposed.  A stride of 4*odd banks keeps the plain reads
   // free of bank conflicts; the transposed ones then conflict in about a fifth of the LDS
   // cycles (a third with D + 16, nearly half with D + 32) -- with < 3 % effect on the time.
-  constexpr int QS = Pad<D>::kPlain;
+  constexpr int QS = D;  // unpadded, chunks permuted per row (Swz<D>): read plainly and transposed
   constexpr int kRing = 3;
   __shared__ __attribute__((aligned(16))) T Qs[kRing][kQTile * QS];
   __shared__ __attribute__((aligned(16))) T dOs[kRing][kQTile * QS];
@@ -207,13 +214,15 @@ __global__ void __launch_bounds__(256, (D <= 64 && KB == 1) ? 2 : 1) dkdv_kernel
     q_next += kQTile;
   };
   auto lstore = [&](int buf) {
-    lq.lstore(Qs[buf], QS);
-    ldo.lstore(dOs[buf], QS);
+    lq.lstore_swz(Qs[buf]);
+    ldo.lstore_swz(dOs[buf]);
     if (tid < kQTile) { lse_s[buf][tid] = lse_r * kLog2e; dsm_s[buf][tid] = -dsm_r; }
   };
 
   struct Unit { float16v s[KB], dp[KB]; };
-  const int frag_rd = r32 * QS + g * 8;  // this lane's plain fragment inside a 32-row unit
+  int frag_rd[D / 16];  // this lane's plain fragments inside a 32-row unit
+#pragma unroll
+  for (int ks = 0; ks < D / 16; ++ks) frag_rd[ks] = Swz<D>::off(r32, ks * 2 + g);
 
   // A: S = Q K^T, dP - D = dO V^T - D for the 32 query rows of unit `qs` of a tile.  The
   // accumulator of dP starts from -D (staged negated in LDS, four consecutive rows per read in
@@ -232,8 +241,8 @@ __global__ void __launch_bounds__(256, (D <= 64 && KB == 1) ? 2 : 1) dkdv_kernel
     for (int kb = 0; kb < KB; ++kb) u.s[kb] = float16v{0};
 #pragma unroll
     for (int ks = 0; ks < D / 16; ++ks) {
-      const vec8 aq = lds_read8<T>(&Qt[qs * 32 * QS + frag_rd + ks * 16]);
-      const vec8 ad = lds_read8<T>(&dOt[qs * 32 * QS + frag_rd + ks * 16]);
+      const vec8 aq = lds_read8<T>(&Qt[qs * 32 * QS + frag_rd[ks]]);
+      const vec8 ad = lds_read8<T>(&dOt[qs * 32 * QS + frag_rd[ks]]);
 #pragma unroll
       for (int kb = 0; kb < KB; ++kb) {
         u.s[kb] = Traits<T>::mfma(aq, kf[kb][ks], u.s[kb]);
@@ -284,8 +293,8 @@ __global__ void __launch_bounds__(256, (D <= 64 && KB == 1) ? 2 : 1) dkdv_kernel
     for (int w = 0; w < 2; ++w)
 #pragma unroll
       for (int db = 0; db < D / 32; ++db) {
-        const vec8 a_do = lds_read_operand_tr<T>(dOt, QS, qs * 32 + w * 16, db * 32);
-        const vec8 a_q = lds_read_operand_tr<T>(Qt, QS, qs * 32 + w * 16, db * 32);
+        const vec8 a_do = lds_read_operand_tr_swz<T, D>(dOt, qs * 32 + w * 16, db);
+        const vec8 a_q = lds_read_operand_tr_swz<T, D>(Qt, qs * 32 + w * 16, db);
 #pragma unroll
         for (int kb = 0; kb < KB; ++kb) {
           dv_acc[kb][db] = Traits<T>::mfma(a_do, pb[kb][w], dv_acc[kb][db]);
@@ -382,7 +391,7 @@ __global__ void __launch_bounds__(256, (D <= 64 && KB == 1) ? 2 : 1) dkdv_kernel
 template <typename T, int D>
 __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) dq_kernel(const Params p) {
   using vec8 = typename Traits<T>::vec8;
-  constexpr int KS = Pad<D>::kPlain;  // K tile: plain and transposed reads (see dkdv_kernel)
+  constexpr int KS = D;               // K tile: plain and transposed reads, laid out with Swz<D>
   constexpr int VS = Pad<D>::kPlain;  // V tile: plain reads only
   constexpr int kRing = 3;
   __shared__ __attribute__((aligned(16))) T Ks[kRing][kKvTile * KS];
@@ -462,10 +471,13 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) dq_kernel(const Params p
   lk.start(kg, p.k_rs, n_min * kKvTile, p.sk);
   lv.start(vg, p.v_rs, n_min * kKvTile, p.sk);
   auto gload = [&]() { lk.gload(); lv.gload(); };
-  auto lstore = [&](int buf) { lk.lstore(Ks[buf], KS); lv.lstore(Vs[buf], VS); };
+  auto lstore = [&](int buf) { lk.lstore_swz(Ks[buf]); lv.lstore(Vs[buf], VS); };
 
   struct Unit { float16v s, dp; };
-  const int frag_k = r32 * KS + g * 8, frag_v = r32 * VS + g * 8;
+  const int frag_v = r32 * VS + g * 8;
+  int frag_k[D / 16];
+#pragma unroll
+  for (int ks = 0; ks < D / 16; ++ks) frag_k[ks] = Swz<D>::off(r32, ks * 2 + g);
 
   // what the wave's 32 rows see of the 32 keys from kv0: 0 nothing, 1 all, 2 an edge crosses
   auto visibility = [&](int kv0) {
@@ -478,7 +490,7 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) dq_kernel(const Params p
   auto fetch = [&](const T *Kt, const T *Vt, int kvb) {
 #pragma unroll
     for (int ks = 0; ks < D / 16; ++ks) {
-      fk[ks] = lds_read8<T>(&Kt[kvb * 32 * KS + frag_k + ks * 16]);
+      fk[ks] = lds_read8<T>(&Kt[kvb * 32 * KS + frag_k[ks]]);
       fv[ks] = lds_read8<T>(&Vt[kvb * 32 * VS + frag_v + ks * 16]);
     }
   };
@@ -521,7 +533,7 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) dq_kernel(const Params p
     for (int w = 0; w < 2; ++w)
 #pragma unroll
       for (int db = 0; db < D / 32; ++db) {
-        const vec8 a = lds_read_operand_tr<T>(Kt, KS, kvb * 32 + w * 16, db * 32);
+        const vec8 a = lds_read_operand_tr_swz<T, D>(Kt, kvb * 32 + w * 16, db);
         dq_acc[db] = Traits<T>::mfma(a, dsb[w], dq_acc[db]);
       }
   };

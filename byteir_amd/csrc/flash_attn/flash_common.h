@@ -102,6 +102,44 @@ template <int D> struct Pad {
   static constexpr int kTr = D % 64 == 32 ? D : D + 32;
 };
 
+// Unpadded tiles that are read both ways (backward: Q, dO and K) cannot satisfy both stride
+// rules, so their 16-byte chunks are permuted inside each row instead: chunk c of row r lives
+// at chunk c ^ key(r).  key() is chosen so that (a) 16 consecutive rows put one logical chunk
+// into 16 different 16-byte bank groups (plain reads), and (b) the 4 rows x 4 chunks that one
+// half-wave fetches in a transposing read fall into four different 64-byte bank windows.
+// A row is D/8 chunks = D/2 banks, so four rows (D = 32), two (D = 64) or one (D = 128) span
+// the 64 banks.  key(r) = key(r + 32), so a lane's offsets inside a 32-row unit do not depend
+// on the unit.
+template <int D> struct Swz {
+  static __device__ __forceinline__ int key(int row) {
+    if constexpr (D == 64) {
+      const int x = (row >> 1) & 7;  // rows 2x, 2x+1 share a key and differ in bank parity
+      return ((x & 1) << 2) | (x >> 1);
+    } else if constexpr (D == 128) {
+      return ((row & 3) << 2) | ((row >> 2) & 3);
+    } else {
+      return (row >> 2) & 3;  // D == 32: four rows span the banks
+    }
+  }
+  // element offset of logical chunk `chunk` of row `row`
+  static __device__ __forceinline__ int off(int row, int chunk) { return row * D + ((chunk ^ key(row)) << 3); }
+};
+
+// lds_read_operand_tr for a tile laid out with Swz<D>: rows row0.., columns db*32..
+template <typename T, int D>
+__device__ __forceinline__ typename Traits<T>::vec8 lds_read_operand_tr_swz(const T *tile, int row0, int db) {
+  const int lane = threadIdx.x & 63;
+  const int i16 = lane & 15, b16 = lane >> 4;
+  const int row = row0 + (b16 >> 1) * 4 + (i16 >> 2);
+  const int chunk = db * 4 + (b16 & 1) * 2 + ((i16 & 3) >> 1), in_chunk = (i16 & 1) * 4;
+  const short4v lo = lds_read_tr4(tile + Swz<D>::off(row, chunk) + in_chunk);
+  const short4v hi = lds_read_tr4(tile + Swz<D>::off(row + 8, chunk) + in_chunk);
+  short8v v;
+  v.s0 = lo.s0; v.s1 = lo.s1; v.s2 = lo.s2; v.s3 = lo.s3;
+  v.s4 = hi.s0; v.s5 = hi.s1; v.s6 = hi.s2; v.s7 = hi.s3;
+  return __builtin_bit_cast(typename Traits<T>::vec8, v);
+}
+
 struct Params {
   const void *q, *k, *v, *o, *dout;  // o is written by forward, read by backward
   void *o_w;                          // forward output
