@@ -1,0 +1,281 @@
+// Attention of a few query rows against a long key/value cache (the decode step of
+// run_flash_attn_kvcache, reference: flash_api.cu:434-567 -> compute_attn_1rowblock_splitkv,
+// flash_fwd_kernel.h:480-970).  HBM-bound: the job is to read K and V once, at full rate.
+//
+// All query heads that share a key/value head (h / h_k of them) times all query rows are the
+// up to 32 columns of one S^T tile, so a cache row is fetched once for the whole group.  The
+// key axis is cut three ways: into `n_splits` chunks over workgroups (so that a small batch
+// still fills the chip), inside a workgroup round-robin over its four waves in units of 32
+// keys, and a wave walks its units with the next one in flight.  There is no barrier in the
+// loop: a wave loads its K fragments straight from global memory in MFMA operand layout and
+// stages V through a private, double-buffered LDS tile for the transposing read.  The waves'
+// partial (max, sum, O) are merged through LDS at the end; with more than one chunk the
+// workgroups write unnormalised fp32 partials and a second kernel merges them
+// (the reference's flash_fwd_splitkv_combine_kernel plays that role; its entry point fixes
+// num_splits = 1 for want of a workspace, flash_api.cu:548-563 -- here the workspace is a
+// stream-ordered allocation).
+// Arithmetic as in the forward kernel: fp32 scores, exp2 with scale*log2(e) folded in, P rounded
+// to the storage type before P V, O divided by the row sum at the very end, LSE = max*scale +
+// ln(sum), a row without keys gives O = 0 and LSE = +inf.
+#include "flash_common.h"
+
+namespace fa {
+namespace {
+
+constexpr int kDecWaves = 4;
+constexpr int kUnit = 32;  // keys per unit
+
+struct DecodeArgs {
+  float *o_part;   // [n_splits][b][h][sq][D] unnormalised O relative to the partial max; null: one chunk
+  float *ml_part;  // [n_splits][b][h][sq][2] partial max (score units) and row sum
+  int n_splits;
+  int chunk;       // keys per chunk, a multiple of kUnit
+};
+
+template <typename T, int D>
+__global__ void __launch_bounds__(kDecWaves * 64, 2) decode_kernel(const Params p, const DecodeArgs a) {
+  using vec8 = typename Traits<T>::vec8;
+  constexpr int VS = Pad<D>::kTr;
+  constexpr int CPR = D / 8;         // 16-byte chunks per V row
+  constexpr int RPP = 64 / CPR;      // V rows per pass of a wave
+  constexpr int NPV = kUnit / RPP;   // passes per unit
+  constexpr int kWaveLds = 2 * kUnit * VS * (int)sizeof(T);  // a wave's two V tiles, reused for the merge
+  static_assert(kWaveLds >= (D * 32 + 64) * 4, "merge buffers must fit the V tiles");
+  __shared__ __attribute__((aligned(16))) unsigned char lds[kDecWaves][kWaveLds];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r32 = lane & 31, g = lane >> 5;
+  const int split = blockIdx.x % a.n_splits;
+  const int bhk = blockIdx.x / a.n_splits;
+  const int bi = bhk / p.h_k, hk = bhk % p.h_k;
+  const int group = p.h / p.h_k;
+  int sk = p.sk;
+  if (p.seqlens_k) sk = min(p.sk, p.seqlens_k[bi] + p.seqlen_knew);
+
+  // column n of the S^T tile: query head hk*group + n / sq, query row n % sq
+  const bool col_ok = r32 < group * p.sq;
+  const int qi = col_ok ? r32 % p.sq : 0, hq = hk * group + (col_ok ? r32 / p.sq : 0);
+  int lo_lim = 0, hi_lim = 0;
+  if (col_ok) row_limits_sk(p, sk, qi, lo_lim, hi_lim);
+  // keys of this chunk that some row can see
+  int lo_all, hi_all, t0, t1;
+  row_limits_sk(p, sk, 0, lo_all, t0);
+  row_limits_sk(p, sk, p.sq - 1, t1, hi_all);
+  const int c0 = max(split * a.chunk, lo_all / kUnit * kUnit);
+  const int c1 = min((split + 1) * a.chunk, hi_all);
+  const int n_units = c1 > c0 ? (c1 - c0 + kUnit - 1) / kUnit : 0;
+
+  const T *kg = static_cast<const T *>(p.k) + bi * p.k_bs + hk * p.k_hs;
+  const T *vg = static_cast<const T *>(p.v) + bi * p.v_bs + hk * p.v_hs;
+  vec8 qf[D / 16];
+  {
+    const T *qg = static_cast<const T *>(p.q) + bi * p.q_bs + (int64_t)qi * p.q_rs + hq * p.q_hs;
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ++ks)
+      qf[ks] = col_ok ? *reinterpret_cast<const vec8 *>(qg + ks * 16 + g * 8) : vec8{0};
+  }
+
+  T *Vt[2] = {reinterpret_cast<T *>(lds[wave]), reinterpret_cast<T *>(lds[wave]) + kUnit * VS};
+  vec8 kc[D / 16], kn[D / 16];
+  uint4 vn[NPV];
+  const int v_c = lane % CPR, v_r = lane / CPR;
+  auto load_unit = [&](int j, vec8 (&kf)[D / 16]) {  // unit j of the chunk: K fragments and V staging registers
+    const int key = c0 + j * kUnit + r32;
+    const T *kr = kg + (int64_t)key * p.k_rs + g * 8;
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ++ks)
+      kf[ks] = key < c1 ? *reinterpret_cast<const vec8 *>(kr + ks * 16) : vec8{0};
+#pragma unroll
+    for (int s = 0; s < NPV; ++s) {
+      const int vk = c0 + j * kUnit + s * RPP + v_r;
+      // zero rows: 0 * finite stays finite in P V
+      vn[s] = vk < c1 ? *reinterpret_cast<const uint4 *>(vg + (int64_t)vk * p.v_rs + v_c * 8) : uint4{0, 0, 0, 0};
+    }
+  };
+  auto store_v = [&](T *tile) {
+#pragma unroll
+    for (int s = 0; s < NPV; ++s) *reinterpret_cast<uint4 *>(&tile[(s * RPP + v_r) * VS + v_c * 8]) = vn[s];
+  };
+
+  float16v o_acc[D / 32];
+#pragma unroll
+  for (int i = 0; i < D / 32; ++i) o_acc[i] = float16v{0};
+  float m_run = -INFINITY, l_run = 0.f;
+  const float c = p.scale_log2;
+
+  if (wave < n_units) {
+    load_unit(wave, kc);
+    store_v(Vt[0]);
+  }
+  int buf = 0;
+  for (int j = wave; j < n_units; j += kDecWaves) {
+    const bool has_next = j + kDecWaves < n_units;
+    if (has_next) load_unit(j + kDecWaves, kn);
+    float16v s = float16v{0};
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ++ks) s = Traits<T>::mfma(kc[ks], qf[ks], s);
+    const int kv0 = c0 + j * kUnit;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int kv = kv0 + (i >> 2) * 8 + g * 4 + (i & 3);
+      if (kv >= hi_lim || kv < lo_lim) s[i] = -INFINITY;
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[i]);
+    mx = fmaxf(mx, partner32(mx));
+    const float m_new = fmaxf(m_run, mx);
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;
+    const float alpha = exp2_fast((m_run - m_use) * c);
+    const float m_scaled = m_use * c;
+    float rs = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const float e = exp2_fast(fmaf(s[i], c, -m_scaled));
+      s[i] = e;
+      rs += e;
+    }
+    l_run = l_run * alpha + rs;
+    m_run = m_new;
+#pragma unroll
+    for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) o_acc[db][i] *= alpha;
+#pragma unroll
+    for (int w = 0; w < 2; ++w) {
+      float pf[8];
+#pragma unroll
+      for (int jj = 0; jj < 8; ++jj) pf[jj] = s[w * 8 + jj];
+      const vec8 pb = pack8<T>(pf);
+#pragma unroll
+      for (int db = 0; db < D / 32; ++db) {
+        const vec8 av = lds_read_operand_tr<T>(Vt[buf], VS, w * 16, db * 32);
+        o_acc[db] = Traits<T>::mfma(av, pb, o_acc[db]);
+      }
+    }
+    if (has_next) {
+      store_v(Vt[buf ^ 1]);
+#pragma unroll
+      for (int ks = 0; ks < D / 16; ++ks) kc[ks] = kn[ks];
+    }
+    buf ^= 1;
+  }
+
+  // ---- merge the four waves' partials through LDS (each wave writes into its own region) ----
+  const float l_wave = l_run + partner32(l_run);
+  float *Ow = reinterpret_cast<float *>(lds[wave]);  // [D][32]
+  float *MLw = Ow + D * 32;                          // [2][32]
+#pragma unroll
+  for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) Ow[(db * 32 + (i >> 2) * 8 + g * 4 + (i & 3)) * 32 + r32] = o_acc[db][i];
+  if (g == 0) { MLw[r32] = m_run; MLw[32 + r32] = l_wave; }
+  __syncthreads();
+
+  const int n = tid & 31, slice = tid >> 5;  // eight slices of D / 8 output elements per column
+  float mw[kDecWaves], wgt[kDecWaves], m_all = -INFINITY, l_all = 0.f;
+#pragma unroll
+  for (int w = 0; w < kDecWaves; ++w) {
+    mw[w] = reinterpret_cast<const float *>(lds[w])[D * 32 + n];
+    m_all = fmaxf(m_all, mw[w]);
+  }
+  const float m_ref = m_all == -INFINITY ? 0.f : m_all;
+#pragma unroll
+  for (int w = 0; w < kDecWaves; ++w) {
+    wgt[w] = exp2_fast((mw[w] - m_ref) * c);  // 0 for a wave that saw no key
+    l_all += wgt[w] * reinterpret_cast<const float *>(lds[w])[D * 32 + 32 + n];
+  }
+  const bool out_ok = n < group * p.sq;
+  const int oi = out_ok ? n % p.sq : 0, oh = hk * group + (out_ok ? n / p.sq : 0);
+  const bool final_pass = a.o_part == nullptr;
+  const bool empty = l_all == 0.f || l_all != l_all;
+  const float inv = final_pass ? (empty ? 1.f : 1.f / l_all) : 1.f;
+  T *og = static_cast<T *>(p.o_w) + bi * p.o_bs + (int64_t)oi * p.o_rs + oh * p.o_hs;
+  const int64_t prow = (((int64_t)split * p.b + bi) * p.h + oh) * p.sq + oi;
+#pragma unroll
+  for (int x = 0; x < D / 8; ++x) {
+    const int dcol = slice * (D / 8) + x;
+    float acc = 0.f;
+#pragma unroll
+    for (int w = 0; w < kDecWaves; ++w) acc += wgt[w] * reinterpret_cast<const float *>(lds[w])[dcol * 32 + n];
+    if (out_ok) {
+      if (final_pass) og[dcol] = (T)(acc * inv);
+      else a.o_part[prow * D + dcol] = acc;
+    }
+  }
+  if (out_ok && slice == 0) {
+    if (final_pass) p.lse[((int64_t)bi * p.h + oh) * p.sq + oi] = empty ? INFINITY : m_all * p.scale + log2_fast(l_all) * kLn2;
+    else { a.ml_part[prow * 2] = m_all; a.ml_part[prow * 2 + 1] = l_all; }
+  }
+}
+
+// merges the chunks' partials of one (batch, head, query row) per workgroup, one thread per output element
+template <typename T, int D>
+__global__ void __launch_bounds__(D) decode_merge_kernel(const Params p, const DecodeArgs a) {
+  const int64_t row = blockIdx.x;  // (batch * h + head) * sq + query row
+  const int64_t rows = (int64_t)p.b * p.h * p.sq;
+  const int dcol = threadIdx.x;
+  float m_all = -INFINITY;
+  for (int s = 0; s < a.n_splits; ++s) m_all = fmaxf(m_all, a.ml_part[(s * rows + row) * 2]);
+  const float m_ref = m_all == -INFINITY ? 0.f : m_all;
+  float l_all = 0.f, acc = 0.f;
+  for (int s = 0; s < a.n_splits; ++s) {
+    const float w = exp2_fast((a.ml_part[(s * rows + row) * 2] - m_ref) * p.scale_log2);
+    l_all += w * a.ml_part[(s * rows + row) * 2 + 1];
+    acc += w * a.o_part[(s * rows + row) * D + dcol];
+  }
+  const bool empty = l_all == 0.f || l_all != l_all;
+  const int qi = (int)(row % p.sq), hq = (int)((row / p.sq) % p.h), bi = (int)(row / ((int64_t)p.sq * p.h));
+  T *og = static_cast<T *>(p.o_w) + bi * p.o_bs + (int64_t)qi * p.o_rs + hq * p.o_hs;
+  og[dcol] = (T)(empty ? 0.f : acc / l_all);
+  if (dcol == 0) p.lse[row] = empty ? INFINITY : m_all * p.scale + log2_fast(l_all) * kLn2;
+}
+
+template <typename T, int D>
+hipError_t decode_td(const Params &p, hipStream_t stream) {
+  const int base = p.b * p.h_k;
+  // enough workgroups for two per CU, but at least 512 keys per chunk
+  int n_splits = (2 * 256 + base - 1) / base;
+  n_splits = max(1, min(n_splits, min(64, p.sk / 512)));
+  DecodeArgs a{};
+  a.n_splits = n_splits;
+  a.chunk = ((p.sk + n_splits - 1) / n_splits + kUnit * kDecWaves - 1) / (kUnit * kDecWaves) * (kUnit * kDecWaves);
+  void *ws = nullptr;
+  const size_t rows = (size_t)p.b * p.h * p.sq;
+  if (n_splits > 1) {
+    if (hipMallocAsync(&ws, (size_t)n_splits * rows * (D + 2) * sizeof(float), stream) != hipSuccess) {
+      (void)hipGetLastError();  // no workspace: one chunk per (batch, key/value head)
+      ws = nullptr;
+      a.n_splits = 1;
+      a.chunk = (p.sk + kUnit - 1) / kUnit * kUnit;
+    } else {
+      a.o_part = static_cast<float *>(ws);
+      a.ml_part = a.o_part + (size_t)n_splits * rows * D;
+    }
+  }
+  decode_kernel<T, D><<<dim3((unsigned)(base * a.n_splits)), dim3(kDecWaves * 64), 0, stream>>>(p, a);
+  hipError_t e = hipGetLastError();
+  if (ws) {
+    if (e == hipSuccess) {
+      decode_merge_kernel<T, D><<<dim3((unsigned)rows), dim3(D), 0, stream>>>(p, a);
+      e = hipGetLastError();
+    }
+    const hipError_t f = hipFreeAsync(ws, stream);
+    if (e == hipSuccess) e = f;
+  }
+  return e;
+}
+
+}  // namespace
+
+bool decode_eligible(const Params &p) {
+  return (p.d == 64 || p.d == 128) && p.sq > 0 && (p.h / p.h_k) * p.sq <= 32 && p.sk >= 1 && !p.drop;
+}
+
+hipError_t launch_decode(Params &p, int dtype, hipStream_t stream) {
+  if (p.b * p.h == 0 || p.sq == 0) return hipSuccess;
+  if (p.d == 64) return dtype == 1 ? decode_td<_Float16, 64>(p, stream) : decode_td<__bf16, 64>(p, stream);
+  return dtype == 1 ? decode_td<_Float16, 128>(p, stream) : decode_td<__bf16, 128>(p, stream);
+}
+
+}  // namespace fa

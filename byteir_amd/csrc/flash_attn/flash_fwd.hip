@@ -388,6 +388,7 @@ hipError_t launch_append_kv(const Params &p, int dtype, hipStream_t stream) {
 hipError_t launch_fwd(Params &p, int dtype, hipStream_t stream) {
   p.xcd_remap = ((p.b * p.h) % 8 == 0) ? (p.wr >= 0 ? 2 : 1) : 0;
   if (p.b * p.h == 0 || p.sq == 0) return hipSuccess;
+  if (decode_eligible(p)) return launch_decode(p, dtype, stream);
   if (p.drop || (p.d != 32 && p.d != 64 && p.d != 128)) return launch_fwd_anyd(p, dtype, stream);
   return dtype == 1 ? launch_fwd_t<_Float16>(p, stream) : launch_fwd_t<__bf16>(p, stream);
 }

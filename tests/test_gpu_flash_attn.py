@@ -74,6 +74,13 @@ CASES = [
     (1, 300, 300, 2, 2, 64, (64, 0)),      # sliding window, left-bounded causal
     (1, 300, 260, 2, 2, 128, (40, 30)),    # local window both sides
     (3, 1, 50, 1, 1, 32, (-1, -1)),        # single query row
+    # few query rows: the decode kernel (all query heads of a key/value head in one score tile,
+    # keys split over waves and, for long sequences, over workgroups)
+    (2, 1, 1000, 8, 2, 128, (-1, -1)),
+    (1, 4, 3000, 8, 8, 64, (-1, 0)),
+    (1, 8, 700, 4, 1, 128, (100, 0)),      # 32 columns, sliding window
+    (1, 2, 9000, 2, 2, 64, (-1, -1)),      # several chunks per head
+    (3, 1, 33, 4, 4, 64, (-1, 0)),
     # head dimensions without a tuned kernel: every multiple of 8 up to 256 is accepted
     (1, 150, 150, 2, 2, 8, (-1, 0)),
     (1, 1, 40, 2, 2, 16, (-1, -1)),
@@ -255,6 +262,8 @@ KV_CASES = [
     (4, 16, 2, 2, 32, 1024, 16, [1000, 3, 500, 64], (-1, 0), True),
     (2, 3, 4, 4, 64, 130, 0, [130, 1], (-1, -1), False),        # no append: read-only cache
     (2, 2, 4, 1, 64, 520, 2, [518, 300], (64, 0), True),        # sliding window, MQA
+    (2, 1, 8, 2, 128, 5000, 1, [4999, 2500], (-1, -1), True),   # long cache: several chunks per head
+    (3, 2, 16, 2, 64, 2100, 2, [0, 2098, 700], (-1, 0), True),
     (2, 3, 4, 2, 96, 260, 3, [250, 17], (-1, 0), True),         # head dimensions without a tuned kernel
     (1, 1, 2, 2, 256, 300, 1, [299], (-1, -1), True),
     (2, 4, 2, 2, 80, 128, 0, [128, 5], (-1, -1), False),
