@@ -151,7 +151,9 @@ def flash_attn_bwd_buffers(q, k, v):
     (dq, dk, dv, d_softmax, dq_accum, rng_state)."""
     b, sq, h, d = q.shape
     sq_r, d_r = round_up(sq, 128), round_up(d, 32)
-    return (torch.empty_like(q), torch.empty_like(k), torch.empty_like(v),
+    like = lambda t: torch.empty_strided(t.shape, t.stride(), dtype=t.dtype, device=t.device)
+    # dq, dk, dv are addressed with the strides of q, k, v (flash_api.cu:377-389)
+    return (like(q), like(k), like(v),
             torch.empty((b, h, sq_r), dtype=torch.float32, device=q.device),
             torch.empty((b, sq_r, h, d_r), dtype=torch.float32, device=q.device),
             torch.zeros(2, dtype=torch.int64, device=q.device))

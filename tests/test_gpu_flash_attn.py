@@ -151,6 +151,57 @@ def test_backward_matches_oracle(case, code):
         assert err <= ATOL, (name, float(err))
 
 
+STRIDED_CASES = [
+    # layout, b, sq, sk, h, h_k, d, window
+    ("packed_qkv", 2, 192, 192, 4, 4, 64, (-1, 0)),       # q, k, v are slices of one [b, s, 3, h, d] tensor
+    ("packed_qkv", 1, 130, 130, 2, 2, 96, (-1, -1)),
+    ("bhsd", 2, 160, 224, 4, 4, 128, (-1, 0)),            # [b, h, s, d] storage viewed as [b, s, h, d]
+    ("bhsd", 1, 100, 300, 3, 3, 32, (20, 5)),
+    ("bhsd", 2, 2, 1500, 8, 2, 128, (-1, -1)),            # decode-shaped, grouped heads (forward only)
+]
+
+
+@pytest.mark.parametrize("code", [oracle.F16, oracle.BF16])
+@pytest.mark.parametrize("case", STRIDED_CASES)
+def test_strided_tensors(case, code):
+    """The blob carries batch, row and head strides; the tensors need not be dense."""
+    from byteir_amd import ops
+    layout, b, sq, sk, h, h_k, d, window = case
+    q, k, v, do = make_inputs((b, sq, sk, h, h_k, d, window), code, seed=sum(case[1:7]) + 3)
+    scale = 1.0 / np.sqrt(d)
+    dq_, dk_, dv_, do_ = (dev(t) for t in (q, k, v, do))
+    if layout == "packed_qkv":
+        pk = torch.empty((b, sq, 3, h, d), dtype=dq_.dtype, device="cuda")
+        pk[:, :, 0], pk[:, :, 1], pk[:, :, 2] = dq_, dk_, dv_
+        sq_, sk_, sv_ = pk[:, :, 0], pk[:, :, 1], pk[:, :, 2]
+        o_buf = torch.empty((b, sq, 2, h, d), dtype=dq_.dtype, device="cuda")[:, :, 1]
+        do_s = torch.zeros((b, sq, 2, h, d), dtype=dq_.dtype, device="cuda")[:, :, 1]
+    else:
+        tr = lambda x: x.permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3)
+        sq_, sk_, sv_ = tr(dq_), tr(dk_), tr(dv_)
+        o_buf = tr(torch.empty_like(dq_))
+        do_s = tr(torch.zeros_like(dq_))
+    do_s.copy_(do_)
+    assert not sq_.is_contiguous() and o_buf.stride() == do_s.stride()
+    lse = torch.empty((b, h, sq), dtype=torch.float32, device="cuda")
+    rng = torch.zeros(2, dtype=torch.int64, device="cuda")
+    ops.flash_attn_fwd(sq_, sk_, sv_, scale, window, out=(o_buf, lse, rng))
+    o_dense, lse_dense = ops.flash_attn_fwd(dq_, dk_, dv_, scale, window)
+    assert torch.equal(o_buf, o_dense) and torch.equal(lse, lse_dense)   # same kernel, same arithmetic
+    _, _, o32 = oracle.flash_fwd(q, k, v, scale, window, round_p=False)
+    assert np.abs(oracle.to_f32(host(o_buf.contiguous())) - o32).max() <= ATOL
+    if h != h_k:
+        return
+    dq, dk, dv = ops.flash_attn_bwd(do_s, sq_, sk_, sv_, o_buf, lse, scale, window)
+    assert dq.stride() == sq_.stride() and dk.stride() == sk_.stride()
+    gq, gk, gv = ops.flash_attn_bwd(do_, dq_, dk_, dv_, o_dense, lse_dense, scale, window)
+    assert torch.equal(dq, gq) and torch.equal(dk, gk) and torch.equal(dv, gv)
+    rq, rk, rv, _ = oracle.flash_bwd(do, q, k, v, host(o_dense), host(lse_dense), scale, window, round_p=False)
+    for name, got, want in (("dq", dq, rq), ("dk", dk, rk), ("dv", dv, rv)):
+        err = np.abs(oracle.to_f32(host(got.contiguous())) - oracle.to_f32(want)).max()
+        assert err <= ATOL, (name, float(err))
+
+
 def test_unsupported_arguments_are_reported_not_run():
     import ctypes
     from byteir_amd import _lib, ops
