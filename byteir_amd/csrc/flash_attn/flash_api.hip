@@ -216,7 +216,8 @@ int flash_attn_kvcache_checked(void **tensors, const void *extra_args, int dtype
     p.seqlen_knew = (int)k.seqlen_knew;
     p.knew_bs = k.knew_bs; p.vnew_bs = k.vnew_bs; p.knew_rs = k.knew_rs; p.vnew_rs = k.vnew_rs;
     p.knew_hs = k.knew_hs; p.vnew_hs = k.vnew_hs;
-    if (hipError_t e = fa::launch_append_kv(p, dtype, stream)) return e;
+    if (fa::decode_can_append(p)) p.fuse_append = 1;
+    else if (hipError_t e = fa::launch_append_kv(p, dtype, stream)) return e;
   }
   // without seqlens_k every batch attends to all seqlen_k cache rows (BlockInfo, block_info.h:27-37)
   return fa::launch_fwd(p, dtype, stream);

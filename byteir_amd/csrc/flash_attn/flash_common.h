@@ -161,6 +161,7 @@ struct Params {
   int seqlen_knew;
   const void *k_new, *v_new;
   int64_t knew_bs, vnew_bs, knew_rs, vnew_rs, knew_hs, vnew_hs;
+  int fuse_append;                    // 1: the decode kernel appends k_new / v_new itself
   // dropout (forward and backward calls): rng_state = {seed, offset} in device memory,
   // keep probability, its reciprocal and its 8-bit threshold floor(p_keep * 255)
   const uint64_t *rng_state;
@@ -189,6 +190,7 @@ hipError_t launch_bwd_anyd(Params &p, int dtype, hipStream_t stream);
 // A few query rows against a long key sequence (flash_decode.hip): all query heads of a
 // key/value head times all query rows must fit the 32 columns of one score tile.
 bool decode_eligible(const Params &p);
+bool decode_can_append(const Params &p);  // then set p.fuse_append and skip launch_append_kv
 hipError_t launch_decode(Params &p, int dtype, hipStream_t stream);
 
 }  // namespace fa

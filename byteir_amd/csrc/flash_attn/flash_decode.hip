@@ -84,15 +84,30 @@ __global__ void __launch_bounds__(kDecWaves * 64, 2) decode_kernel(const Params 
   uint4 kn[NPV], vn[NPV];
   const int v_c = lane % CPR, v_r = lane / CPR;
   typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+  // Appending (p.fuse_append): rows [new0, new0 + seqlen_knew) of this batch come from k_new /
+  // v_new instead of the cache and are written to the cache by the one lane that loads them
+  // (reference: the Append_KV branch of compute_attn_1rowblock_splitkv, flash_fwd_kernel.h:660-740).
+  const int new0 = p.fuse_append ? p.seqlens_k[bi] : 0x7fffffff;
+  const T *kng = p.fuse_append ? static_cast<const T *>(p.k_new) + bi * p.knew_bs + hk * p.knew_hs : nullptr;
+  const T *vng = p.fuse_append ? static_cast<const T *>(p.v_new) + bi * p.vnew_bs + hk * p.vnew_hs : nullptr;
   auto load_unit = [&](int j) {  // unit j of the chunk into the staging registers
 #pragma unroll
     for (int s = 0; s < NPV; ++s) {
       const int key = c0 + j * kUnit + s * RPP + v_r;
       if (key < c1) {
-        const u32x4 a = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(kg + (int64_t)key * p.k_rs + v_c * 8));
-        const u32x4 b = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(vg + (int64_t)key * p.v_rs + v_c * 8));
+        const bool fresh = key >= new0;
+        T *kc_row = const_cast<T *>(kg) + (int64_t)key * p.k_rs + v_c * 8;
+        T *vc_row = const_cast<T *>(vg) + (int64_t)key * p.v_rs + v_c * 8;
+        const T *ks_row = fresh ? kng + (int64_t)(key - new0) * p.knew_rs + v_c * 8 : kc_row;
+        const T *vs_row = fresh ? vng + (int64_t)(key - new0) * p.vnew_rs + v_c * 8 : vc_row;
+        const u32x4 a = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(ks_row));
+        const u32x4 b = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(vs_row));
         kn[s] = uint4{a.x, a.y, a.z, a.w};
         vn[s] = uint4{b.x, b.y, b.z, b.w};
+        if (fresh) {
+          *reinterpret_cast<uint4 *>(kc_row) = kn[s];
+          *reinterpret_cast<uint4 *>(vc_row) = vn[s];
+        }
       } else {  // zero rows: 0 * finite stays finite in P V
         kn[s] = uint4{0, 0, 0, 0};
         vn[s] = uint4{0, 0, 0, 0};
@@ -214,21 +229,31 @@ __global__ void __launch_bounds__(kDecWaves * 64, 2) decode_kernel(const Params 
   }
 }
 
-// merges the chunks' partials of one (batch, head, query row) per workgroup, one thread per output element
+// merges the chunks' partials of one (batch, head, query row) per workgroup, one thread per
+// output element; n_splits <= 64, so lane s of every wave takes chunk s for the statistics
 template <typename T, int D>
 __global__ void __launch_bounds__(D) decode_merge_kernel(const Params p, const DecodeArgs a) {
+  __shared__ float wgt[64];
   const int64_t row = blockIdx.x;  // (batch * h + head) * sq + query row
   const int64_t rows = (int64_t)p.b * p.h * p.sq;
-  const int dcol = threadIdx.x;
-  float m_all = -INFINITY;
-  for (int s = 0; s < a.n_splits; ++s) m_all = fmaxf(m_all, a.ml_part[(s * rows + row) * 2]);
+  const int dcol = threadIdx.x, lane = threadIdx.x & 63;
+  const bool has = lane < a.n_splits;
+  const float m_s = has ? a.ml_part[(lane * rows + row) * 2] : -INFINITY;
+  const float l_s = has ? a.ml_part[(lane * rows + row) * 2 + 1] : 0.f;
+  float m_all = m_s;
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) m_all = fmaxf(m_all, __shfl_xor(m_all, off, 64));
   const float m_ref = m_all == -INFINITY ? 0.f : m_all;
-  float l_all = 0.f, acc = 0.f;
-  for (int s = 0; s < a.n_splits; ++s) {
-    const float w = exp2_fast((a.ml_part[(s * rows + row) * 2] - m_ref) * p.scale_log2);
-    l_all += w * a.ml_part[(s * rows + row) * 2 + 1];
-    acc += w * a.o_part[(s * rows + row) * D + dcol];
-  }
+  const float w_s = exp2_fast((m_s - m_ref) * p.scale_log2);  // 0 for a chunk that saw no key
+  float l_all = w_s * l_s;
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) l_all += __shfl_xor(l_all, off, 64);
+  if (threadIdx.x < 64) wgt[threadIdx.x] = w_s;
+  __syncthreads();
+  float acc = 0.f;
+  const float *op = a.o_part + row * D + dcol;
+#pragma unroll 8
+  for (int s = 0; s < a.n_splits; ++s) acc += wgt[s] * op[s * rows * D];
   const bool empty = l_all == 0.f || l_all != l_all;
   const int qi = (int)(row % p.sq), hq = (int)((row / p.sq) % p.h), bi = (int)(row / ((int64_t)p.sq * p.h));
   T *og = static_cast<T *>(p.o_w) + bi * p.o_bs + (int64_t)qi * p.o_rs + hq * p.o_hs;
@@ -275,6 +300,12 @@ hipError_t decode_td(const Params &p, hipStream_t stream) {
 
 bool decode_eligible(const Params &p) {
   return (p.d == 64 || p.d == 128) && p.sq > 0 && (p.h / p.h_k) * p.sq <= 32 && p.sk >= 1 && !p.drop;
+}
+
+// The decode kernel can do the append itself when every appended row is certain to be loaded by
+// it: no left window (rows below the window are never fetched).
+bool decode_can_append(const Params &p) {
+  return decode_eligible(p) && p.k_new && p.v_new && p.seqlens_k && p.seqlen_knew > 0 && p.wl < 0;
 }
 
 hipError_t launch_decode(Params &p, int dtype, hipStream_t stream) {
