@@ -81,6 +81,9 @@ CASES = [
     (1, 8, 700, 4, 1, 128, (100, 0)),      # 32 columns, sliding window
     (1, 2, 9000, 2, 2, 64, (-1, -1)),      # several chunks per head
     (3, 1, 33, 4, 4, 64, (-1, 0)),
+    (1, 32, 40, 2, 2, 64, (-1, 0)),        # all 32 columns are rows of one head
+    (2, 7, 5, 4, 1, 128, (-1, 0)),         # causal with sq > sk: leading rows keep no key
+    (1, 3, 600, 6, 2, 128, (-1, 5)),       # right window only
     # head dimensions without a tuned kernel: every multiple of 8 up to 256 is accepted
     (1, 150, 150, 2, 2, 8, (-1, 0)),
     (1, 1, 40, 2, 2, 16, (-1, -1)),
