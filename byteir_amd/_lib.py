@@ -63,6 +63,7 @@ def kernels():
         L.brt_rocm_reduce.argtypes = [i32, i32, vp, vp, sz, sz, sz, vp, sz, vp]
         L.brt_rocm_reduce_ex.argtypes = [i32, i32, vp, vp, sz, sz, sz, vp, sz, vp, vp]
         L.brt_rocm_softmax.argtypes = [i32, vp, vp, sz, sz, vp]
+        L.brt_rocm_softmax_axis.argtypes = [i32, vp, vp, sz, sz, sz, vp]
         _kernels = L
     return _kernels
 

@@ -155,24 +155,24 @@ public:
     BRT_ENFORCE(!s.empty(), "softmax of a rank-0 tensor");
     int64_t axis = acc.HasAttr("axis") ? acc.GetAttrAsInt("axis") : (int64_t)s.size() - 1;
     if (axis < 0) axis += (int64_t)s.size();
-    BRT_ENFORCE(axis == (int64_t)s.size() - 1, "softmax is implemented along the last axis only");
+    BRT_ENFORCE(axis >= 0 && axis < (int64_t)s.size(), "softmax axis out of range");
     switch (acc.GetArgDTypeEnum(0)) {
     case DTypeEnum::Float32: dtype_ = BRT_ROCM_F32; break;
     case DTypeEnum::Float16: dtype_ = BRT_ROCM_F16; break;
     case DTypeEnum::BFloat16: dtype_ = BRT_ROCM_BF16; break;
     default: BRT_THROW("softmax element type must be f32, f16 or bf16");
     }
-    cols_ = (size_t)s.back();
-    rows_ = cols_ ? (size_t)LinearizedShape(s) / cols_ : 0;
+    a_ = b_ = c_ = 1;
+    for (int64_t i = 0; i < (int64_t)s.size(); ++i) (i < axis ? a_ : i == axis ? b_ : c_) *= (size_t)s[i];
   }
   common::Status RunImpl(const ExecutionContext &ctx) override {
     OpAccessor acc(info_, ctx.exec_frame);
-    return HipStatus(brt_rocm_softmax(dtype_, acc.GetArgAsyncValueRef(0), acc.GetArgAsyncValueRef(1), rows_, cols_, StreamOf(ctx)), "softmax");
+    return HipStatus(brt_rocm_softmax_axis(dtype_, acc.GetArgAsyncValueRef(0), acc.GetArgAsyncValueRef(1), a_, b_, c_, StreamOf(ctx)), "softmax");
   }
 
 private:
   int dtype_ = 0;
-  size_t rows_ = 0, cols_ = 0;
+  size_t a_ = 1, b_ = 1, c_ = 1;  // softmax over the middle axis of [a, b, c]
 };
 
 // ---- custom -----------------------------------------------------------------------------------------------

@@ -1,6 +1,10 @@
 // Fused row softmax for gfx950: y = exp(x - max(x)) / sum(exp(x - max(x))) over the last
 // axis of a dense [rows, cols] tensor, float internals, one rounding at the store.
 //
+// (A softmax over an inner axis, [A, B, C] over B with C > 1, takes softmax_inner_kernel: lanes
+// along the contiguous C axis, one online max/sum pass over B and a second pass that re-reads
+// the tile -- mostly from L2 -- and writes.)
+//
 // softmax_wave_kernel keeps a whole row in the registers of one wave (NV 128-bit vectors per
 // lane), so a row is read from HBM once and written once; max and sum are wave64 shuffle
 // trees.  Rows too long for registers, or not 16-byte aligned, take softmax_block_kernel,
@@ -141,6 +145,45 @@ softmax_block_kernel(const T *in, T *out, uint64_t cols) {
     y[j] = Elem<T>::make(fast_exp(Elem<T>::get(x[j]) - m) * inv);
 }
 
+// Softmax over the middle axis of a dense [A, B, C] tensor: one thread per (a, c) column, lanes
+// along c.  Pass 1 keeps a running maximum and a sum rescaled on the fly (so the column is read
+// once for both), pass 2 re-reads and writes.
+template <typename T>
+__global__ void __launch_bounds__(kBlock)
+softmax_inner_kernel(const T *__restrict__ in, T *__restrict__ out, uint64_t B, uint64_t C) {
+  const uint64_t c = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (c >= C) return;
+  const T *x = in + (uint64_t)blockIdx.y * B * C + c;
+  T *y = out + (uint64_t)blockIdx.y * B * C + c;
+  float m = -INFINITY, s = 0.f;
+  for (uint64_t b = 0; b < B; ++b) {
+    const float v = Elem<T>::get(x[b * C]);
+    const float m_new = fmaxf(m, v);
+    // exp(-inf - -inf) would be NaN: a column that is -inf so far keeps s = 0 (if it stays
+    // -inf to the end, pass 2 produces the NaN the two-pass definition gives)
+    s = m_new == -INFINITY ? 0.f : s * fast_exp(m - m_new) + fast_exp(v - m_new);
+    m = m_new;
+  }
+  const float inv = 1.0f / s;
+  for (uint64_t b = 0; b < B; ++b) y[b * C] = Elem<T>::make(fast_exp(Elem<T>::get(x[b * C]) - m) * inv);
+}
+
+template <typename T>
+hipError_t run_inner(const T *in, T *out, uint64_t A, uint64_t B, uint64_t C, hipStream_t stream) {
+  const uint64_t bx = (C + kBlock - 1) / kBlock;
+  if (bx > 0x7fffffffull || A > 65535) {
+    // the grid's y extent is 16 bits: fold batches into several launches
+    for (uint64_t a0 = 0; a0 < A; a0 += 65535) {
+      const uint64_t na = A - a0 < 65535 ? A - a0 : 65535;
+      if (bx > 0x7fffffffull) return hipErrorInvalidValue;
+      softmax_inner_kernel<T><<<dim3((unsigned)bx, (unsigned)na), dim3(kBlock), 0, stream>>>(in + a0 * B * C, out + a0 * B * C, B, C);
+    }
+    return hipGetLastError();
+  }
+  softmax_inner_kernel<T><<<dim3((unsigned)bx, (unsigned)A), dim3(kBlock), 0, stream>>>(in, out, B, C);
+  return hipGetLastError();
+}
+
 template <typename T>
 hipError_t run(const T *in, T *out, uint64_t rows, uint64_t cols, hipStream_t stream) {
   constexpr int EPV = Elem<T>::EPV;
@@ -164,6 +207,24 @@ hipError_t run(const T *in, T *out, uint64_t rows, uint64_t cols, hipStream_t st
 }
 
 }  // namespace
+
+extern "C" int brt_rocm_softmax_axis(int dtype, const void *input, void *output, size_t A, size_t B,
+                                     size_t C, void *stream_) {
+  if (C == 1) return brt_rocm_softmax(dtype, input, output, A, B, stream_);
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  if (A == 0 || B == 0 || C == 0) return hipSuccess;
+  if (!input || !output) return hipErrorInvalidValue;
+  switch (dtype) {
+  case BRT_ROCM_F32:
+    return run_inner(static_cast<const float *>(input), static_cast<float *>(output), A, B, C, stream);
+  case BRT_ROCM_F16:
+    return run_inner(static_cast<const __half *>(input), static_cast<__half *>(output), A, B, C, stream);
+  case BRT_ROCM_BF16:
+    return run_inner(static_cast<const __bf16 *>(input), static_cast<__bf16 *>(output), A, B, C, stream);
+  default:
+    return hipErrorInvalidValue;
+  }
+}
 
 extern "C" int brt_rocm_softmax(int dtype, const void *input, void *output, size_t rows,
                                 size_t cols, void *stream_) {

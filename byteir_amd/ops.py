@@ -84,14 +84,18 @@ def reduce(op, x, dims, stream=None):
     return reduce_abc(op, x, out, A, B, C, stream=stream)
 
 
-def softmax(x, out=None, stream=None):
-    """byteir.softmax over the last axis."""
+def softmax(x, out=None, stream=None, axis=-1):
+    """byteir.softmax over `axis` of a dense tensor (the last one by default)."""
     if out is None:
         out = torch.empty_like(x)
-    cols = x.shape[-1]
-    rows = x.numel() // cols if cols else 0
-    _lib.check(_lib.kernels().brt_rocm_softmax(_DT[x.dtype], _dev(x), _dev(out), rows, cols,
-                                               _stream(stream)), "brt_rocm_softmax")
+    axis = axis % x.dim()
+    a, b, c = 1, x.shape[axis], 1
+    for n in x.shape[:axis]:
+        a *= n
+    for n in x.shape[axis + 1:]:
+        c *= n
+    _lib.check(_lib.kernels().brt_rocm_softmax_axis(_DT[x.dtype], _dev(x), _dev(out), a, b, c,
+                                                    _stream(stream)), "brt_rocm_softmax_axis")
     return out
 
 

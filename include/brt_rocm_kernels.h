@@ -101,6 +101,13 @@ int brt_rocm_reduce_ex(int op, int dtype, const void *input, void *output, size_
 int brt_rocm_softmax(int dtype, const void *input, void *output, size_t rows, size_t cols,
                      void *stream);
 
+/* The same over the middle axis of a dense row-major [A, B, C] tensor (byteir.softmax with an
+ * `axis` that is not the last one, compiler/lib/Conversion/ToLinalg/HloToLinalg.cpp:393-467:
+ * A = product of the dimensions before the axis, C = product of those after).  C == 1 is the
+ * row softmax above. */
+int brt_rocm_softmax_axis(int dtype, const void *input, void *output, size_t A, size_t B, size_t C,
+                          void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -201,8 +201,11 @@ def reduce_sum_f64(x, A, B, C):
 
 
 # ---- softmax ------------------------------------------------------------------------
-def softmax(x):
-    """Row softmax over the last axis; x is f32 / f16 / bf16-bits; same storage out."""
+def softmax(x, axis=-1):
+    """Softmax over `axis` (the last one by default); x is f32 / f16 / bf16-bits; same storage
+    out.  Another axis is moved last, reduced by the same C routine and moved back."""
+    if axis % x.ndim != x.ndim - 1:
+        return np.ascontiguousarray(np.moveaxis(softmax(np.moveaxis(x, axis, -1)), -1, axis))
     x = np.ascontiguousarray(x)
     cols = x.shape[-1]
     rows = x.size // cols if cols else 0

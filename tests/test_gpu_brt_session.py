@@ -124,14 +124,14 @@ def test_softmax_through_backend(dtype, code):
     reference's own softmax test shapes."""
     import tempfile
     from byteir_amd.brt import BRTBackend
-    for shape, axis in (([10, 128], 1), ([2, 3, 256, 256], -1)):
+    for shape, axis in (([10, 128], 1), ([2, 3, 256, 256], -1), ([4, 50, 96], 1)):
         with tempfile.NamedTemporaryFile("w", suffix=".mlir", delete=False) as f:
             f.write(softmax_module("cuda", shape, dtype, axis))
         be = BRTBackend("cuda", f.name)
         x32 = (np.random.default_rng(9).standard_normal(shape) * 2).astype(np.float32)
         xs = oracle.from_f32(x32, code)
         (y,) = be.run([dev(xs)])
-        got, want = oracle.to_f32(host(y)), oracle.to_f32(oracle.softmax(xs))
+        got, want = oracle.to_f32(host(y)), oracle.to_f32(oracle.softmax(xs, axis=axis))
         rel = {oracle.F32: 1e-5, oracle.F16: 2.0 ** -10, oracle.BF16: 2.0 ** -7}[code]
         assert np.all(np.abs(got - want) <= rel * np.abs(want) + 6e-8)
         ms = be.profile_with_outputs([dev(xs)], [y], warmup=2, iters=3)

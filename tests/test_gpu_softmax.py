@@ -38,6 +38,34 @@ def test_softmax_matches_oracle(shape, code):
     run_case(shape, code)
 
 
+@pytest.mark.parametrize("code", [oracle.F32, oracle.F16, oracle.BF16])
+@pytest.mark.parametrize("shape,axis", [((4, 33, 70), 1), ((2, 3, 5, 7), 2), ((129, 1000), 0), ((3, 260, 2), 1),
+                                        ((2, 1, 300), 1), ((5, 64, 64), -2)])
+def test_softmax_over_an_inner_axis(shape, axis, code):
+    from byteir_amd import ops
+    x32 = (np.random.default_rng(sum(shape)).standard_normal(shape) * 2.0).astype(np.float32)
+    xs = oracle.from_f32(x32, code)
+    got = oracle.to_f32(host(ops.softmax(dev(xs), axis=axis)))
+    want = oracle.to_f32(oracle.softmax(xs, axis=axis))
+    rel, ab = TOL[code]
+    assert np.all(np.abs(got - want) <= rel * np.abs(want) + ab), float(np.abs(got - want).max())
+    np.testing.assert_allclose(got.sum(axis=axis), 1.0, atol=2e-2 if code != oracle.F32 else 1e-5)
+
+
+def test_softmax_inner_axis_with_infinities():
+    from byteir_amd import ops
+    x = torch.randn((2, 6, 130), device="cuda")
+    x[0, :3, 5] = -float("inf")          # the column starts with -inf values
+    x[1, :, 7] = -float("inf")           # a column of -inf only: NaN, as exp(-inf - -inf) / 0 in the reference lowering
+    x[1, 2, 9] = float("nan")
+    y = host(ops.softmax(x, axis=1))
+    want = oracle.softmax(host(x), axis=1)
+    assert np.array_equal(np.isnan(y), np.isnan(want))
+    ok = ~np.isnan(want)
+    assert np.abs(y[ok] - want[ok]).max() <= 1e-5
+    assert np.all(y[0, :3, 5] == 0)
+
+
 def test_softmax_properties_f32():
     from byteir_amd import ops
     x = dev((np.random.default_rng(3).standard_normal((256, 4096)) * 2).astype(np.float32))
