@@ -450,3 +450,45 @@ def test_dropout_without_rng_state_is_reported():
     buf = ctypes.create_string_buffer(blob, len(blob))
     assert L.flash_attn_fwd_checked(arr, ctypes.cast(buf, ctypes.c_void_p), 1, None) == -1
     assert b"p_dropout" in L.flash_attn_last_error()
+
+
+def test_decode_call_inside_a_hip_graph():
+    """Serving stacks capture the decode step in a graph.  The call appends, splits the keys over
+    workgroups (stream-ordered scratch) and merges; replays with fresh cache contents and
+    lengths, with eager work in between, must match the eager result every time."""
+    from byteir_amd import ops
+    b, h, h_k, d, cap = 2, 8, 2, 128, 6000
+    gen = torch.Generator(device="cuda").manual_seed(7)
+    mk = lambda *s: torch.randn(s, generator=gen, device="cuda").half()
+    q, kc, vc, kn, vn = mk(b, 1, h, d), mk(b, cap, h_k, d), mk(b, cap, h_k, d), mk(b, 1, h_k, d), mk(b, 1, h_k, d)
+    lens = torch.tensor([5000, 3000], dtype=torch.int32, device="cuda")
+    scale = 1.0 / np.sqrt(d)
+    o = torch.empty_like(q)
+    lse = torch.empty((b, h, 1), dtype=torch.float32, device="cuda")
+    L = __import__("byteir_amd._lib", fromlist=["x"]).flash_attn()
+
+    def call(stream):
+        ops._call_custom(L.run_flash_attn_kvcache, [q, kc, vc, kn, vn, lens, o, lse],
+                         ops.pack_flash_kvcache_args(q, kc, vc, kn, vn, o, scale, (-1, -1)), stream)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        call(side)  # warm-up outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        call(side)
+    for step in range(3):
+        q.copy_(mk(b, 1, h, d)); kn.copy_(mk(b, 1, h_k, d)); vn.copy_(mk(b, 1, h_k, d))
+        lens.copy_(torch.tensor([5001 + 7 * step, 3001 + step], dtype=torch.int32, device="cuda"))
+        kc_before, vc_before = kc.clone(), vc.clone()
+        graph.replay()
+        torch.cuda.synchronize()
+        o_graph, lse_graph, kc_graph = o.clone(), lse.clone(), kc.clone()
+        kc.copy_(kc_before); vc.copy_(vc_before)
+        o_eager, lse_eager = ops.flash_attn_kvcache(q, kc, vc, kn, vn, lens, scale, (-1, -1))
+        torch.cuda.synchronize()
+        assert torch.equal(o_graph, o_eager) and torch.equal(lse_graph, lse_eager), step
+        assert torch.equal(kc_graph, kc), step
