@@ -154,6 +154,9 @@ __device__ __forceinline__ void block_of(const Params &p, int n_blocks, bool rev
     const int xcd = L & 7, slot = L >> 3, per_xcd = (p.b * p.h) >> 3;
     bh = (slot % per_xcd) * 8 + xcd;
     blk = slot / per_xcd;
+  } else if (p.xcd_remap == 3) {  // the same order when b*h is not a multiple of the XCD count
+    bh = L % (p.b * p.h);
+    blk = L / (p.b * p.h);
   } else if (p.xcd_remap) {  // consecutive workgroup ids go round-robin over the 8 XCDs
     const int xcd = L & 7, slot = L >> 3;
     bh = (slot / n_blocks) * 8 + xcd;

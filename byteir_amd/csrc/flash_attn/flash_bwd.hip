@@ -138,6 +138,9 @@ __global__ void __launch_bounds__(256, (D <= 64 && KB == 1) ? 2 : 1) dkdv_kernel
       const int xcd = L & 7, slot = L >> 3, per_xcd = (p.b * p.h) >> 3;
       bh = (slot % per_xcd) * 8 + xcd;
       n_block = slot / per_xcd;
+    } else if (p.xcd_remap == 3) {
+      bh = L % (p.b * p.h);
+      n_block = L / (p.b * p.h);
     } else if (p.xcd_remap) {
       const int xcd = L & 7, slot = L >> 3;
       bh = (slot / p.n_nblocks) * 8 + xcd;
@@ -409,6 +412,9 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) dq_kernel(const Params p
       const int xcd = L & 7, slot = L >> 3, per_xcd = (p.b * p.h) >> 3;
       bh = (slot % per_xcd) * 8 + xcd;
       m_block = slot / per_xcd;
+    } else if (p.xcd_remap == 3) {
+      bh = L % (p.b * p.h);
+      m_block = L / (p.b * p.h);
     } else if (p.xcd_remap) {
       const int xcd = L & 7, slot = L >> 3;
       bh = (slot / p.n_mblocks) * 8 + xcd;
@@ -632,7 +638,7 @@ hipError_t launch_bwd_t(const Params &p, hipStream_t stream) {
 hipError_t launch_bwd(Params &p, int dtype, hipStream_t stream) {
   p.n_mblocks = (p.sq + kQBlock - 1) / kQBlock;
   p.n_nblocks = (p.sk + kKvBlock - 1) / kKvBlock;
-  p.xcd_remap = ((p.b * p.h) % 8 == 0) ? (p.wr >= 0 ? 2 : 1) : 0;
+  p.xcd_remap = ((p.b * p.h) % 8 == 0) ? (p.wr >= 0 ? 2 : 1) : (p.wr >= 0 ? 3 : 0);
   if (p.b * p.h == 0) return hipSuccess;
   if (p.drop || (p.d != 32 && p.d != 64 && p.d != 128)) return launch_bwd_anyd(p, dtype, stream);
   return dtype == 1 ? launch_bwd_t<_Float16>(p, stream) : launch_bwd_t<__bf16>(p, stream);

@@ -154,7 +154,7 @@ struct Params {
   float scale, scale_log2;
   int wl, wr;                         // window sizes after normalisation; < 0 = unbounded
   int n_mblocks, n_nblocks;
-  int xcd_remap;                      // 1: blocks of one (batch, head) share an XCD; 2: also longest blocks of all heads first
+  int xcd_remap;                      // 0: by (batch, head); 1: blocks of a (batch, head) share an XCD; 2: 1 + longest blocks of all heads first; 3: longest first without XCD grouping
   // key/value cache calls only: per-batch number of keys already in the cache (the cache
   // holds p.sk rows), rows appended from k_new / v_new before attending
   const int *seqlens_k;

@@ -61,6 +61,9 @@ __global__ void __launch_bounds__(NW * 64, NW * QB >= 16 ? 2 : (QB == 2 ? 1 : 2)
       const int xcd = L & 7, slot = L >> 3, per_xcd = (p.b * p.h) >> 3;
       bh = (slot % per_xcd) * 8 + xcd;
       m_block = slot / per_xcd;
+    } else if (p.xcd_remap == 3) {  // the same order when b*h is not a multiple of the XCD count
+      bh = L % (p.b * p.h);
+      m_block = L / (p.b * p.h);
     } else if (p.xcd_remap) {  // consecutive workgroup ids go round-robin over the 8 XCDs
       const int xcd = L & 7, slot = L >> 3;
       bh = (slot / p.n_mblocks) * 8 + xcd;
@@ -386,7 +389,7 @@ hipError_t launch_append_kv(const Params &p, int dtype, hipStream_t stream) {
 }
 
 hipError_t launch_fwd(Params &p, int dtype, hipStream_t stream) {
-  p.xcd_remap = ((p.b * p.h) % 8 == 0) ? (p.wr >= 0 ? 2 : 1) : 0;
+  p.xcd_remap = ((p.b * p.h) % 8 == 0) ? (p.wr >= 0 ? 2 : 1) : (p.wr >= 0 ? 3 : 0);
   if (p.b * p.h == 0 || p.sq == 0) return hipSuccess;
   if (decode_eligible(p)) return launch_decode(p, dtype, stream);
   if (p.drop || (p.d != 32 && p.d != 64 && p.d != 128)) return launch_fwd_anyd(p, dtype, stream);
