@@ -180,7 +180,19 @@ def main():
             for f in c2_fns:
                 f()
         torch.cuda.synchronize()
-        print(json.dumps({"pmc_probe": True, "copy_bytes_read": in_bytes, "copy_bytes_written": in_bytes}))
+        # two calls of the cache-decode configuration (64 sequences x 8192 cached keys, 32 query
+        # heads on 8 key/value heads of 128, fp16): 2 GiB of cache rows per call
+        del dst
+        b_, h_, hk_, sk_, d_ = 64, 32, 8, 8192, 128
+        qd = torch.randn((b_, 1, h_, d_), generator=gen, device="cuda").half()
+        kc, vc = (torch.randn((b_, sk_, hk_, d_), generator=gen, device="cuda").half() for _ in range(2))
+        kn, vn = (torch.randn((b_, 1, hk_, d_), generator=gen, device="cuda").half() for _ in range(2))
+        lens = torch.full((b_,), sk_ - 1, dtype=torch.int32, device="cuda")
+        for _ in range(2):
+            ops.flash_attn_kvcache(qd, kc, vc, kn, vn, lens, 1.0 / np.sqrt(d_), (-1, -1))
+        torch.cuda.synchronize()
+        print(json.dumps({"pmc_probe": True, "copy_bytes_read": in_bytes, "copy_bytes_written": in_bytes,
+                          "decode_cache_bytes": 2 * b_ * sk_ * hk_ * d_ * 2}))
         return
 
     ms_step, per, host_ms = time_ops(ev, c2_fns, args.steps, args.warmup)
