@@ -162,6 +162,12 @@ struct Params {
   const void *k_new, *v_new;
   int64_t knew_bs, vnew_bs, knew_rs, vnew_rs, knew_hs, vnew_hs;
   int fuse_append;                    // 1: the decode kernel appends k_new / v_new itself
+  // forward with the key axis split over workgroups (few query blocks, many keys): grid.y =
+  // n_splits, split s takes key tiles [s * split_tiles, (s + 1) * split_tiles) and writes
+  // unnormalised fp32 partials, merged by launch_split_merge
+  float *o_part;                      // [n_splits][b][h][sq][d]
+  float *ml_part;                     // [n_splits][b][h][sq][2]: reference maximum, row sum
+  int n_splits, split_tiles;
   // dropout (forward and backward calls): rng_state = {seed, offset} in device memory,
   // keep probability, its reciprocal and its 8-bit threshold floor(p_keep * 255)
   const uint64_t *rng_state;
@@ -189,6 +195,8 @@ hipError_t launch_bwd_anyd(Params &p, int dtype, hipStream_t stream);
 
 // A few query rows against a long key sequence (flash_decode.hip): all query heads of a
 // key/value head times all query rows must fit the 32 columns of one score tile.
+// merges p.n_splits partials (p.o_part, p.ml_part) into p.o_w and p.lse
+hipError_t launch_split_merge(const Params &p, int dtype, hipStream_t stream);
 bool decode_eligible(const Params &p);
 bool decode_can_append(const Params &p);  // then set p.fuse_append and skip launch_append_kv
 hipError_t launch_decode(Params &p, int dtype, hipStream_t stream);

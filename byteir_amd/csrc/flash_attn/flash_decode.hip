@@ -232,11 +232,11 @@ __global__ void __launch_bounds__(kDecWaves * 64, 2) decode_kernel(const Params 
 // merges the chunks' partials of one (batch, head, query row) per workgroup, one thread per
 // output element; n_splits <= 64, so lane s of every wave takes chunk s for the statistics
 template <typename T, int D>
-__global__ void __launch_bounds__(D) decode_merge_kernel(const Params p, const DecodeArgs a) {
+__global__ void __launch_bounds__(D < 64 ? 64 : D) decode_merge_kernel(const Params p, const DecodeArgs a) {
   __shared__ float wgt[64];
   const int64_t row = blockIdx.x;  // (batch * h + head) * sq + query row
   const int64_t rows = (int64_t)p.b * p.h * p.sq;
-  const int dcol = threadIdx.x, lane = threadIdx.x & 63;
+  const int dcol = threadIdx.x < D ? threadIdx.x : D - 1, lane = threadIdx.x & 63;  // whole waves only
   const bool has = lane < a.n_splits;
   const float m_s = has ? a.ml_part[(lane * rows + row) * 2] : -INFINITY;
   const float l_s = has ? a.ml_part[(lane * rows + row) * 2 + 1] : 0.f;
@@ -257,8 +257,8 @@ __global__ void __launch_bounds__(D) decode_merge_kernel(const Params p, const D
   const bool empty = l_all == 0.f || l_all != l_all;
   const int qi = (int)(row % p.sq), hq = (int)((row / p.sq) % p.h), bi = (int)(row / ((int64_t)p.sq * p.h));
   T *og = static_cast<T *>(p.o_w) + bi * p.o_bs + (int64_t)qi * p.o_rs + hq * p.o_hs;
-  og[dcol] = (T)(empty ? 0.f : acc / l_all);
-  if (dcol == 0) p.lse[row] = empty ? INFINITY : m_all * p.scale + log2_fast(l_all) * kLn2;
+  if (threadIdx.x < D) og[dcol] = (T)(empty ? 0.f : acc / l_all);
+  if (threadIdx.x == 0) p.lse[row] = empty ? INFINITY : m_all * p.scale + log2_fast(l_all) * kLn2;
 }
 
 template <typename T, int D>
@@ -287,7 +287,7 @@ hipError_t decode_td(const Params &p, hipStream_t stream) {
   hipError_t e = hipGetLastError();
   if (ws) {
     if (e == hipSuccess) {
-      decode_merge_kernel<T, D><<<dim3((unsigned)rows), dim3(D), 0, stream>>>(p, a);
+      decode_merge_kernel<T, D><<<dim3((unsigned)rows), dim3(D < 64 ? 64 : D), 0, stream>>>(p, a);
       e = hipGetLastError();
     }
     const hipError_t f = hipFreeAsync(ws, stream);
@@ -296,7 +296,26 @@ hipError_t decode_td(const Params &p, hipStream_t stream) {
   return e;
 }
 
+template <typename T>
+hipError_t split_merge_t(const Params &p, hipStream_t stream) {
+  DecodeArgs a{};
+  a.o_part = p.o_part; a.ml_part = p.ml_part; a.n_splits = p.n_splits;
+  const dim3 grid((unsigned)((size_t)p.b * p.h * p.sq));
+  switch (p.d) {
+  case 32: decode_merge_kernel<T, 32><<<grid, dim3(64), 0, stream>>>(p, a); break;
+  case 64: decode_merge_kernel<T, 64><<<grid, dim3(64), 0, stream>>>(p, a); break;
+  case 128: decode_merge_kernel<T, 128><<<grid, dim3(128), 0, stream>>>(p, a); break;
+  default: return hipErrorInvalidValue;
+  }
+  return hipGetLastError();
+}
+
 }  // namespace
+
+hipError_t launch_split_merge(const Params &p, int dtype, hipStream_t stream) {
+  if (p.n_splits > 64) return hipErrorInvalidValue;
+  return dtype == 1 ? split_merge_t<_Float16>(p, stream) : split_merge_t<__bf16>(p, stream);
+}
 
 bool decode_eligible(const Params &p) {
   return (p.d == 64 || p.d == 128) && p.sq > 0 && (p.h / p.h_k) * p.sq <= 32 && p.sk >= 1 && !p.drop;

@@ -95,8 +95,13 @@ __global__ void __launch_bounds__(NW * 64, NW * QB >= 16 ? 2 : (QB == 2 ? 1 : 2)
   int b_lo, b_hi, t0, t1;
   row_limits_sk(p, sk, m0, b_lo, t0);
   row_limits_sk(p, sk, m0 + kBM - 1, t1, b_hi);
-  const int n_min = b_lo / kBN;
-  const int n_max = b_hi > 0 ? (b_hi + kBN - 1) / kBN : 0;
+  int n_min = b_lo / kBN;
+  int n_max = b_hi > 0 ? (b_hi + kBN - 1) / kBN : 0;
+  const int split = blockIdx.y;  // key axis split over workgroups: this one's share of the tiles
+  if (p.n_splits > 1) {
+    n_min = max(n_min, split * p.split_tiles);
+    n_max = min(n_max, (split + 1) * p.split_tiles);
+  }
 
   const T *kg = static_cast<const T *>(p.k) + bi * p.k_bs + hk * p.k_hs;
   const T *vg = static_cast<const T *>(p.v) + bi * p.v_bs + hk * p.v_hs;
@@ -308,6 +313,20 @@ __global__ void __launch_bounds__(NW * 64, NW * QB >= 16 ? 2 : (QB == 2 ? 1 : 2)
     const float l_tot = l_run[qb] + partner32(l_run[qb]);
     const bool empty = l_tot == 0.f || l_tot != l_tot;
     const float inv = empty ? 1.f : 1.f / l_tot;
+    if (p.n_splits > 1) {  // unnormalised partial, relative to this split's reference maximum
+      if (qrow[qb] < p.sq) {
+        const int64_t prow = (((int64_t)split * p.b + bi) * p.h + hi) * p.sq + qrow[qb];
+        float *og = p.o_part + prow * D;
+#pragma unroll
+        for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+          for (int i4 = 0; i4 < 4; ++i4)
+            *reinterpret_cast<float4 *>(og + db * 32 + i4 * 8 + g * 4) =
+                float4{o_acc[qb][db][i4 * 4], o_acc[qb][db][i4 * 4 + 1], o_acc[qb][db][i4 * 4 + 2], o_acc[qb][db][i4 * 4 + 3]};
+        if (g == 0) { p.ml_part[prow * 2] = m_run[qb]; p.ml_part[prow * 2 + 1] = l_tot; }
+      }
+      continue;
+    }
     if (qrow[qb] < p.sq) {
       T *og = static_cast<T *>(p.o_w) + bi * p.o_bs + (int64_t)qrow[qb] * p.o_rs + hi * p.o_hs;
 #pragma unroll
@@ -339,10 +358,35 @@ hipError_t launch_fwd_d(Params &p, hipStream_t stream) {
   constexpr int BM = 32 * QB * NW;
   p.n_mblocks = (p.sq + BM - 1) / BM;
   if (p.n_mblocks == 0) return hipSuccess;
-  const dim3 grid((unsigned)(p.n_mblocks * p.b * p.h)), block(NW * 64);
+  // Few query blocks and many keys (a long prompt chunk of one sequence): split the key axis over
+  // workgroups until the chip is full, at least eight tiles per split (the reference's
+  // num_splits_heuristic has the same aim, flash_api.cu:118-160, but its entry points never
+  // enable it).  The partials live in a stream-ordered allocation; without it: one split.
+  const int n_wg = p.n_mblocks * p.b * p.h, n_tiles = (p.sk + kBN - 1) / kBN;
+  int n_splits = 1;
+  if (n_wg < 200 && n_tiles >= 16) n_splits = max(1, min(min((256 + n_wg - 1) / n_wg, n_tiles / 8), 32));
+  void *ws = nullptr;
+  const size_t rows = (size_t)p.b * p.h * p.sq;
+  p.n_splits = 1;
+  if (n_splits > 1 && hipMallocAsync(&ws, (size_t)n_splits * rows * (D + 2) * sizeof(float), stream) == hipSuccess) {
+    p.n_splits = n_splits;
+    p.split_tiles = (n_tiles + n_splits - 1) / n_splits;
+    p.o_part = static_cast<float *>(ws);
+    p.ml_part = p.o_part + (size_t)n_splits * rows * D;
+  } else if (n_splits > 1) {
+    (void)hipGetLastError();
+    ws = nullptr;
+  }
+  const dim3 grid((unsigned)n_wg, (unsigned)p.n_splits), block(NW * 64);
   if (p.seqlens_k) flash_fwd_kernel<T, D, QB, NW, true><<<grid, block, 0, stream>>>(p);
   else flash_fwd_kernel<T, D, QB, NW, false><<<grid, block, 0, stream>>>(p);
-  return hipGetLastError();
+  hipError_t e = hipGetLastError();
+  if (ws) {
+    if (e == hipSuccess) e = launch_split_merge(p, std::is_same<T, _Float16>::value ? 1 : 2, stream);
+    const hipError_t fr = hipFreeAsync(ws, stream);
+    if (e == hipSuccess) e = fr;
+  }
+  return e;
 }
 
 template <typename T>

@@ -84,6 +84,11 @@ CASES = [
     (1, 32, 40, 2, 2, 64, (-1, 0)),        # all 32 columns are rows of one head
     (2, 7, 5, 4, 1, 128, (-1, 0)),         # causal with sq > sk: leading rows keep no key
     (1, 3, 600, 6, 2, 128, (-1, 5)),       # right window only
+    # few query blocks against many keys: the key axis is split over workgroups and merged
+    (1, 300, 2000, 2, 2, 64, (-1, 0)),
+    (1, 256, 4096, 4, 1, 128, (-1, -1)),
+    (2, 100, 1500, 1, 1, 32, (200, 0)),
+    (1, 40, 2500, 3, 3, 128, (-1, 0)),
     # head dimensions without a tuned kernel: every multiple of 8 up to 256 is accepted
     (1, 150, 150, 2, 2, 8, (-1, 0)),
     (1, 1, 40, 2, 2, 16, (-1, -1)),
@@ -317,6 +322,7 @@ KV_CASES = [
     (2, 3, 4, 4, 64, 130, 0, [130, 1], (-1, -1), False),        # no append: read-only cache
     (2, 2, 4, 1, 64, 520, 2, [518, 300], (64, 0), True),        # sliding window, MQA
     (2, 1, 8, 2, 128, 5000, 1, [4999, 2500], (-1, -1), True),   # long cache: several chunks per head
+    (1, 64, 4, 4, 64, 3000, 64, [2900], (-1, 0), True),         # a prompt chunk against a long cache: split forward kernel
     (3, 2, 16, 2, 64, 2100, 2, [0, 2098, 700], (-1, 0), True),
     (2, 3, 4, 2, 96, 260, 3, [250, 17], (-1, 0), True),         # head dimensions without a tuned kernel
     (1, 1, 2, 2, 256, 300, 1, [299], (-1, -1), True),
