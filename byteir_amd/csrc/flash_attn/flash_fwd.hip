@@ -23,6 +23,9 @@
 // would grow by more than kRescaleSlack (in log2 units), or from -inf; exp2 then stays below
 // 2^kRescaleSlack, the identities O = acc / sum and LSE = max*scale + ln(sum) hold for any
 // reference maximum, and the accumulator rescale (D/2 multiplies per lane per tile) rarely runs.
+#include <algorithm>
+#include <cmath>
+
 #include "flash_common.h"
 
 namespace fa {
@@ -346,6 +349,28 @@ __global__ void __launch_bounds__(NW * 64, NW * QB >= 16 ? 2 : (QB == 2 ? 1 : 2)
   }
 }
 
+// Number of key-axis splits for `n_wg` workgroups over `n_tiles` key tiles on 256 CUs: as the
+// reference's num_splits_heuristic (flash_api.cu:118-160) -- one split when the chip is already
+// 80 % full; otherwise the smallest count whose last round of workgroups is at least 85 % as
+// full as the best count's -- with at most 32 splits of at least eight tiles.
+inline int pick_splits(int n_wg, int n_tiles) {
+  constexpr int kCUs = 256;
+  if (n_wg >= 0.8f * kCUs) return 1;
+  const int max_splits = std::min(32, n_tiles / 8);
+  auto tiles_per = [&](int s) { return (n_tiles + s - 1) / s; };
+  auto eligible = [&](int s) { return s == 1 || tiles_per(s) != tiles_per(s - 1); };
+  auto eff = [&](int s) {
+    const float waves = float(n_wg * s) / kCUs;
+    return waves / std::ceil(waves);
+  };
+  float best = 0.f;
+  for (int s = 1; s <= max_splits; ++s)
+    if (eligible(s)) best = std::max(best, eff(s));
+  for (int s = 1; s <= max_splits; ++s)
+    if (eligible(s) && eff(s) >= 0.85f * best) return s;
+  return 1;
+}
+
 // Geometry: 8 waves of 32 rows, two waves per SIMD.  The kernel is written for 32*QB rows per
 // wave; QB = 2 halves the LDS traffic per MFMA, but either needs a whole SIMD per wave
 // (head_dim 128: slower, the compiler's schedule leaves the single wave stalled) or brought no
@@ -363,8 +388,7 @@ hipError_t launch_fwd_d(Params &p, hipStream_t stream) {
   // num_splits_heuristic has the same aim, flash_api.cu:118-160, but its entry points never
   // enable it).  The partials live in a stream-ordered allocation; without it: one split.
   const int n_wg = p.n_mblocks * p.b * p.h, n_tiles = (p.sk + kBN - 1) / kBN;
-  int n_splits = 1;
-  if (n_wg < 200 && n_tiles >= 16) n_splits = max(1, min(min((256 + n_wg - 1) / n_wg, n_tiles / 8), 32));
+  const int n_splits = pick_splits(n_wg, n_tiles);
   void *ws = nullptr;
   const size_t rows = (size_t)p.b * p.h * p.sq;
   p.n_splits = 1;
