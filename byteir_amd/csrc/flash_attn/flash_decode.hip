@@ -38,7 +38,7 @@ struct DecodeArgs {
 };
 
 template <typename T, int D>
-__global__ void __launch_bounds__(kDecWaves * 64, 2) decode_kernel(const Params p, const DecodeArgs a) {
+__global__ void __launch_bounds__(kDecWaves * 64, D <= 128 ? 2 : 1) decode_kernel(const Params p, const DecodeArgs a) {
   using vec8 = typename Traits<T>::vec8;
   constexpr int KS = Pad<D>::kPlain, VS = Pad<D>::kTr;
   constexpr int CPR = D / 8;         // 16-byte chunks per row
@@ -318,7 +318,7 @@ hipError_t launch_split_merge(const Params &p, int dtype, hipStream_t stream) {
 }
 
 bool decode_eligible(const Params &p) {
-  return (p.d == 64 || p.d == 128) && p.sq > 0 && (p.h / p.h_k) * p.sq <= 32 && p.sk >= 1 && !p.drop;
+  return (p.d == 32 || p.d == 64 || p.d == 128 || p.d == 256) && p.sq > 0 && (p.h / p.h_k) * p.sq <= 32 && p.sk >= 1 && !p.drop;
 }
 
 // The decode kernel can do the append itself when every appended row is certain to be loaded by
@@ -329,7 +329,9 @@ bool decode_can_append(const Params &p) {
 
 hipError_t launch_decode(Params &p, int dtype, hipStream_t stream) {
   if (p.b * p.h == 0 || p.sq == 0) return hipSuccess;
+  if (p.d == 32) return dtype == 1 ? decode_td<_Float16, 32>(p, stream) : decode_td<__bf16, 32>(p, stream);
   if (p.d == 64) return dtype == 1 ? decode_td<_Float16, 64>(p, stream) : decode_td<__bf16, 64>(p, stream);
+  if (p.d == 256) return dtype == 1 ? decode_td<_Float16, 256>(p, stream) : decode_td<__bf16, 256>(p, stream);
   return dtype == 1 ? decode_td<_Float16, 128>(p, stream) : decode_td<__bf16, 128>(p, stream);
 }
 

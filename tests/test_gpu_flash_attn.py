@@ -81,6 +81,8 @@ CASES = [
     (1, 8, 700, 4, 1, 128, (100, 0)),      # 32 columns, sliding window
     (1, 2, 9000, 2, 2, 64, (-1, -1)),      # several chunks per head
     (3, 1, 33, 4, 4, 64, (-1, 0)),
+    (2, 1, 2100, 4, 2, 256, (-1, -1)),     # decode kernel at head_dim 256 and 32
+    (2, 3, 1300, 8, 1, 32, (-1, 0)),
     (1, 32, 40, 2, 2, 64, (-1, 0)),        # all 32 columns are rows of one head
     (2, 7, 5, 4, 1, 128, (-1, 0)),         # causal with sq > sk: leading rows keep no key
     (1, 3, 600, 6, 2, 128, (-1, 5)),       # right window only
