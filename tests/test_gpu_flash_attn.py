@@ -500,3 +500,35 @@ def test_decode_call_inside_a_hip_graph():
         torch.cuda.synchronize()
         assert torch.equal(o_graph, o_eager) and torch.equal(lse_graph, lse_eager), step
         assert torch.equal(kc_graph, kc), step
+
+
+def test_decode_benchmark_size_sampled_heads():
+    """The benchmark's decode call (fp16, 64 sequences with up to 8192 cached keys, 32 query heads on
+    8 key/value heads of 128, one new token): ragged lengths, the appended rows land in the caches
+    bit for bit and nothing else changes; sampled (batch, head) pairs match the float64 closed
+    form over exactly the valid rows."""
+    from byteir_amd import ops
+    b, h, h_k, d, cap = 64, 32, 8, 128, 8192
+    g = torch.Generator(device="cuda").manual_seed(0xDC)
+    q = torch.randn((b, 1, h, d), generator=g, device="cuda").half()
+    kc, vc = (torch.randn((b, cap, h_k, d), generator=g, device="cuda").half() for _ in range(2))
+    kn, vn = (torch.randn((b, 1, h_k, d), generator=g, device="cuda").half() for _ in range(2))
+    lens = torch.randint(1, cap, (b,), generator=g, device="cuda", dtype=torch.int32)
+    lens[0], lens[1] = cap - 1, 0
+    kc0, vc0 = kc.clone(), vc.clone()
+    scale = 1.0 / np.sqrt(d)
+    o, lse = ops.flash_attn_kvcache(q, kc, vc, kn, vn, lens, scale, (-1, -1))
+    rows = lens.long()
+    bi_all = torch.arange(b, device="cuda")
+    assert torch.equal(kc[bi_all, rows], kn[:, 0]) and torch.equal(vc[bi_all, rows], vn[:, 0])
+    kc0[bi_all, rows], vc0[bi_all, rows] = kn[:, 0], vn[:, 0]
+    assert torch.equal(kc, kc0) and torch.equal(vc, vc0)
+    rng = np.random.default_rng(3)
+    for bi, hi in [(0, 0), (1, 31)] + [(int(rng.integers(b)), int(rng.integers(h))) for _ in range(10)]:
+        n = int(lens[bi]) + 1
+        K, V = kc[bi, :n, hi // (h // h_k)].double(), vc[bi, :n, hi // (h // h_k)].double()
+        s = (K @ q[bi, 0, hi].double()) * scale
+        p = torch.softmax(s, dim=0)
+        want_o, want_lse = p @ V, torch.logsumexp(s, dim=0)
+        assert float((o[bi, 0, hi].double() - want_o).abs().max()) <= ATOL
+        assert abs(float(lse[bi, hi, 0]) - float(want_lse)) <= ATOL
