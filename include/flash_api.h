@@ -27,6 +27,9 @@
  * have tuned kernels), 0 <= p_dropout < 1, any seqlen, h % h_k == 0
  * (backward: h == h_k).  Anything else is reported on stderr and the process aborts, since
  * the ABI has no error channel; the *_checked variants return an error code instead.
+ * Calls with few query rows or few query blocks against many keys split the key axis over
+ * workgroups and keep their partial results in a stream-ordered allocation
+ * (hipMallocAsync / hipFreeAsync on `stream`); no other call allocates.
  */
 #ifndef BYTEIR_AMD_FLASH_API_H_
 #define BYTEIR_AMD_FLASH_API_H_
