@@ -148,15 +148,17 @@ struct DropCtx {
   }
 };
 
-__device__ __forceinline__ void block_of(const Params &p, int n_blocks, bool reversed, int &blk, int &bh) {
+__device__ __forceinline__ void block_of(const Params &p, int n_blocks, bool reversed, int &blk, int &bh,
+                                         int n_bh = -1) {  // n_bh: (batch, head) pairs, b * h by default
+  if (n_bh < 0) n_bh = p.b * p.h;
   const int L = blockIdx.x;
   if (p.xcd_remap == 2) {  // unequal blocks: the longest block of every (batch, head) first
-    const int xcd = L & 7, slot = L >> 3, per_xcd = (p.b * p.h) >> 3;
+    const int xcd = L & 7, slot = L >> 3, per_xcd = n_bh >> 3;
     bh = (slot % per_xcd) * 8 + xcd;
     blk = slot / per_xcd;
   } else if (p.xcd_remap == 3) {  // the same order when b*h is not a multiple of the XCD count
-    bh = L % (p.b * p.h);
-    blk = L / (p.b * p.h);
+    bh = L % n_bh;
+    blk = L / n_bh;
   } else if (p.xcd_remap) {  // consecutive workgroup ids go round-robin over the 8 XCDs
     const int xcd = L & 7, slot = L >> 3;
     bh = (slot / n_blocks) * 8 + xcd;
@@ -364,18 +366,17 @@ __global__ void __launch_bounds__(256) dkdv_anyd_kernel(const Params p) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r32 = lane & 31, g = lane >> 5;
   int n_block, bh;
-  block_of(p, p.n_nblocks, false, n_block, bh);
-  const int bi = bh / p.h, hi = bh % p.h;
+  block_of(p, p.n_nblocks, false, n_block, bh, p.b * p.h_k);
+  // a workgroup belongs to a key/value head; its dK, dV sum over the query heads of the group
+  const int bi = bh / p.h_k, hk = bh % p.h_k, group = p.h / p.h_k;
   const int kvb0 = n_block * kRows;
   const int kvcol = kvb0 + wave * 32 + r32;  // the key this lane owns
   const int off = p.sk - p.sq;
 
-  const T *qg = static_cast<const T *>(p.q) + bi * p.q_bs + hi * p.q_hs;
-  const T *dog = static_cast<const T *>(p.dout) + bi * p.o_bs + hi * p.o_hs;
-  const T *kg = static_cast<const T *>(p.k) + bi * p.k_bs + (int64_t)kvcol * p.k_rs + hi * p.k_hs;
-  const T *vg = static_cast<const T *>(p.v) + bi * p.v_bs + (int64_t)kvcol * p.v_rs + hi * p.v_hs;
-  const float *lse_g = p.lse + ((int64_t)bi * p.h + hi) * p.sq;
-  const float *dsm_g = p.dsoftmax + ((int64_t)bi * p.h + hi) * p.sq_rounded;
+  const T *qg = nullptr, *dog = nullptr;  // of the query head being streamed (set per head below)
+  const float *lse_g = nullptr, *dsm_g = nullptr;
+  const T *kg = static_cast<const T *>(p.k) + bi * p.k_bs + (int64_t)kvcol * p.k_rs + hk * p.k_hs;
+  const T *vg = static_cast<const T *>(p.v) + bi * p.v_bs + (int64_t)kvcol * p.v_rs + hk * p.v_hs;
 
   vec8 kf[DR / 16], vf[DR / 16];
 #pragma unroll
@@ -395,7 +396,6 @@ __global__ void __launch_bounds__(256) dkdv_anyd_kernel(const Params p) {
   const int m_max = q_hi > 0 ? (q_hi + kTile - 1) / kTile : 0;
   const float c = p.scale_log2;
   DropCtx drop;
-  if constexpr (Drop) drop.init(p, bh);
 
   AnyTileLoader<T, DR, kTile> lq, ldo;
   float lse_r = 0.f, dsm_r = 0.f;
@@ -414,6 +414,15 @@ __global__ void __launch_bounds__(256) dkdv_anyd_kernel(const Params p) {
     if (tid < kTile) { lse_s[tid] = lse_r * kLog2e; dsm_s[tid] = dsm_r; }
   };
 
+  int drop_bh = 0;  // batch * heads + query head: the dropout stream of the head being processed
+  for (int gq = 0; gq < group; ++gq) {  // the query heads that share this key/value head
+  const int hi = hk * group + gq;
+  qg = static_cast<const T *>(p.q) + bi * p.q_bs + hi * p.q_hs;
+  dog = static_cast<const T *>(p.dout) + bi * p.o_bs + hi * p.o_hs;
+  lse_g = p.lse + ((int64_t)bi * p.h + hi) * p.sq;
+  dsm_g = p.dsoftmax + ((int64_t)bi * p.h + hi) * p.sq_rounded;
+  drop_bh = bi * p.h + hi;
+  if constexpr (Drop) drop.init(p, drop_bh);
   if (kPrefetch && m_min < m_max) {
     gload(m_min);
     lstore();
@@ -482,9 +491,10 @@ __global__ void __launch_bounds__(256) dkdv_anyd_kernel(const Params p) {
     }
   }
 
+  }
   if (kvcol < p.sk) {
-    T *dkg = static_cast<T *>(p.dk) + bi * p.k_bs + (int64_t)kvcol * p.k_rs + hi * p.k_hs;
-    T *dvg = static_cast<T *>(p.dv) + bi * p.v_bs + (int64_t)kvcol * p.v_rs + hi * p.v_hs;
+    T *dkg = static_cast<T *>(p.dk) + bi * p.k_bs + (int64_t)kvcol * p.k_rs + hk * p.k_hs;
+    T *dvg = static_cast<T *>(p.dv) + bi * p.v_bs + (int64_t)kvcol * p.v_rs + hk * p.v_hs;
 #pragma unroll
     for (int db = 0; db < DR / 32; ++db) {
       store_acc<T>(dkg, dk_acc[db], db, g, Drop ? p.scale * p.rp_keep : p.scale, p.d);
@@ -521,8 +531,9 @@ __global__ void __launch_bounds__(256) dq_anyd_kernel(const Params p) {
 
   const T *qg = static_cast<const T *>(p.q) + bi * p.q_bs + (int64_t)qrow * p.q_rs + hi * p.q_hs;
   const T *dog = static_cast<const T *>(p.dout) + bi * p.o_bs + (int64_t)qrow * p.o_rs + hi * p.o_hs;
-  const T *kg = static_cast<const T *>(p.k) + bi * p.k_bs + hi * p.k_hs;
-  const T *vg = static_cast<const T *>(p.v) + bi * p.v_bs + hi * p.v_hs;
+  const int hk = hi / (p.h / p.h_k);
+  const T *kg = static_cast<const T *>(p.k) + bi * p.k_bs + hk * p.k_hs;
+  const T *vg = static_cast<const T *>(p.v) + bi * p.v_bs + hk * p.v_hs;
 
   vec8 qf[DR / 16], dof[DR / 16];
 #pragma unroll
@@ -632,10 +643,12 @@ hipError_t fwd_anyd_d(const Params &p, hipStream_t stream) {
 
 template <typename T, int DR>
 hipError_t bwd_anyd_d(const Params &p, hipStream_t stream) {
-  const dim3 gk((unsigned)(p.n_nblocks * p.b * p.h)), gq((unsigned)(p.n_mblocks * p.b * p.h)), block(256);
+  const dim3 gk((unsigned)(p.n_nblocks * p.b * p.h_k)), gq((unsigned)(p.n_mblocks * p.b * p.h)), block(256);
   if (p.n_nblocks > 0) {
-    if (p.drop) dkdv_anyd_kernel<T, DR, true><<<gk, block, 0, stream>>>(p);
-    else dkdv_anyd_kernel<T, DR, false><<<gk, block, 0, stream>>>(p);
+    Params pk = p;  // the dK/dV grid runs over key/value heads
+    pk.xcd_remap = ((p.b * p.h_k) % 8 == 0) ? (p.wr >= 0 ? 2 : 1) : (p.wr >= 0 ? 3 : 0);
+    if (p.drop) dkdv_anyd_kernel<T, DR, true><<<gk, block, 0, stream>>>(pk);
+    else dkdv_anyd_kernel<T, DR, false><<<gk, block, 0, stream>>>(pk);
   }
   if (p.n_mblocks > 0) {
     if (p.drop) dq_anyd_kernel<T, DR, true><<<gq, block, 0, stream>>>(p);

@@ -159,7 +159,6 @@ int flash_attn_bwd_checked(void **tensors, const void *extra_args, int dtype, vo
   const Blob a = parse(extra_args);
   fa::Params p{};
   if (int r = fill(a, p)) return r;
-  if (a.h != a.h_k) return fail("backward needs h == h_k (got %ld, %ld)", (long)a.h, (long)a.h_k);
   if (a.seqlen_q_rounded < a.seqlen_q) return fail("seqlen_q_rounded < seqlen_q");
   // tensors: dout, q, k, v, out, softmax_lse, rng_state, dq, dk, dv, d_softmax, dq_accum
   p.dout = tensors[0]; p.q = tensors[1]; p.k = tensors[2]; p.v = tensors[3]; p.o = tensors[4];

@@ -135,12 +135,12 @@ __global__ void __launch_bounds__(256, (D <= 64 && KB == 1) ? 2 : 1) dkdv_kernel
   {
     const int L = blockIdx.x;
     if (p.xcd_remap == 2) {  // unequal blocks: the longest (first) key block of every head first
-      const int xcd = L & 7, slot = L >> 3, per_xcd = (p.b * p.h) >> 3;
+      const int xcd = L & 7, slot = L >> 3, per_xcd = (p.b * p.h_k) >> 3;
       bh = (slot % per_xcd) * 8 + xcd;
       n_block = slot / per_xcd;
     } else if (p.xcd_remap == 3) {
-      bh = L % (p.b * p.h);
-      n_block = L / (p.b * p.h);
+      bh = L % (p.b * p.h_k);
+      n_block = L / (p.b * p.h_k);
     } else if (p.xcd_remap) {
       const int xcd = L & 7, slot = L >> 3;
       bh = (slot / p.n_nblocks) * 8 + xcd;
@@ -150,24 +150,24 @@ __global__ void __launch_bounds__(256, (D <= 64 && KB == 1) ? 2 : 1) dkdv_kernel
       n_block = L % p.n_nblocks;
     }
   }
-  const int bi = bh / p.h, hi = bh % p.h;
+  // a workgroup belongs to a key/value head; its dK, dV sum over the query heads of the group
+  const int bi = bh / p.h_k, hk = bh % p.h_k, group = p.h / p.h_k;
   constexpr int kKeys = kKvBlock * KB;
   const int kvb0 = n_block * kKeys;
   const int wkv0 = kvb0 + wave * 32 * KB;  // first key of the wave
   const int off = p.sk - p.sq;
 
-  const T *qg = static_cast<const T *>(p.q) + bi * p.q_bs + hi * p.q_hs;
-  const T *dog = static_cast<const T *>(p.dout) + bi * p.o_bs + hi * p.o_hs;
-  const float *lse_g = p.lse + ((int64_t)bi * p.h + hi) * p.sq;
-  const float *dsm_g = p.dsoftmax + ((int64_t)bi * p.h + hi) * p.sq_rounded;
+  // pointers of the query head being streamed (set per head below)
+  const T *qg = nullptr, *dog = nullptr;
+  const float *lse_g = nullptr, *dsm_g = nullptr;
 
   int kvcol[KB];  // the keys this lane owns
   vec8 kf[KB][D / 16], vf[KB][D / 16];
 #pragma unroll
   for (int kb = 0; kb < KB; ++kb) {
     kvcol[kb] = wkv0 + kb * 32 + r32;
-    const T *kg = static_cast<const T *>(p.k) + bi * p.k_bs + (int64_t)kvcol[kb] * p.k_rs + hi * p.k_hs;
-    const T *vg = static_cast<const T *>(p.v) + bi * p.v_bs + (int64_t)kvcol[kb] * p.v_rs + hi * p.v_hs;
+    const T *kg = static_cast<const T *>(p.k) + bi * p.k_bs + (int64_t)kvcol[kb] * p.k_rs + hk * p.k_hs;
+    const T *vg = static_cast<const T *>(p.v) + bi * p.v_bs + (int64_t)kvcol[kb] * p.v_rs + hk * p.v_hs;
 #pragma unroll
     for (int ks = 0; ks < D / 16; ++ks) {
       if (kvcol[kb] < p.sk) {
@@ -203,10 +203,8 @@ __global__ void __launch_bounds__(256, (D <= 64 && KB == 1) ? 2 : 1) dkdv_kernel
   const unsigned win_span = (unsigned)((p.wr >= 0 ? p.wr : (1 << 30)) - win_lo);
 
   TileLoader<T, D, kQTile> lq, ldo;  // tiles are fetched in order, m_min first
-  lq.start(qg, p.q_rs, m_min * kQTile, p.sq);
-  ldo.start(dog, p.o_rs, m_min * kQTile, p.sq);
   float lse_r = 0.f, dsm_r = 0.f;
-  int q_next = m_min * kQTile + tid;  // the row whose LSE and D this thread stages next
+  int q_next = 0;  // the row whose LSE and D this thread stages next
   auto gload = [&]() {
     lq.gload();
     ldo.gload();
@@ -330,8 +328,24 @@ __global__ void __launch_bounds__(256, (D <= 64 && KB == 1) ? 2 : 1) dkdv_kernel
       for (int w = 0; w < 2; ++w) { pb[kb][w] = pb_new[kb][w]; dsb[kb][w] = dsb_new[kb][w]; }
   };
 
-  // prologue: tiles m_min and m_min+1 into the ring, tile m_min+2 into registers
   const int n_tiles = m_max > m_min ? m_max - m_min : 0;
+  for (int gq = 0; gq < group; ++gq) {  // the query heads that share this key/value head
+  const int hi = hk * group + gq;
+  qg = static_cast<const T *>(p.q) + bi * p.q_bs + hi * p.q_hs;
+  dog = static_cast<const T *>(p.dout) + bi * p.o_bs + hi * p.o_hs;
+  lse_g = p.lse + ((int64_t)bi * p.h + hi) * p.sq;
+  dsm_g = p.dsoftmax + ((int64_t)bi * p.h + hi) * p.sq_rounded;
+  lq.start(qg, p.q_rs, m_min * kQTile, p.sq);
+  ldo.start(dog, p.o_rs, m_min * kQTile, p.sq);
+  q_next = m_min * kQTile + tid;
+  if (gq > 0) {
+    __syncthreads();  // every wave has left the previous head's last tile
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+      for (int w = 0; w < 2; ++w) { pb[kb][w] = vec8{0}; dsb[kb][w] = vec8{0}; }
+  }
+  // prologue: tiles m_min and m_min+1 into the ring, tile m_min+2 into registers
   if (n_tiles > 0) {
     gload();
     lstore(0);
@@ -356,12 +370,13 @@ __global__ void __launch_bounds__(256, (D <= 64 && KB == 1) ? 2 : 1) dkdv_kernel
     buf = buf1;
   }
   if (n_tiles > 0) part_c(Qs[pbuf], dOs[pbuf], 1, pb, dsb);
+  }
 
 #pragma unroll
   for (int kb = 0; kb < KB; ++kb) {
     if (kvcol[kb] < p.sk) {
-      T *dkg = static_cast<T *>(p.dk) + bi * p.k_bs + (int64_t)kvcol[kb] * p.k_rs + hi * p.k_hs;
-      T *dvg = static_cast<T *>(p.dv) + bi * p.v_bs + (int64_t)kvcol[kb] * p.v_rs + hi * p.v_hs;
+      T *dkg = static_cast<T *>(p.dk) + bi * p.k_bs + (int64_t)kvcol[kb] * p.k_rs + hk * p.k_hs;
+      T *dvg = static_cast<T *>(p.dv) + bi * p.v_bs + (int64_t)kvcol[kb] * p.v_rs + hk * p.v_hs;
       typedef T vec4 __attribute__((ext_vector_type(4)));
 #pragma unroll
       for (int db = 0; db < D / 32; ++db)
@@ -440,8 +455,9 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) dq_kernel(const Params p
   const int n_min = b_lo / kKvTile;
   const int n_max = b_hi > 0 ? (b_hi + kKvTile - 1) / kKvTile : 0;
 
-  const T *kg = static_cast<const T *>(p.k) + bi * p.k_bs + hi * p.k_hs;
-  const T *vg = static_cast<const T *>(p.v) + bi * p.v_bs + hi * p.v_hs;
+  const int hk = hi / (p.h / p.h_k);
+  const T *kg = static_cast<const T *>(p.k) + bi * p.k_bs + hk * p.k_hs;
+  const T *vg = static_cast<const T *>(p.v) + bi * p.v_bs + hk * p.v_hs;
 
   vec8 qf[D / 16], dof[D / 16];
   float lse_l = INFINITY, dsm_l = 0.f;  // +inf: a row beyond seqlen_q contributes P = 0
@@ -616,8 +632,9 @@ hipError_t launch_bwd_td(const Params &p, hipStream_t stream) {
   constexpr int KB = 1;
   Params pk = p;
   pk.n_nblocks = (p.sk + kKvBlock * KB - 1) / (kKvBlock * KB);
+  pk.xcd_remap = ((p.b * p.h_k) % 8 == 0) ? (p.wr >= 0 ? 2 : 1) : (p.wr >= 0 ? 3 : 0);
   if (pk.n_nblocks > 0)
-    dkdv_kernel<T, D, KB><<<dim3((unsigned)(pk.n_nblocks * p.b * p.h)), dim3(256), 0, stream>>>(pk);
+    dkdv_kernel<T, D, KB><<<dim3((unsigned)(pk.n_nblocks * p.b * p.h_k)), dim3(256), 0, stream>>>(pk);
   Params pq = p;
   pq.n_mblocks = (p.sq + kQBlock - 1) / kQBlock;
   if (pq.n_mblocks > 0)

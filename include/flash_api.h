@@ -25,7 +25,8 @@
  *
  * Supported here: head_dim a multiple of 8 up to 256 (the reference's range; 32, 64 and 128
  * have tuned kernels), 0 <= p_dropout < 1, any seqlen, h % h_k == 0
- * (backward: h == h_k).  Anything else is reported on stderr and the process aborts, since
+ * (backward with h_k < h: dK, dV of a key/value head are the sums over its query heads -- the
+ * gradient; the reference's own addressing of dK / dV is only right for h == h_k).  Anything else is reported on stderr and the process aborts, since
  * the ABI has no error channel; the *_checked variants return an error code instead.
  * Calls with few query rows or few query blocks against many keys split the key axis over
  * workgroups and keep their partial results in a stream-ordered allocation

@@ -301,7 +301,7 @@ def flash_bwd(dout, q, k, v, o, lse, scale, window=(-1, -1), round_p=True, p_dro
     lse = np.ascontiguousarray(lse, dtype=np.float32)
     b, sq, h, d = q.shape
     sk, h_k = k.shape[1], k.shape[2]
-    assert h == h_k, "backward needs h == h_k"
+    assert h % h_k == 0
     a = fa_args(b, sq, sk, h, h_k, d, scale, window, p_dropout)
     dq, dk, dv = np.empty_like(q), np.empty_like(k), np.empty_like(v)
     dsm = np.empty((b, h, sq), dtype=np.float32)

@@ -494,8 +494,9 @@ void oracle_flash_fwd(const oracle_fa_args *a, int dtype, int round_p, const voi
  *   ds_ij = p_ij (dp_ij - D_i); dV_j = sum_i round16(p_ij) dO_i;
  *   dK_j = scale sum_i round16(ds_ij) q_i; dQ_i = scale sum_j round16(ds_ij) k_j.
  * Accumulation in float; outputs rounded to storage.  round_p = 0 keeps p and ds unrounded.
- * dq/dk/dv use the strides of q/k/v (flash_api.cu:377-389).  h must equal h_k (the
- * reference's dK/dV addressing is only right in that case).  d_softmax [b, h, sq] float,
+ * dq/dk/dv use the strides of q/k/v (flash_api.cu:377-389).  With grouped heads (h_k < h) dK and
+ * dV of a key/value head are the sums over its h / h_k query heads -- the mathematical gradient;
+ * the reference's own dK/dV addressing is only right for h == h_k, where this reduces to it.  d_softmax [b, h, sq] float,
  * when non-null, receives D.
  * With a->p_dropout > 0 (rng_state = {seed, offset} required), as the reference arranges it
  * (flash_bwd_preprocess_kernel.h:124-128, flash_bwd_kernel.h:524-536,571-573,667,713-718):
@@ -505,7 +506,8 @@ void oracle_flash_bwd_rng(const oracle_fa_args *a, int dtype, int round_p, const
                           const void *q, const void *k, const void *v, const void *o,
                           const float *lse, const uint64_t *rng_state, void *dq, void *dk, void *dv,
                           float *d_softmax) {
-  const int64_t b = a->b, h = a->h, d = a->d, sq = a->seqlen_q, sk = a->seqlen_k;
+  const int64_t b = a->b, h = a->h, hk = a->h_k, d = a->d, sq = a->seqlen_q, sk = a->seqlen_k;
+  const int64_t ratio = h / hk; /* query heads per key/value head: their dK, dV contributions add up */
   const int drop = a->p_dropout > 0.f && rng_state;
   float p_keep, rp_keep; uint8_t thr;
   dropout_consts(drop ? a->p_dropout : 0.f, &p_keep, &thr, &rp_keep);
@@ -513,12 +515,13 @@ void oracle_flash_bwd_rng(const oracle_fa_args *a, int dtype, int round_p, const
   const float scale_log2 = (float)(a->softmax_scale * M_LOG2E);
 #pragma omp parallel for num_threads(g_threads) schedule(dynamic, 1) collapse(2)
   for (int64_t bi = 0; bi < b; ++bi)
-    for (int64_t hi = 0; hi < h; ++hi) {
+    for (int64_t hki = 0; hki < hk; ++hki) {
       float *dkacc = (float *)calloc((size_t)(sk * d), sizeof(float));
       float *dvacc = (float *)calloc((size_t)(sk * d), sizeof(float));
       float *dqacc = (float *)malloc(sizeof(float) * (size_t)d);
       float *qf = (float *)malloc(sizeof(float) * (size_t)d);
       float *dof = (float *)malloc(sizeof(float) * (size_t)d);
+      for (int64_t hi = hki * ratio; hi < (hki + 1) * ratio; ++hi)
       for (int64_t i = 0; i < sq; ++i) {
         size_t qoff = (size_t)(bi * a->q_batch_stride + i * a->q_row_stride + hi * a->q_head_stride);
         size_t ooff = (size_t)(bi * a->o_batch_stride + i * a->o_row_stride + hi * a->o_head_stride);
@@ -535,8 +538,8 @@ void oracle_flash_bwd_rng(const oracle_fa_args *a, int dtype, int round_p, const
         int64_t lo, hi_;
         window_bounds(i, sq, sk, a->window_size_left, a->window_size_right, &lo, &hi_);
         for (int64_t j = lo; j < hi_; ++j) {
-          size_t koff = (size_t)(bi * a->k_batch_stride + j * a->k_row_stride + hi * a->k_head_stride);
-          size_t voff = (size_t)(bi * a->v_batch_stride + j * a->v_row_stride + hi * a->v_head_stride);
+          size_t koff = (size_t)(bi * a->k_batch_stride + j * a->k_row_stride + hki * a->k_head_stride);
+          size_t voff = (size_t)(bi * a->v_batch_stride + j * a->v_row_stride + hki * a->v_head_stride);
           float dot = 0.f, dp = 0.f;
           for (int64_t x = 0; x < d; ++x) {
             dot += qf[x] * load_elem(k, koff + x, dtype);
@@ -556,8 +559,8 @@ void oracle_flash_bwd_rng(const oracle_fa_args *a, int dtype, int round_p, const
         for (int64_t x = 0; x < d; ++x) store_elem(dq, qoff + x, dtype, dqacc[x] * scale);
       }
       for (int64_t j = 0; j < sk; ++j) {
-        size_t koff = (size_t)(bi * a->k_batch_stride + j * a->k_row_stride + hi * a->k_head_stride);
-        size_t voff = (size_t)(bi * a->v_batch_stride + j * a->v_row_stride + hi * a->v_head_stride);
+        size_t koff = (size_t)(bi * a->k_batch_stride + j * a->k_row_stride + hki * a->k_head_stride);
+        size_t voff = (size_t)(bi * a->v_batch_stride + j * a->v_row_stride + hki * a->v_head_stride);
         for (int64_t x = 0; x < d; ++x) {
           store_elem(dk, koff + x, dtype, dkacc[j * d + x] * scale);
           store_elem(dv, voff + x, dtype, drop ? dvacc[j * d + x] * rp_keep : dvacc[j * d + x]);

@@ -70,10 +70,12 @@ CASES = [
     (1, 200, 333, 2, 2, 64, (-1, -1)),     # ragged, sq != sk
     (1, 333, 200, 2, 2, 128, (-1, 0)),     # causal with sq > sk: leading rows keep no key
     (1, 77, 500, 8, 8, 32, (-1, 0)),
-    (1, 513, 513, 8, 2, 64, (-1, 0)),      # grouped-query heads (forward only)
+    (1, 513, 513, 8, 2, 64, (-1, 0)),      # grouped-query heads
     (1, 300, 300, 2, 2, 64, (64, 0)),      # sliding window, left-bounded causal
     (1, 300, 260, 2, 2, 128, (40, 30)),    # local window both sides
     (3, 1, 50, 1, 1, 32, (-1, -1)),        # single query row
+    (2, 260, 260, 8, 2, 128, (-1, 0)),     # grouped-query heads: dK, dV sum over the group
+    (1, 190, 300, 6, 1, 32, (50, 20)),     # one key/value head for all query heads
     # few query rows: the decode kernel (all query heads of a key/value head in one score tile,
     # keys split over waves and, for long sequences, over workgroups)
     (2, 1, 1000, 8, 2, 128, (-1, -1)),
@@ -99,7 +101,7 @@ CASES = [
     (1, 96, 96, 2, 2, 48, (-1, 0)),
     (1, 200, 200, 2, 2, 72, (30, 0)),
     (1, 130, 190, 2, 2, 96, (-1, 0)),
-    (2, 100, 100, 2, 1, 96, (-1, -1)),     # grouped-query heads (forward only)
+    (2, 100, 100, 2, 1, 96, (-1, -1)),     # grouped-query heads
     (1, 64, 64, 1, 1, 104, (-1, -1)),
     (1, 140, 260, 2, 2, 160, (-1, 0)),
     (1, 257, 129, 1, 1, 192, (-1, -1)),
@@ -144,7 +146,7 @@ def test_forward_matches_oracle(case, code):
 
 
 @pytest.mark.parametrize("code", [oracle.F16, oracle.BF16])
-@pytest.mark.parametrize("case", [c for c in CASES if c[3] == c[4]])
+@pytest.mark.parametrize("case", CASES)
 def test_backward_matches_oracle(case, code):
     from byteir_amd import ops
     b, sq, sk, h, h_k, d, window = case
@@ -156,9 +158,13 @@ def test_backward_matches_oracle(case, code):
     # fp32 reference: gradients of plain float attention on the same (rounded) inputs
     o_h, lse_h = host(o), host(lse)
     rq, rk, rv, rD = oracle.flash_bwd(do, q, k, v, o_h, lse_h, scale, window, round_p=False)
+    # both sides round their result to the storage type: one storage ulp on top of the tolerance
+    # (with grouped heads dK and dV sum over several heads and exceed 2.56, where a bf16 ulp is 0.02)
+    ulp = 2.0 ** -10 if code == oracle.F16 else 2.0 ** -7
     for name, got, want in (("dq", dq, rq), ("dk", dk, rk), ("dv", dv, rv)):
-        err = np.abs(oracle.to_f32(host(got)) - oracle.to_f32(want)).max()
-        assert err <= ATOL, (name, float(err))
+        w32 = oracle.to_f32(want)
+        err = np.abs(oracle.to_f32(host(got)) - w32)
+        assert np.all(err <= ATOL + ulp * np.abs(w32)), (name, float(err.max()))
 
 
 STRIDED_CASES = [
@@ -167,7 +173,7 @@ STRIDED_CASES = [
     ("packed_qkv", 1, 130, 130, 2, 2, 96, (-1, -1)),
     ("bhsd", 2, 160, 224, 4, 4, 128, (-1, 0)),            # [b, h, s, d] storage viewed as [b, s, h, d]
     ("bhsd", 1, 100, 300, 3, 3, 32, (20, 5)),
-    ("bhsd", 2, 2, 1500, 8, 2, 128, (-1, -1)),            # decode-shaped, grouped heads (forward only)
+    ("bhsd", 2, 2, 1500, 8, 2, 128, (-1, -1)),            # decode-shaped, grouped heads
 ]
 
 
@@ -200,8 +206,6 @@ def test_strided_tensors(case, code):
     assert torch.equal(o_buf, o_dense) and torch.equal(lse, lse_dense)   # same kernel, same arithmetic
     _, _, o32 = oracle.flash_fwd(q, k, v, scale, window, round_p=False)
     assert np.abs(oracle.to_f32(host(o_buf.contiguous())) - o32).max() <= ATOL
-    if h != h_k:
-        return
     dq, dk, dv = ops.flash_attn_bwd(do_s, sq_, sk_, sv_, o_buf, lse, scale, window)
     assert dq.stride() == sq_.stride() and dk.stride() == sk_.stride()
     gq, gk, gv = ops.flash_attn_bwd(do_, dq_, dk_, dv_, o_dense, lse_dense, scale, window)

@@ -351,3 +351,22 @@ def test_dropout_backward_is_the_gradient_with_the_mask_held_fixed():
         np.testing.assert_allclose(got, want.numpy(), atol=3e-5, rtol=1e-4)
     # D is kept scaled by p_keep (flash_bwd_preprocess_kernel.h:124-128)
     np.testing.assert_allclose(dsm, np.einsum("bihd,bihd->bhi", do, o32) * p_keep, atol=1e-5, rtol=1e-5)
+
+
+def test_backward_with_grouped_heads_is_the_gradient():
+    """h_k < h: dK and dV of a key/value head are the sums over its query heads (torch autograd
+    through attention with repeated K / V heads)."""
+    rng = np.random.default_rng(8)
+    b, sq, sk, h, h_k, d, scale = 2, 20, 28, 6, 2, 8, 0.3
+    q, do = (rng.standard_normal((b, sq, h, d)).astype(np.float32) for _ in range(2))
+    k, v = (rng.standard_normal((b, sk, h_k, d)).astype(np.float32) for _ in range(2))
+    tq, tk, tv = (torch.from_numpy(t).double().requires_grad_(True) for t in (q, k, v))
+    ke, ve = (t.repeat_interleave(h // h_k, dim=2) for t in (tk, tv))
+    s = torch.einsum("bihd,bjhd->bhij", tq, ke) * scale
+    i, j = torch.arange(sq)[:, None], torch.arange(sk)[None, :]
+    s = s.masked_fill(j > i + sk - sq, float("-inf"))
+    torch.einsum("bhij,bjhd->bihd", torch.softmax(s, -1), ve).backward(torch.from_numpy(do).double())
+    o, lse, o32 = oracle.flash_fwd(q, k, v, scale, (-1, 0), round_p=False)
+    dq, dk, dv, _ = oracle.flash_bwd(do, q, k, v, o32, lse, scale, (-1, 0), round_p=False)
+    for got, want in ((dq, tq.grad), (dk, tk.grad), (dv, tv.grad)):
+        np.testing.assert_allclose(got, want.numpy(), atol=3e-5, rtol=1e-4)
