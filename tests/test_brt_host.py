@@ -276,3 +276,29 @@ def test_static_memory_plan_of_intermediates(session):
     assert session.get_intermediate_bytes("cuda") == 4096 + 4096   # 4000 B -> 4096, twice
     assert session.get_intermediate_bytes("cpu") == 0              # %s0 is never used
     assert session.get_intermediate_bytes("nowhere") == 0
+
+
+def test_product_code_never_touches_the_oracle():
+    """The oracle is test infrastructure: nothing under the shipped package may import, load or
+    name it, and the package has no CPU fallback to fall back on."""
+    root = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "byteir_amd")
+    for dirpath, _, files in os.walk(root):
+        for name in files:
+            if name.endswith((".py", ".hip", ".cc", ".h", ".c", ".cpp")):
+                text = open(os.path.join(dirpath, name), errors="replace").read()
+                assert "oracle" not in text.lower(), os.path.join(dirpath, name)
+
+
+def test_missing_kernel_library_fails_loudly(tmp_path, monkeypatch):
+    """Without its HIP library the package must raise, not compute something else."""
+    import importlib
+    from byteir_amd import _lib
+    fresh = importlib.reload(_lib)
+    try:
+        monkeypatch.setattr(fresh, "LIB_DIR", str(tmp_path), raising=False)
+        monkeypatch.setattr(fresh, "_kernels", None, raising=False)
+        monkeypatch.setattr(fresh, "_flash", None, raising=False)
+        with pytest.raises((OSError, RuntimeError)):
+            fresh.flash_attn()
+    finally:
+        importlib.reload(_lib)
