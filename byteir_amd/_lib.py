@@ -7,7 +7,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_DIR = os.path.join(_HERE, "lib")
 
 F32, F16, BF16 = 0, 1, 2
-REDUCE_SUM, REDUCE_MAX = 0, 1
+REDUCE_SUM, REDUCE_MAX, REDUCE_MIN, REDUCE_PROD, REDUCE_MEAN, REDUCE_SUMSQR = range(6)
 
 
 class LibraryMissing(RuntimeError):

@@ -264,6 +264,17 @@ void RegisterRocmOps(KernelRegistry *r) {
   reduce("ReduceSumOp_f16_f16", BRT_ROCM_REDUCE_SUM, BRT_ROCM_F16);
   reduce("ReduceMaxOp_f32_f32", BRT_ROCM_REDUCE_MAX, BRT_ROCM_F32);
   reduce("ReduceMaxOp_f16_f16", BRT_ROCM_REDUCE_MAX, BRT_ROCM_F16);
+  // The reference defines these four operators (reduction_helper.h:37-137) but instantiates no
+  // op kernel for them; the keys follow the naming of the registered ones
+  // (reduction/op_registration.cc:27-49).
+  reduce("ReduceMinOp_f32_f32", BRT_ROCM_REDUCE_MIN, BRT_ROCM_F32);
+  reduce("ReduceMinOp_f16_f16", BRT_ROCM_REDUCE_MIN, BRT_ROCM_F16);
+  reduce("ReduceProdOp_f32_f32", BRT_ROCM_REDUCE_PROD, BRT_ROCM_F32);
+  reduce("ReduceProdOp_f16_f16", BRT_ROCM_REDUCE_PROD, BRT_ROCM_F16);
+  reduce("ReduceMeanOp_f32_f32", BRT_ROCM_REDUCE_MEAN, BRT_ROCM_F32);
+  reduce("ReduceMeanOp_f16_f16", BRT_ROCM_REDUCE_MEAN, BRT_ROCM_F16);
+  reduce("ReduceSumSqrOp_f32_f32", BRT_ROCM_REDUCE_SUMSQR, BRT_ROCM_F32);
+  reduce("ReduceSumSqrOp_f16_f16", BRT_ROCM_REDUCE_SUMSQR, BRT_ROCM_F16);
   r->Register("byteir.softmax", [](const OpKernelInfo &info) -> std::shared_ptr<OpKernel> {
     return std::make_shared<SoftmaxOpKernel>(info);
   });

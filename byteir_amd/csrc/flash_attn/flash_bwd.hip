@@ -196,6 +196,12 @@ __global__ void __launch_bounds__(256, (D <= 64 && KB == 1) ? 2 : 1) dkdv_kernel
   if (p.wl >= 0) q_hi = min(p.sq, kvb0 + kKeys - off + p.wl);      // lo(q) = q+off-wl < kvb0+kKeys
   const int m_min = q_lo / kQTile;
   const int m_max = q_hi > 0 ? (q_hi + kQTile - 1) / kQTile : 0;
+  // the same for the wave's own keys [wkv0, wkv0 + 32*KB)
+  int qw_lo = 0, qw_hi = p.sq;
+  if (p.wr >= 0) qw_lo = max(0, wkv0 - off - p.wr);
+  if (p.wl >= 0) qw_hi = min(p.sq, wkv0 + 32 * KB - off + p.wl);
+  const int m_w_min = min(m_max, max(m_min, qw_lo / kQTile));
+  const int m_w_max = max(m_w_min, min(m_max, qw_hi > 0 ? (qw_hi + kQTile - 1) / kQTile : 0));
   const float c = p.scale_log2;
   // a key is kept for a query when key - (query + sk - sq) lies in [win_lo, win_lo + win_span]
   // (mask.h:160-200 of the reference; an unbounded side becomes +-2^30)
@@ -354,7 +360,19 @@ __global__ void __launch_bounds__(256, (D <= 64 && KB == 1) ? 2 : 1) dkdv_kernel
     __syncthreads();
   }
   int buf = 0, pbuf = 0;  // ring slots of tile m and of the tile of the pending unit
-  for (int m = m_min; m < m_max; ++m) {
+  int m = m_min;
+  // query tiles that the wave's own 32*KB keys cannot see (the first ones under a right window,
+  // the last ones under a left window): keep loading and meeting the barriers, compute nothing
+  auto idle_tile = [&]() {
+    const int buf1 = buf + 1 == kRing ? 0 : buf + 1;
+    const int buf2 = buf1 + 1 == kRing ? 0 : buf1 + 1;
+    __syncthreads();
+    if (m + 2 < m_max) lstore(buf2);
+    if (m + 3 < m_max) gload();
+    buf = buf1;
+  };
+  for (; m < m_w_min; ++m) idle_tile();
+  for (; m < m_w_max; ++m) {
     const int buf1 = buf + 1 == kRing ? 0 : buf + 1;
     const int buf2 = buf1 + 1 == kRing ? 0 : buf1 + 1;
     const int q0 = m * kQTile;
@@ -369,7 +387,8 @@ __global__ void __launch_bounds__(256, (D <= 64 && KB == 1) ? 2 : 1) dkdv_kernel
     pbuf = buf;
     buf = buf1;
   }
-  if (n_tiles > 0) part_c(Qs[pbuf], dOs[pbuf], 1, pb, dsb);
+  if (m_w_max > m_w_min) part_c(Qs[pbuf], dOs[pbuf], 1, pb, dsb);  // the last unit's C, before its slot is reused
+  for (; m < m_max; ++m) idle_tile();
   }
 
 #pragma unroll
@@ -587,6 +606,9 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) dq_kernel(const Params p
     part_a(ua);
     fetch(Ks[0], Vs[0], 1);
   }
+  // Under a right window (causal) the wave's rows see no key from w_hi_last on: it computes up
+  // to the tile that holds that key and only keeps loading and meeting the barriers afterwards.
+  const int n_w_max = min(n_max, max(n_min, (w_hi_last + kKvTile - 1) / kKvTile));
   int buf = 0;  // ring slot of tile t
   for (int t = n_min; t < n_max; ++t) {
     const int buf1 = buf + 1 == kRing ? 0 : buf + 1;
@@ -596,10 +618,12 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) dq_kernel(const Params p
     // tile t+2: registers -> the ring slot tile t-1 occupied; tile t+3 in flight
     if (t + 2 < n_max) lstore(buf2);
     if (t + 3 < n_max) gload();
-    // unit 0 of tile t (in ua); unit 1 is produced into ub; fragments of unit 0 of tile t+1
-    step(visibility(kv0), ua, kv0, buf, 0, ub, buf1, 0);
-    // unit 1 of tile t (in ub); unit 0 of tile t+1 into ua; fragments of its unit 1
-    step(visibility(kv0 + 32), ub, kv0 + 32, buf, 1, ua, buf1, 1);
+    if (t < n_w_max) {
+      // unit 0 of tile t (in ua); unit 1 is produced into ub; fragments of unit 0 of tile t+1
+      step(visibility(kv0), ua, kv0, buf, 0, ub, buf1, 0);
+      // unit 1 of tile t (in ub); unit 0 of tile t+1 into ua; fragments of its unit 1
+      step(visibility(kv0 + 32), ub, kv0 + 32, buf, 1, ua, buf1, 1);
+    }
     buf = buf1;
   }
 

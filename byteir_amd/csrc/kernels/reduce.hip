@@ -36,16 +36,47 @@ constexpr int kColWideW = 2, kColWideU = 2;  // column groups per lane and rows 
 constexpr int kBlock = 256;            // threads per workgroup (4 waves)
 constexpr uint64_t kFillThreads = 256ull * 1024;  // threads wanted in flight chip-wide
 
+// A fold operator: init, apply (associative up to rounding), map (applied to every element as
+// it is read from the tensor, never to partials) and finish (applied once, to the final value,
+// with the fold length as a float).
+struct FoldPlain {
+  static __device__ __forceinline__ float map(float x) { return x; }
+  static __device__ __forceinline__ float finish(float r, float) { return r; }
+};
 template <int OP> struct Fold;
-template <> struct Fold<BRT_ROCM_REDUCE_SUM> {
+template <> struct Fold<BRT_ROCM_REDUCE_SUM> : FoldPlain {
   static __device__ __forceinline__ float init() { return 0.f; }
   static __device__ __forceinline__ float apply(float l, float r) { return l + r; }
 };
-template <> struct Fold<BRT_ROCM_REDUCE_MAX> {
+template <> struct Fold<BRT_ROCM_REDUCE_MAX> : FoldPlain {
   static __device__ __forceinline__ float init() { return -INFINITY; }
   static __device__ __forceinline__ float apply(float l, float r) {
     return (l != l || l > r) ? l : r;  // NaN on either side wins
   }
+};
+template <> struct Fold<BRT_ROCM_REDUCE_MIN> : FoldPlain {
+  static __device__ __forceinline__ float init() { return INFINITY; }
+  static __device__ __forceinline__ float apply(float l, float r) {
+    return (l != l || l < r) ? l : r;  // NaN on either side wins
+  }
+};
+template <> struct Fold<BRT_ROCM_REDUCE_PROD> : FoldPlain {
+  static __device__ __forceinline__ float init() { return 1.f; }
+  static __device__ __forceinline__ float apply(float l, float r) { return l * r; }
+};
+template <> struct Fold<BRT_ROCM_REDUCE_MEAN> : Fold<BRT_ROCM_REDUCE_SUM> {
+  static __device__ __forceinline__ float finish(float r, float len) { return r / len; }
+};
+template <> struct Fold<BRT_ROCM_REDUCE_SUMSQR> : Fold<BRT_ROCM_REDUCE_SUM> {
+  static __device__ __forceinline__ float map(float x) { return x * x; }
+};
+// With partials in a workspace the first pass maps and the second one finishes.
+template <int OP> struct Passes { static constexpr int first = OP, second = OP; };
+template <> struct Passes<BRT_ROCM_REDUCE_MEAN> {
+  static constexpr int first = BRT_ROCM_REDUCE_SUM, second = BRT_ROCM_REDUCE_MEAN;
+};
+template <> struct Passes<BRT_ROCM_REDUCE_SUMSQR> {
+  static constexpr int first = BRT_ROCM_REDUCE_SUMSQR, second = BRT_ROCM_REDUCE_SUM;
 };
 
 // ---- typed loads into float -----------------------------------------------------------
@@ -93,7 +124,7 @@ template <int OP> __device__ __forceinline__ float wave_fold(float r, int width)
 template <typename T, typename TO, int OP, int VEC, int G>
 __global__ void __launch_bounds__(kBlock)
 reduce_row_kernel(const T *__restrict__ in, TO *__restrict__ out, uint64_t units, uint64_t B,
-                  uint32_t S, uint64_t seg_len) {
+                  uint32_t S, uint64_t seg_len, float len) {
   constexpr int GPB = kBlock / G;
   constexpr int U = kRowU;
   const int lane = threadIdx.x % G;
@@ -118,13 +149,13 @@ reduce_row_kernel(const T *__restrict__ in, TO *__restrict__ out, uint64_t units
 #pragma unroll
     for (int u = 0; u < U; ++u)
 #pragma unroll
-      for (int k = 0; k < VEC; ++k) acc[u] = Fold<OP>::apply(acc[u], v[u][k]);
+      for (int k = 0; k < VEC; ++k) acc[u] = Fold<OP>::apply(acc[u], Fold<OP>::map(v[u][k]));
   }
   for (; i < end; i += step) {
     float v[VEC];
     Loader<T, VEC>::load(row + i, v);
 #pragma unroll
-    for (int k = 0; k < VEC; ++k) acc[0] = Fold<OP>::apply(acc[0], v[k]);
+    for (int k = 0; k < VEC; ++k) acc[0] = Fold<OP>::apply(acc[0], Fold<OP>::map(v[k]));
   }
   float r = acc[0];
 #pragma unroll
@@ -139,7 +170,7 @@ reduce_row_kernel(const T *__restrict__ in, TO *__restrict__ out, uint64_t units
     __syncthreads();
     r = Fold<OP>::apply(Fold<OP>::apply(part[0], part[1]), Fold<OP>::apply(part[2], part[3]));
   }
-  if (valid && lane == 0) out[unit] = to_out<TO>(r);
+  if (valid && lane == 0) out[unit] = to_out<TO>(Fold<OP>::finish(r, len));
 }
 
 // ---- columns: C > 1 ---------------------------------------------------------------------
@@ -148,7 +179,7 @@ reduce_row_kernel(const T *__restrict__ in, TO *__restrict__ out, uint64_t units
 template <typename T, typename TO, int OP, int VEC, int TX>
 __global__ void __launch_bounds__(kBlock)
 reduce_col_kernel(const T *__restrict__ in, TO *__restrict__ out, uint64_t B, uint64_t C,
-                  uint32_t S, uint64_t seg_rows, uint32_t col_tiles) {
+                  uint32_t S, uint64_t seg_rows, uint32_t col_tiles, float len) {
   constexpr int TY = kBlock / TX;
   constexpr int U = kColU;
   __shared__ float part[TY][TX * VEC + 1];
@@ -176,13 +207,13 @@ reduce_col_kernel(const T *__restrict__ in, TO *__restrict__ out, uint64_t B, ui
 #pragma unroll
       for (int u = 0; u < U; ++u)
 #pragma unroll
-        for (int k = 0; k < VEC; ++k) acc[k] = Fold<OP>::apply(acc[k], v[u][k]);
+        for (int k = 0; k < VEC; ++k) acc[k] = Fold<OP>::apply(acc[k], Fold<OP>::map(v[u][k]));
     }
     for (; r < r1; r += TY) {
       float v[VEC];
       Loader<T, VEC>::load(p + r * C, v);
 #pragma unroll
-      for (int k = 0; k < VEC; ++k) acc[k] = Fold<OP>::apply(acc[k], v[k]);
+      for (int k = 0; k < VEC; ++k) acc[k] = Fold<OP>::apply(acc[k], Fold<OP>::map(v[k]));
     }
   }
 #pragma unroll
@@ -194,7 +225,7 @@ reduce_col_kernel(const T *__restrict__ in, TO *__restrict__ out, uint64_t B, ui
 #pragma unroll 4
     for (int y = 1; y < TY; ++y) r = Fold<OP>::apply(r, part[y][j]);
     const uint64_t cj = (uint64_t)tile * TX * VEC + j;
-    if (cj < C) out[(a * S + s) * C + cj] = to_out<TO>(r);
+    if (cj < C) out[(a * S + s) * C + cj] = to_out<TO>(Fold<OP>::finish(r, len));
   }
 }
 
@@ -206,7 +237,7 @@ reduce_col_kernel(const T *__restrict__ in, TO *__restrict__ out, uint64_t B, ui
 template <typename T, typename TO, int OP, int VEC, int W, int U>
 __global__ void __launch_bounds__(kBlock)
 reduce_colwide_kernel(const T *__restrict__ in, TO *__restrict__ out, uint64_t B, uint64_t C,
-                      uint32_t S, uint64_t seg_rows, uint32_t col_tiles) {
+                      uint32_t S, uint64_t seg_rows, uint32_t col_tiles, float len) {
   uint64_t bid = blockIdx.x;
   const uint32_t tile = bid % col_tiles; bid /= col_tiles;
   const uint32_t s = bid % S;
@@ -243,7 +274,7 @@ reduce_colwide_kernel(const T *__restrict__ in, TO *__restrict__ out, uint64_t B
         for (int w = 0; w < W; ++w)
           if (kFull || ok[w]) {
 #pragma unroll
-            for (int k = 0; k < VEC; ++k) acc[w][k] = Fold<OP>::apply(acc[w][k], v[u][w][k]);
+            for (int k = 0; k < VEC; ++k) acc[w][k] = Fold<OP>::apply(acc[w][k], Fold<OP>::map(v[u][w][k]));
           }
     }
     for (; r < r1; ++r) {
@@ -253,14 +284,14 @@ reduce_colwide_kernel(const T *__restrict__ in, TO *__restrict__ out, uint64_t B
           float v[VEC];
           Loader<T, VEC>::load(p + r * C + w * kGroupStep, v);
 #pragma unroll
-          for (int k = 0; k < VEC; ++k) acc[w][k] = Fold<OP>::apply(acc[w][k], v[k]);
+          for (int k = 0; k < VEC; ++k) acc[w][k] = Fold<OP>::apply(acc[w][k], Fold<OP>::map(v[k]));
         }
     }
 #pragma unroll
     for (int w = 0; w < W; ++w)
       if (kFull || ok[w]) {
 #pragma unroll
-        for (int k = 0; k < VEC; ++k) o[w * kGroupStep + k] = to_out<TO>(acc[w][k]);
+        for (int k = 0; k < VEC; ++k) o[w * kGroupStep + k] = to_out<TO>(Fold<OP>::finish(acc[w][k], len));
       }
   };
   if (((uint64_t)tile + 1) * W * kGroupStep <= C) fold(std::true_type{});
@@ -338,7 +369,7 @@ inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 
 
 template <typename T, typename TO, int OP>
 hipError_t launch(const Plan &p, const T *in, TO *out, uint64_t A, uint64_t B, uint64_t C,
-                  hipStream_t stream) {
+                  float len, hipStream_t stream) {
   constexpr int VF = sizeof(T) == 4 ? 4 : 8;
   const bool vec = p.vec > 1 && aligned16(in);
   if (p.kind == 1) {
@@ -347,8 +378,8 @@ hipError_t launch(const Plan &p, const T *in, TO *out, uint64_t A, uint64_t B, u
     if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
     const dim3 grid((unsigned)blocks), block(kBlock);
 #define ROW(G)                                                                                   \
-  if (vec) reduce_row_kernel<T, TO, OP, VF, G><<<grid, block, 0, stream>>>(in, out, units, B, p.S, p.seg); \
-  else reduce_row_kernel<T, TO, OP, 1, G><<<grid, block, 0, stream>>>(in, out, units, B, p.S, p.seg)
+  if (vec) reduce_row_kernel<T, TO, OP, VF, G><<<grid, block, 0, stream>>>(in, out, units, B, p.S, p.seg, len); \
+  else reduce_row_kernel<T, TO, OP, 1, G><<<grid, block, 0, stream>>>(in, out, units, B, p.S, p.seg, len)
     switch (p.g) {
     case 4: ROW(4); break;
     case 16: ROW(16); break;
@@ -367,12 +398,12 @@ hipError_t launch(const Plan &p, const T *in, TO *out, uint64_t A, uint64_t B, u
   if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
   const dim3 grid((unsigned)blocks), block(kBlock);
   if (p.kind == 3 && vec) {
-    reduce_colwide_kernel<T, TO, OP, VF, kColWideW, kColWideU><<<grid, block, 0, stream>>>(in, out, B, C, p.S, p.seg, col_tiles);
+    reduce_colwide_kernel<T, TO, OP, VF, kColWideW, kColWideU><<<grid, block, 0, stream>>>(in, out, B, C, p.S, p.seg, col_tiles, len);
     return hipGetLastError();
   }
 #define COL(TX)                                                                                  \
-  if (vec) reduce_col_kernel<T, TO, OP, VF, TX><<<grid, block, 0, stream>>>(in, out, B, C, p.S, p.seg, col_tiles); \
-  else reduce_col_kernel<T, TO, OP, 1, TX><<<grid, block, 0, stream>>>(in, out, B, C, p.S, p.seg, col_tiles)
+  if (vec) reduce_col_kernel<T, TO, OP, VF, TX><<<grid, block, 0, stream>>>(in, out, B, C, p.S, p.seg, col_tiles, len); \
+  else reduce_col_kernel<T, TO, OP, 1, TX><<<grid, block, 0, stream>>>(in, out, B, C, p.S, p.seg, col_tiles, len)
   switch (tx) {
   case 8: COL(8); break;
   case 32: COL(32); break;
@@ -387,19 +418,20 @@ template <typename T, int OP>
 hipError_t run(const T *in, T *out, uint64_t A, uint64_t B, uint64_t C, void *ws, size_t ws_bytes,
                int dtype, hipStream_t stream, hipEvent_t first_pass_done) {
   const Plan p = make_plan(dtype, A, B, C, true);
+  const float len = static_cast<float>(B);  // MeanOp divides by static_cast<wtype>(B)
   if (p.S == 1) {
-    const hipError_t e = launch<T, T, OP>(p, in, out, A, B, C, stream);
+    const hipError_t e = launch<T, T, OP>(p, in, out, A, B, C, len, stream);
     if (e == hipSuccess && first_pass_done) return hipEventRecord(first_pass_done, stream);
     return e;
   }
   const size_t need = sizeof(float) * A * p.S * C;
   if (ws == nullptr || ws_bytes < need) return hipErrorInvalidValue;
   float *part = static_cast<float *>(ws);
-  hipError_t e = launch<T, float, OP>(p, in, part, A, B, C, stream);
+  hipError_t e = launch<T, float, Passes<OP>::first>(p, in, part, A, B, C, len, stream);
   if (e != hipSuccess) return e;
   if (first_pass_done && (e = hipEventRecord(first_pass_done, stream)) != hipSuccess) return e;
   const Plan p2 = make_plan(BRT_ROCM_F32, A, p.S, C, false);
-  return launch<float, T, OP>(p2, part, out, A, p.S, C, stream);
+  return launch<float, T, Passes<OP>::second>(p2, part, out, A, p.S, C, len, stream);
 }
 
 }  // namespace
@@ -415,7 +447,7 @@ extern "C" int brt_rocm_reduce_ex(int op, int dtype, const void *input, void *ou
                                   void *stream_, void *first_pass_done_) {
   hipStream_t stream = static_cast<hipStream_t>(stream_);
   hipEvent_t first_pass_done = static_cast<hipEvent_t>(first_pass_done_);
-  if ((op != BRT_ROCM_REDUCE_SUM && op != BRT_ROCM_REDUCE_MAX) ||
+  if (op < BRT_ROCM_REDUCE_SUM || op > BRT_ROCM_REDUCE_SUMSQR ||
       (dtype != BRT_ROCM_F32 && dtype != BRT_ROCM_F16))
     return hipErrorInvalidValue;
   const size_t es = dtype == BRT_ROCM_F32 ? 4 : 2;
@@ -425,18 +457,25 @@ extern "C" int brt_rocm_reduce_ex(int op, int dtype, const void *input, void *ou
     return hipMemcpyAsync(output, input, C * es, hipMemcpyDeviceToDevice, stream);
   }
   if (!input || !output) return hipErrorInvalidValue;
+#define RUN(T, OP) \
+  case OP: return run<T, OP>(in, out, A, B, C, workspace, workspace_bytes, dtype, stream, first_pass_done)
+#define RUN_ALL(T)                                                                               \
+  switch (op) {                                                                                  \
+    RUN(T, BRT_ROCM_REDUCE_SUM); RUN(T, BRT_ROCM_REDUCE_MAX); RUN(T, BRT_ROCM_REDUCE_MIN);       \
+    RUN(T, BRT_ROCM_REDUCE_PROD); RUN(T, BRT_ROCM_REDUCE_MEAN); RUN(T, BRT_ROCM_REDUCE_SUMSQR);  \
+  }
   if (dtype == BRT_ROCM_F32) {
     const float *in = static_cast<const float *>(input);
     float *out = static_cast<float *>(output);
-    return op == BRT_ROCM_REDUCE_SUM
-               ? run<float, BRT_ROCM_REDUCE_SUM>(in, out, A, B, C, workspace, workspace_bytes, dtype, stream, first_pass_done)
-               : run<float, BRT_ROCM_REDUCE_MAX>(in, out, A, B, C, workspace, workspace_bytes, dtype, stream, first_pass_done);
+    RUN_ALL(float)
+  } else {
+    const __half *in = static_cast<const __half *>(input);
+    __half *out = static_cast<__half *>(output);
+    RUN_ALL(__half)
   }
-  const __half *in = static_cast<const __half *>(input);
-  __half *out = static_cast<__half *>(output);
-  return op == BRT_ROCM_REDUCE_SUM
-             ? run<__half, BRT_ROCM_REDUCE_SUM>(in, out, A, B, C, workspace, workspace_bytes, dtype, stream, first_pass_done)
-             : run<__half, BRT_ROCM_REDUCE_MAX>(in, out, A, B, C, workspace, workspace_bytes, dtype, stream, first_pass_done);
+#undef RUN_ALL
+#undef RUN
+  return hipErrorInvalidValue;
 }
 
 extern "C" int brt_rocm_reduce(int op, int dtype, const void *input, void *output, size_t A,

@@ -77,7 +77,8 @@ def reduce_abc(op, x, out, A, B, C, workspace=None, stream=None):
 
 
 def reduce(op, x, dims, stream=None):
-    """ReduceSumOp / ReduceMaxOp over `dims` of a dense tensor (op: _lib.REDUCE_SUM / REDUCE_MAX)."""
+    """Reduce<Op>Op over `dims` of a dense tensor (op: _lib.REDUCE_SUM / MAX / MIN / PROD / MEAN /
+    SUMSQR)."""
     out_shape = deduce_output_shape(list(x.shape), list(dims))
     A, B, C = canonicalize_reduce(list(x.shape), out_shape, list(dims))
     out = torch.empty(out_shape, dtype=x.dtype, device=x.device)

@@ -23,9 +23,20 @@ extern "C" {
 /* element types (the subset of brt::DTypeEnum, runtime/include/brt/core/framework/dtype.h,
  * that the op kernels on this path accept) */
 enum { BRT_ROCM_F32 = 0, BRT_ROCM_F16 = 1, BRT_ROCM_BF16 = 2 };
-/* fold operators: kernel::reduction::SumOp / MaxOp,
- * runtime/lib/backends/cuda/providers/default/reduction/kernels/reduction_helper.h:18-36,140-179 */
-enum { BRT_ROCM_REDUCE_SUM = 0, BRT_ROCM_REDUCE_MAX = 1 };
+/* fold operators of
+ * runtime/lib/backends/cuda/providers/default/reduction/kernels/reduction_helper.h:
+ * SumOp :18-36, MaxOp :140-179 (the two the reference registers op kernels for) and MinOp
+ * :98-137, ProdOp :80-95, MeanOp :37-56 (sum, then divided by float(B) at the store), SumSqrOp
+ * :58-77 (elements squared in float as they are read), which the reference defines but never
+ * instantiates.  Max and Min let a NaN on either side win. */
+enum {
+  BRT_ROCM_REDUCE_SUM = 0,
+  BRT_ROCM_REDUCE_MAX = 1,
+  BRT_ROCM_REDUCE_MIN = 2,
+  BRT_ROCM_REDUCE_PROD = 3,
+  BRT_ROCM_REDUCE_MEAN = 4,
+  BRT_ROCM_REDUCE_SUMSQR = 5
+};
 
 /* library identification; returns a static string */
 const char *brt_rocm_version(void);

@@ -17,7 +17,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "liboracle.so")
 
 F32, F16, BF16 = 0, 1, 2
-SUM, MAX = 0, 1
+SUM, MAX, MIN, PROD, MEAN, SUMSQR = range(6)
 
 
 def build(force=False):

@@ -213,11 +213,28 @@ uint64_t oracle_reference_workspace_bytes(uint64_t A, uint64_t B, uint64_t C, ui
 /* SumOp::apply / MaxOp<...,float>::apply, .../reduction/kernels/reduction_helper.h:18-36,158-179 */
 static inline float op_sum(float l, float r) { return l + r; }
 static inline float op_max(float l, float r) { return (isnan(l) || l > r) ? l : r; }
+/* The operators the reference defines without registering an op kernel for them: MeanOp
+ * :37-56 (sum; the store divides by float(B)), SumSqrOp :58-77 (read squares in float), ProdOp
+ * :80-95 (init 1), MinOp<...,float> :116-137 (init +inf, NaN from either side wins). */
+static inline float fold_init(int op) {
+  return op == 1 ? -INFINITY : op == 2 ? INFINITY : op == 3 ? 1.f : 0.f;
+}
+static inline float fold_map(int op, float x) { return op == 5 ? x * x : x; }
+static inline float fold_apply(int op, float l, float r) {
+  switch (op) {
+  case 1: return op_max(l, r);
+  case 2: return (isnan(l) || l < r) ? l : r;
+  case 3: return l * r;
+  default: return l + r;
+  }
+}
+static inline float fold_finish(int op, float r, uint64_t B) { return op == 4 ? r / (float)B : r; }
 
 /* out[a,c] = fold_b in[a,b,c] as one left-to-right chain per output in the working type
  * float, the order of the reference's own test oracle GoldenReduction
  * (runtime/test/backends/cuda/providers/default/kernel/reduction_test.cc:66-92) and of the
- * linalg loop nest the CPU path executes.  op: 0 = sum (init 0), 1 = max (init -inf).
+ * linalg loop nest the CPU path executes.  op: 0 = sum (init 0), 1 = max (init -inf),
+ * 2 = min, 3 = prod, 4 = mean, 5 = sum of squares.
  * dtype 0 = f32, 1 = f16 (accumulated in float, reduce_impl.h:64-69).
  * A == 0 means "plain copy of C elements" (reduce_impl.h:71-74). */
 void oracle_reduce(int op, int dtype, const void *in, void *out, uint64_t A, uint64_t B,
@@ -227,7 +244,7 @@ void oracle_reduce(int op, int dtype, const void *in, void *out, uint64_t A, uin
     memcpy(out, in, C * es);
     return;
   }
-  if (dtype == 0 && C == 1) { /* tight loop for the timed baseline */
+  if (dtype == 0 && C == 1 && op <= 1) { /* tight loop for the timed baseline */
     const float *x = (const float *)in;
     float *y = (float *)out;
 #pragma omp parallel for num_threads(g_threads) schedule(static)
@@ -238,7 +255,7 @@ void oracle_reduce(int op, int dtype, const void *in, void *out, uint64_t A, uin
     }
     return;
   }
-  if (dtype == 0) {
+  if (dtype == 0 && op <= 1) {
     const float *x = (const float *)in;
     float *y = (float *)out;
     for (uint64_t a = 0; a < A; ++a) {
@@ -261,12 +278,12 @@ void oracle_reduce(int op, int dtype, const void *in, void *out, uint64_t A, uin
   }
   for (uint64_t a = 0; a < A; ++a)
     for (uint64_t c = 0; c < C; ++c) {
-      float acc = op == 0 ? 0.f : -INFINITY;
+      float acc = fold_init(op);
       for (uint64_t b = 0; b < B; ++b) {
-        float v = load_elem(in, (a * B + b) * C + c, dtype);
-        acc = op == 0 ? op_sum(acc, v) : op_max(acc, v);
+        float v = fold_map(op, load_elem(in, (a * B + b) * C + c, dtype));
+        acc = fold_apply(op, acc, v);
       }
-      store_elem(out, a * C + c, dtype, acc);
+      store_elem(out, a * C + c, dtype, fold_finish(op, acc, B));
     }
 }
 

@@ -102,8 +102,8 @@ def test_registry_has_the_reference_keys(session):
 
 def test_unknown_op_fails_at_load(session):
     # execution_plan.cc:435-438: "No providers support Op <key>"
-    text = reduction_module("cuda", [4, 8], [1], "ReduceProdOp_f32_f32")
-    with pytest.raises(RuntimeError, match="No providers support Op ReduceProdOp_f32_f32"):
+    text = reduction_module("cuda", [4, 8], [1], "ReduceArgMaxOp_f32_f32")
+    with pytest.raises(RuntimeError, match="No providers support Op ReduceArgMaxOp_f32_f32"):
         session.load_from_memory(text)
 
 

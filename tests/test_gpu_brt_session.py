@@ -57,6 +57,29 @@ def test_reduction_through_session_twice(session, shape, dims, op_name, op):
     req.close()
 
 
+@pytest.mark.parametrize("op_name,op", [("ReduceMinOp_f32_f32", oracle.MIN), ("ReduceProdOp_f32_f32", oracle.PROD),
+                                        ("ReduceMeanOp_f32_f32", oracle.MEAN), ("ReduceSumSqrOp_f32_f32", oracle.SUMSQR)])
+@pytest.mark.parametrize("shape,dims", [((2, 16, 8, 64), (1, 2)), ((3000, 520), (0,))])
+def test_unregistered_reference_operators_through_session(session, shape, dims, op_name, op):
+    """Keys for the operators reduction_helper.h:37-137 defines and no reference op kernel uses."""
+    session.load_from_memory(reduction_module("cuda", list(shape), list(dims), op_name))
+    req = session.new_request_context()
+    rng = np.random.default_rng(9)
+    if op == oracle.PROD:  # signs and rare factors of two: exact in any order
+        xs = np.where(rng.random(shape) < 0.005, 2.0, 1.0) * rng.choice(np.array([-1.0, 1.0]), size=shape)
+    else:
+        xs = rng.integers(-2, 3, size=shape)
+    x = dev(xs.astype(np.float32))
+    y = torch.full(oracle.deduce_output_shape(shape, dims), -7.0, device="cuda")
+    req.bind_arg(0, x.data_ptr())
+    req.bind_arg(1, y.data_ptr())
+    req.finish_io_binding()
+    req.run()
+    req.sync()
+    assert np.array_equal(host(y), oracle.reduce_op(op, host(x), dims))
+    req.close()
+
+
 @pytest.mark.parametrize("op_name", ["ReduceSumOp_f32_f32", "ReduceMaxOp_f32_f32"])
 def test_nan_propagation_through_session(session, op_name):
     # reduction_test.cc:182-215: 1024 elements, NaN first; runtime-allocated arguments

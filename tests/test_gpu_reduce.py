@@ -101,6 +101,72 @@ def test_reduce_f16(shape, dims, op):
         assert np.all(np.abs(got.astype(np.float64) - want) <= 2.0 ** -10 * np.abs(want) + 1e-6 * sabs + 1e-7)
 
 
+# ---- MinOp, ProdOp, MeanOp, SumSqrOp (reduction_helper.h:37-137) ------------------------------
+OTHER_OPS = [oracle.MIN, oracle.PROD, oracle.MEAN, oracle.SUMSQR]
+OTHER_SHAPES = REF_CASES + [
+    ((7, 13), (1,)), ((7, 13), (0,)), ((3, 1000003), (1,)), ((1000003, 3), (0,)), ((5, 333, 7), (1,)),
+    ((1 << 20,), (0,)), ((4096, 64), (0,)), ((16, 2049, 260), (1,)), ((4096, 8192), (0,)), ((300, 2600), (0,)),
+]
+
+
+def exact_input(op, shape, dims, rng):
+    """Values for which every partial result of the fold is exact in float whatever the order,
+    so that the sequential oracle is the expected value bit for bit: small integers for
+    min / mean / sum of squares; for the product, signs and a few factors of 2 and 1/2."""
+    if op != oracle.PROD:
+        return rng.integers(-2, 3, size=shape).astype(np.float32)
+    fold = int(np.prod([shape[d] for d in dims]))
+    e = rng.integers(-1, 2, size=shape) * (rng.random(shape) < min(1.0, 24.0 / fold))
+    return (np.exp2(e) * rng.choice(np.array([-1.0, 1.0]), size=shape)).astype(np.float32)
+
+
+@pytest.mark.parametrize("shape,dims", OTHER_SHAPES)
+@pytest.mark.parametrize("op", OTHER_OPS)
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_other_operators_bit_exact_on_exact_inputs(shape, dims, op, dtype):
+    from byteir_amd import ops
+    if dtype == np.float16 and int(np.prod(shape)) > (1 << 22):
+        pytest.skip("the scalar f16 oracle is slow at this size; f32 covers the shape")
+    rng = np.random.default_rng(abs(hash((shape, dims, op))) % (2 ** 32))
+    x = exact_input(op, shape, dims, rng).astype(dtype)
+    got = host(ops.reduce(op, dev(x), dims))
+    want = oracle.reduce_op(op, x, dims)
+    assert got.dtype == dtype and got.shape == want.shape
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("shape,dims", [((64, 4096), (1,)), ((4096, 64), (0,)), ((3, 100003), (1,)), ((5000, 2600), (0,))])
+def test_other_operators_on_real_values(shape, dims):
+    """1e-5 relative against the fp64 fold (the bar of the registered sum)."""
+    from byteir_amd import ops
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal(shape).astype(np.float32)
+    x64 = x.astype(np.float64)
+    n = int(np.prod([shape[d] for d in dims]))
+    got = host(ops.reduce(oracle.SUMSQR, dev(x), dims)).astype(np.float64)
+    np.testing.assert_allclose(got, (x64 * x64).sum(axis=dims), rtol=1e-5)
+    got = host(ops.reduce(oracle.MEAN, dev(x), dims)).astype(np.float64)
+    assert np.all(np.abs(got - x64.mean(axis=dims)) <= 1e-5 * 1e-2 * np.abs(x64).sum(axis=dims) / n)
+    assert np.array_equal(host(ops.reduce(oracle.MIN, dev(x), dims)), x.min(axis=dims))
+    # factors near one: the product stays in range and its rounding error is that of a
+    # chain of n multiplications in any order, at most n * 2^-24 relative
+    y = (1.0 + 1e-3 * rng.standard_normal(shape)).astype(np.float32)
+    got = host(ops.reduce(oracle.PROD, dev(y), dims)).astype(np.float64)
+    np.testing.assert_allclose(got, y.astype(np.float64).prod(axis=dims), rtol=max(1e-5, n * 2.0 ** -24))
+
+
+def test_min_nan_and_infinities():
+    from byteir_amd import ops
+    x = np.full((3, 70000), np.inf, dtype=np.float32)
+    assert np.array_equal(host(ops.reduce(oracle.MIN, dev(x), (1,))), np.full(3, np.inf, np.float32))
+    x[1, 69999] = -np.inf
+    x[2, 12345] = np.nan
+    got = host(ops.reduce(oracle.MIN, dev(x), (1,)))
+    assert got[0] == np.inf and got[1] == -np.inf and np.isnan(got[2])
+    got = host(ops.reduce(oracle.MIN, dev(x), (0,)))
+    assert np.isnan(got[12345]) and got[69999] == -np.inf and got[0] == np.inf
+
+
 @pytest.mark.parametrize("shape,dims", [((1000, 4096), (0,)), ((1000, 4096), (1,)), ((3000, 64), (0,)), ((2, 500, 2048), (1,)),
                                         ((40000, 8), (0,))])
 @pytest.mark.parametrize("op", [oracle.SUM, oracle.MAX])

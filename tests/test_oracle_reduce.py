@@ -148,3 +148,41 @@ def test_half_conversions_exhaustive():
     finite = np.isfinite(vals)
     assert np.array_equal(oracle.to_bf16_bits(vals)[finite], want[finite])
     assert np.array_equal(oracle.from_bf16_bits(want), (want.astype(np.uint32) << 16).view(np.float32))
+
+
+# ---- the operators the reference defines but never registers (reduction_helper.h:37-137) -------
+def test_min_prod_mean_sumsqr_against_closed_forms():
+    """Pins chosen so that a swapped init, a missing division, a square of the sum instead of a
+    sum of squares or a min that behaves like max each fail: integers small enough that every
+    float operation is exact, so numpy's integer arithmetic is the expected value bit for bit."""
+    rng = np.random.default_rng(11)
+    xi = rng.integers(-9, 10, size=(6, 64, 5))
+    x = xi.astype(np.float32)
+    assert np.array_equal(oracle.reduce_op(oracle.MIN, x, (1,)), xi.min(axis=1).astype(np.float32))
+    assert np.array_equal(oracle.reduce_op(oracle.SUMSQR, x, (1,)), (xi * xi).sum(axis=1).astype(np.float32))
+    # 64 is a power of two: sum / 64 is exact
+    assert np.array_equal(oracle.reduce_op(oracle.MEAN, x, (1,)), (xi.sum(axis=1) / 64.0).astype(np.float32))
+    # products of +-1 and +-2 stay exact powers of two
+    pi = rng.choice(np.array([-2, -1, 1, 2]), size=(4, 40, 3))
+    assert np.array_equal(oracle.reduce_op(oracle.PROD, pi.astype(np.float32), (1,)),
+                          pi.astype(np.float64).prod(axis=1).astype(np.float32))
+    # a fold length that is no power of two: one float division of the float sum by float(B)
+    y = rng.integers(-50, 50, size=(3, 7)).astype(np.float32)
+    want = (y.sum(axis=1, dtype=np.float32) / np.float32(7)).astype(np.float32)
+    assert np.array_equal(oracle.reduce_op(oracle.MEAN, y, (1,)), want)
+
+
+def test_min_identity_nan_and_empty_product():
+    x = np.full((2, 9), np.inf, dtype=np.float32)
+    assert np.array_equal(oracle.reduce_op(oracle.MIN, x, (1,)), np.full(2, np.inf, np.float32))
+    x[1, 4] = -np.inf
+    assert oracle.reduce_op(oracle.MIN, x, (1,))[1] == -np.inf
+    for pos in (0, 4, 8):  # NaN from either side of apply wins
+        z = np.arange(9, dtype=np.float32)
+        z[pos] = np.nan
+        assert np.isnan(oracle.reduce_op(oracle.MIN, z, (0,)))
+        assert np.isnan(oracle.reduce_op(oracle.PROD, z, (0,)))
+    # f16 storage: squares and the chain are float, one rounding at the store
+    h = np.array([[255.0, 3.0, 0.5]], dtype=np.float16)  # 255^2 = 65025 rounds to 65024 in f16
+    got = oracle.reduce_op(oracle.SUMSQR, h, (1,))
+    assert got.dtype == np.float16 and got[0] == np.float16(65025.0 + 9.0 + 0.25)
