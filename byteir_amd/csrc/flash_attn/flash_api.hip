@@ -168,12 +168,17 @@ int flash_attn_bwd_checked(void **tensors, const void *extra_args, int dtype, vo
   p.dsoftmax = static_cast<float *>(tensors[10]);
   if (p.b == 0) return 0;
   if (p.drop && !p.rng_state) return fail("p_dropout > 0 needs the rng_state tensor {seed, offset}");
-  const void *need[] = {p.dout, p.q, p.k, p.v, p.o, p.dq, p.dk, p.dv};
-  for (const void *t : need) {
-    if (!t) return fail("null tensor pointer");
+  // a side without rows (seqlen_q == 0 or seqlen_k == 0) may come as null pointers
+  const void *q_side[] = {p.dout, p.q, p.o, p.dq}, *k_side[] = {p.k, p.v, p.dk, p.dv};
+  if (p.sq > 0 && (!p.lse || !p.dsoftmax)) return fail("null tensor pointer");
+  for (const void *t : q_side) {
+    if (!t && p.sq > 0) return fail("null tensor pointer");
     if (!aligned16(t)) return fail("tensors must be 16-byte aligned");
   }
-  if (!p.lse || !p.dsoftmax) return fail("null tensor pointer");
+  for (const void *t : k_side) {
+    if (!t && p.sk > 0) return fail("null tensor pointer");
+    if (!aligned16(t)) return fail("tensors must be 16-byte aligned");
+  }
   return fa::launch_bwd(p, dtype, static_cast<hipStream_t>(stream));
 }
 

@@ -145,6 +145,39 @@ def test_forward_matches_oracle(case, code):
     assert np.all(np.abs(got - ref_r) <= tight * np.abs(ref_r) + 2e-3)
 
 
+@pytest.mark.parametrize("d", [64, 80, 128])
+@pytest.mark.parametrize("sq", [3, 200])
+def test_no_keys_at_all(d, sq):
+    """seqlen_k = 0: every row keeps no key, so O = 0 and LSE = +inf (flash_fwd_kernel.h:70-104);
+    backward: dQ = 0.  The key-side tensors have no storage (null pointers)."""
+    from byteir_amd import ops
+    b, h = 2, 4
+    q = torch.randn((b, sq, h, d), device="cuda").half()
+    k = torch.empty((b, 0, h, d), device="cuda", dtype=torch.float16)
+    v = torch.empty_like(k)
+    o, lse = ops.flash_attn_fwd(q, k, v, 0.3, (-1, -1))
+    assert torch.all(o == 0) and torch.all(torch.isposinf(lse))
+    dq, dk, dv = ops.flash_attn_bwd(torch.randn_like(q), q, k, v, o, lse, 0.3, (-1, -1))
+    assert dq.shape == q.shape and torch.all(dq == 0) and dk.numel() == 0 and dv.numel() == 0
+
+
+@pytest.mark.parametrize("d", [64, 80, 128])
+def test_no_queries_at_all(d):
+    """seqlen_q = 0: nothing to write forward; backward: dK = dV = 0."""
+    from byteir_amd import ops
+    b, h, sk = 2, 4, 150
+    q = torch.empty((b, 0, h, d), device="cuda", dtype=torch.float16)
+    k = torch.randn((b, sk, h, d), device="cuda").half()
+    v = torch.randn_like(k)
+    o, lse = ops.flash_attn_fwd(q, k, v, 0.3, (-1, 0))
+    assert o.numel() == 0 and lse.numel() == 0
+    bufs = ops.flash_attn_bwd_buffers(q, k, v)
+    for t in bufs[1:3]:
+        t.fill_(7.0)
+    dq, dk, dv = ops.flash_attn_bwd(torch.empty_like(q), q, k, v, o, lse, 0.3, (-1, 0), out=bufs)[:3]
+    assert dq.numel() == 0 and torch.all(dk == 0) and torch.all(dv == 0)
+
+
 @pytest.mark.parametrize("code", [oracle.F16, oracle.BF16])
 @pytest.mark.parametrize("case", CASES)
 def test_backward_matches_oracle(case, code):
