@@ -298,6 +298,13 @@ reduce_colwide_kernel(const T *__restrict__ in, TO *__restrict__ out, uint64_t B
   else fold(std::false_type{});
 }
 
+// An empty fold axis: every output is the operator's identity run through finish().
+template <typename TO>
+__global__ void __launch_bounds__(kBlock) reduce_fill_kernel(TO *__restrict__ out, uint64_t n, float value) {
+  const uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i < n) out[i] = to_out<TO>(value);
+}
+
 // ---- host-side planning -------------------------------------------------------------------
 struct Plan {
   int kind;       // 0 copy, 1 row, 2 col, 3 wide col (reduce_colwide_kernel)
@@ -313,7 +320,7 @@ inline uint64_t round_up(uint64_t a, uint64_t b) { return ceil_div(a, b) * b; }
 
 Plan make_plan(int dtype, uint64_t A, uint64_t B, uint64_t C, bool allow_split) {
   Plan p{};
-  if (!(A && B && C)) { p.kind = 0; p.S = 1; return p; }
+  if (!(A && B && C)) { p.kind = 0; p.S = 1; return p; }  // copy, fill or nothing: no workspace
   const int vec_full = dtype == BRT_ROCM_F32 ? 4 : 8;
   if (C == 1) {
     p.kind = 1;
@@ -451,10 +458,31 @@ extern "C" int brt_rocm_reduce_ex(int op, int dtype, const void *input, void *ou
       (dtype != BRT_ROCM_F32 && dtype != BRT_ROCM_F16))
     return hipErrorInvalidValue;
   const size_t es = dtype == BRT_ROCM_F32 ? 4 : 2;
-  if (!(A && B && C)) {  // nothing to fold: copy C elements (reduce_impl.h:71-74)
+  if (A == 0 && B == 0) {  // nothing to fold: copy C elements (reduce_impl.h:55-58,71-74)
     if (C == 0) return hipSuccess;
     if (!input || !output) return hipErrorInvalidValue;
     return hipMemcpyAsync(output, input, C * es, hipMemcpyDeviceToDevice, stream);
+  }
+  if (A == 0 || C == 0) return hipSuccess;  // no output element
+  if (B == 0) {
+    // An empty fold axis.  The reference sends this to its copy branch too, which reads C
+    // elements of an input that has none; here every output gets the operator's identity.
+    if (!output) return hipErrorInvalidValue;
+    float value = 0.f;
+    switch (op) {
+    case BRT_ROCM_REDUCE_MAX: value = -INFINITY; break;
+    case BRT_ROCM_REDUCE_MIN: value = INFINITY; break;
+    case BRT_ROCM_REDUCE_PROD: value = 1.f; break;
+    case BRT_ROCM_REDUCE_MEAN: value = NAN; break;  // 0 / float(0)
+    default: break;
+    }
+    const uint64_t n = (uint64_t)A * C, blocks = (n + kBlock - 1) / kBlock;
+    if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
+    if (dtype == BRT_ROCM_F32) reduce_fill_kernel<float><<<dim3((unsigned)blocks), dim3(kBlock), 0, stream>>>(static_cast<float *>(output), n, value);
+    else reduce_fill_kernel<__half><<<dim3((unsigned)blocks), dim3(kBlock), 0, stream>>>(static_cast<__half *>(output), n, value);
+    const hipError_t e = hipGetLastError();
+    if (e == hipSuccess && first_pass_done) return hipEventRecord(first_pass_done, stream);
+    return e;
   }
   if (!input || !output) return hipErrorInvalidValue;
 #define RUN(T, OP) \

@@ -86,8 +86,12 @@ int brt_rocm_event_elapsed_ms(float *ms, void *start, void *stop);
  *  reduction.cu:415-426), and
  *   kernel::get_reduce_workspace_in_bytes<T>(A, B, C)          (reduction.h:17-18,
  *  reduction.cu:428-434).
- * A == 0 or B == 0 means "nothing to fold": C elements are copied device to device, as
- * ReduceImpl::Execute does (reduce_impl.h:61-75).
+ * A == 0 and B == 0 means "nothing to fold": C elements are copied device to device, as
+ * ReduceImpl::Execute does for the (0, 0, numel) it sets up when every reduced dimension has
+ * extent 1 (reduce_impl.h:55-58,61-75).  Tensors without elements: A == 0 or C == 0 writes
+ * nothing; B == 0 with A, C > 0 (an empty fold axis, which the reference also sends to its copy
+ * branch, reading C elements of an input that has none) writes the operator's identity to all
+ * A * C outputs (0, -inf, +inf, 1, NaN for the mean, 0).
  * The workspace holds float partials of the split first pass; its size depends only on
  * (dtype, A, B, C), so it can be queried once when an execution plan is built.  A NULL or
  * too small workspace is an error (hipErrorInvalidValue) when the size is non-zero.

@@ -175,7 +175,7 @@ def reference_workspace_bytes(A, B, C, elem_size=4):
 def reduce_abc(op, x, A, B, C):
     """Fold the middle axis of x viewed as [A,B,C]; sequential float chain per output."""
     x = np.ascontiguousarray(x)
-    n_out = (A * C) if (A and B and C) else C
+    n_out = C if (A == 0 and B == 0) else A * C
     out = np.empty(n_out, dtype=x.dtype)
     lib().oracle_reduce(op, _code(x), _p(x), _p(out), A, B, C)
     return out

@@ -236,14 +236,17 @@ static inline float fold_finish(int op, float r, uint64_t B) { return op == 4 ? 
  * linalg loop nest the CPU path executes.  op: 0 = sum (init 0), 1 = max (init -inf),
  * 2 = min, 3 = prod, 4 = mean, 5 = sum of squares.
  * dtype 0 = f32, 1 = f16 (accumulated in float, reduce_impl.h:64-69).
- * A == 0 means "plain copy of C elements" (reduce_impl.h:71-74). */
+ * A == 0 and B == 0 means "plain copy of C elements" (reduce_impl.h:55-58,71-74). */
 void oracle_reduce(int op, int dtype, const void *in, void *out, uint64_t A, uint64_t B,
                    uint64_t C) {
-  if (!(A && B && C)) {
+  if (A == 0 && B == 0) {
     size_t es = dtype == 0 ? 4 : 2;
     memcpy(out, in, C * es);
     return;
   }
+  /* an empty tensor: no output, or (B == 0) an empty fold per output, which the loops below
+   * turn into the operator's identity; the reference's copy branch would read past an input
+   * without elements here (reduce_impl.h:61-75) */
   if (dtype == 0 && C == 1 && op <= 1) { /* tight loop for the timed baseline */
     const float *x = (const float *)in;
     float *y = (float *)out;

@@ -155,6 +155,20 @@ def test_other_operators_on_real_values(shape, dims):
     np.testing.assert_allclose(got, y.astype(np.float64).prod(axis=dims), rtol=max(1e-5, n * 2.0 ** -24))
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_tensors_without_elements(dtype):
+    """An empty fold axis writes the operator's identity to every output; a tensor with no
+    output element writes nothing (the reference would copy from an input without elements)."""
+    from byteir_amd import ops
+    x = np.empty((4, 0, 8), dtype=dtype)
+    for op in (oracle.SUM, oracle.MAX, oracle.MIN, oracle.PROD, oracle.SUMSQR):
+        assert np.array_equal(host(ops.reduce(op, dev(x), (1,))), oracle.reduce_op(op, x, (1,)))
+    assert np.all(np.isnan(host(ops.reduce(oracle.MEAN, dev(x), (1,)))))
+    assert ops.reduce(oracle.SUM, dev(np.empty((0, 5), dtype)), (1,)).shape == (0,)
+    assert ops.reduce(oracle.MAX, dev(np.empty((3, 5, 0), dtype)), (1,)).shape == (3, 0)
+    assert ops.reduce(oracle.SUM, dev(np.empty((0, 1, 5), dtype)), (1,)).shape == (0, 5)  # the copy branch, no element
+
+
 def test_min_nan_and_infinities():
     from byteir_amd import ops
     x = np.full((3, 70000), np.inf, dtype=np.float32)

@@ -186,3 +186,14 @@ def test_min_identity_nan_and_empty_product():
     h = np.array([[255.0, 3.0, 0.5]], dtype=np.float16)  # 255^2 = 65025 rounds to 65024 in f16
     got = oracle.reduce_op(oracle.SUMSQR, h, (1,))
     assert got.dtype == np.float16 and got[0] == np.float16(65025.0 + 9.0 + 0.25)
+
+
+def test_tensors_without_elements():
+    """An empty fold axis gives the operator's identity; no output element, nothing written."""
+    x = np.empty((4, 0, 8), dtype=np.float32)
+    want = {oracle.SUM: 0.0, oracle.MAX: -np.inf, oracle.MIN: np.inf, oracle.PROD: 1.0, oracle.SUMSQR: 0.0}
+    for op, v in want.items():
+        assert np.array_equal(oracle.reduce_op(op, x, (1,)), np.full((4, 8), v, np.float32))
+    assert np.all(np.isnan(oracle.reduce_op(oracle.MEAN, x, (1,))))
+    assert oracle.reduce_op(oracle.SUM, np.empty((0, 5), np.float32), (1,)).shape == (0,)
+    assert oracle.reduce_op(oracle.SUM, np.empty((3, 5, 0), np.float32), (1,)).shape == (3, 0)
