@@ -76,6 +76,10 @@ CASES = [
     (3, 1, 50, 1, 1, 32, (-1, -1)),        # single query row
     (2, 260, 260, 8, 2, 128, (-1, 0)),     # grouped-query heads: dK, dV sum over the group
     (1, 190, 300, 6, 1, 32, (50, 20)),     # one key/value head for all query heads
+    # narrow windows over many tiles: waves of a backward workgroup idle at both ends of its range
+    (1, 1000, 1000, 4, 2, 64, (100, 60)),
+    (1, 900, 1100, 2, 2, 128, (70, 0)),
+    (1, 700, 700, 2, 1, 32, (0, 90)),
     # few query rows: the decode kernel (all query heads of a key/value head in one score tile,
     # keys split over waves and, for long sequences, over workgroups)
     (2, 1, 1000, 8, 2, 128, (-1, -1)),
