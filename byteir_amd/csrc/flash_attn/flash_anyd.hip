@@ -87,8 +87,9 @@ __device__ __forceinline__ uint4 philox7(uint32_t k0, uint32_t k1, uint64_t offs
 #pragma unroll
   for (int r = 0; r < 7; ++r) {
     if (r > 0) { k0 += 0x9E3779B9u; k1 += 0xBB67AE85u; }
-    const uint32_t hi0 = __umulhi(0xD2511F53u, c0), lo0 = 0xD2511F53u * c0;
-    const uint32_t hi1 = __umulhi(0xCD9E8D57u, c2), lo1 = 0xCD9E8D57u * c2;
+    // one 32 x 32 -> 64-bit multiply per product (v_mad_u64_u32) instead of a high and a low one
+    const uint64_t p0 = (uint64_t)0xD2511F53u * c0, p1 = (uint64_t)0xCD9E8D57u * c2;
+    const uint32_t hi0 = (uint32_t)(p0 >> 32), lo0 = (uint32_t)p0, hi1 = (uint32_t)(p1 >> 32), lo1 = (uint32_t)p1;
     const uint32_t n0 = hi1 ^ c1 ^ k0, n2 = hi0 ^ c3 ^ k1;
     c0 = n0; c1 = lo1; c2 = n2; c3 = lo0;
   }
@@ -111,39 +112,52 @@ struct DropCtx {
     off = p.rng_state[1] + (uint64_t)(bh * 32);
     thr = p.keep_thr;
   }
-  // Scores held with the query on the lane (column of S^T): bit i of the result is set when
-  // key kv32 + 8*(i/4) + 4*g + i%4 is kept for query q; kv32 is a multiple of 32.
-  __device__ __forceinline__ uint32_t keep_q_on_lane(int q, int kv32, int g) const {
+  // One Philox value per lane covers a whole 32 x 32 block of the attention matrix (rows q32..,
+  // columns kv32.., both multiples of 32): lane L draws the value of warp lane L % 32 in row
+  // block q32/16 + L/32.  Bit 4*tile + 2*(row half) + (column & 1) of the result is set when
+  // that byte is kept.  Every lane of the wave must take part (the callers below exchange the
+  // words across lanes).
+  __device__ __forceinline__ uint32_t draw(int q32, int kv32) const {
+    const int L = threadIdx.x & 63;
+    const uint4 r = philox7(k0, k1, off + (uint32_t)(L & 31), (uint32_t)((q32 >> 4) + (L >> 5)), (uint32_t)(kv32 >> 5));
+    const uint32_t w[4] = {r.x, r.y, r.z, r.w};
     uint32_t m = 0;
-    const int sh = ((q >> 3) & 1) * 16;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int b = 0; b < 4; ++b)
+        if (((w[t] >> (8 * b)) & 0xffu) <= thr) m |= 1u << (4 * t + b);
+    return m;
+  }
+  // Scores held with the query on the lane (column of S^T): bit i of the result is set when
+  // key kv32 + 8*(i/4) + 4*g + i%4 is kept for query q = q32 + lane % 32.  The 16 elements lie
+  // in the values of warp lanes (q%8)*4 + 2*g + {0, 1} of row block q/16.
+  __device__ __forceinline__ uint32_t keep_q_on_lane(int q, int kv32, int g) const {
+    const uint32_t own = draw(q & ~31, kv32);
+    const int src = ((q >> 4) & 1) * 32 + (q & 7) * 4 + g * 2, sh = ((q >> 3) & 1) * 2;
+    uint32_t m = 0;
 #pragma unroll
     for (int c2 = 0; c2 < 2; ++c2) {
-      const uint4 r = philox7(k0, k1, off + (uint32_t)((q & 7) * 4 + g * 2 + c2), (uint32_t)(q >> 4), (uint32_t)(kv32 >> 5));
-      const uint32_t w[4] = {r.x, r.y, r.z, r.w};
-#pragma unroll
-      for (int t = 0; t < 4; ++t)
-#pragma unroll
-        for (int e = 0; e < 2; ++e)
-          if (((w[t] >> (sh + 8 * e)) & 0xffu) <= thr) m |= 1u << (t * 4 + c2 * 2 + e);
+      const uint32_t w = (uint32_t)__builtin_amdgcn_ds_bpermute((src + c2) * 4, (int)own);
+      m |= ((w >> sh) & 0x3333u) << (2 * c2);
     }
     return m;
   }
   // Scores held with the key on the lane (column of S): bit i is set when query
-  // q32 + 8*(i/4) + 4*g + i%4 is kept for key kv; q32 is a multiple of 32.
+  // q32 + 8*(i/4) + 4*g + i%4 is kept for key kv = kv32 + lane % 32.  The 16 elements lie in the
+  // values of warp lanes (4*g + j)*4 + (kv%8)/2, j = 0..3, of both row blocks.
   __device__ __forceinline__ uint32_t keep_k_on_lane(int q32, int kv, int g) const {
+    const uint32_t own = draw(q32, kv & ~31);
+    const uint32_t other = (uint32_t)__builtin_amdgcn_ds_bpermute(((threadIdx.x & 63) ^ 32) * 4, (int)own);
+    const uint32_t both = (threadIdx.x & 32) ? (other | own << 16) : (own | other << 16);  // row block 0 low
+    const int sh = ((kv & 31) >> 3) * 4 + (kv & 1);
     uint32_t m = 0;
-    const int tile = (kv & 31) >> 3, e = kv & 1;
 #pragma unroll
-    for (int rb = 0; rb < 2; ++rb)
-#pragma unroll
-      for (int c4 = 0; c4 < 4; ++c4) {
-        const uint4 r = philox7(k0, k1, off + (uint32_t)((g * 4 + c4) * 4 + ((kv & 7) >> 1)),
-                                (uint32_t)((q32 >> 4) + rb), (uint32_t)(kv >> 5));
-        const uint32_t w = tile == 0 ? r.x : tile == 1 ? r.y : tile == 2 ? r.z : r.w;
-#pragma unroll
-        for (int rh = 0; rh < 2; ++rh)
-          if (((w >> (8 * (2 * rh + e))) & 0xffu) <= thr) m |= 1u << (rb * 8 + rh * 4 + c4);
-      }
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t x = (uint32_t)__builtin_amdgcn_ds_bpermute(((g * 4 + j) * 4 + ((kv & 7) >> 1)) * 4, (int)both) >> sh;
+      // bits 0, 2 (row halves of row block 0) and 16, 18 (row block 1) -> rows 8*a + 4*g + j, a = 0..3
+      m |= ((x & 1u) | ((x & 4u) << 2) | ((x >> 8) & 0x100u) | ((x >> 6) & 0x1000u)) << j;
+    }
     return m;
   }
 };
@@ -354,7 +368,7 @@ __global__ void __launch_bounds__(256) dot_do_o_anyd_kernel(const Params p) {
 
 // ---- backward 2: dK, dV -----------------------------------------------------------------------------
 template <typename T, int DR, bool Drop>
-__global__ void __launch_bounds__(256) dkdv_anyd_kernel(const Params p) {
+__global__ void __launch_bounds__(256, DR <= 64 ? 2 : 1) dkdv_anyd_kernel(const Params p) {
   using vec8 = typename Traits<T>::vec8;
   constexpr int QS = Pad<DR>::kPlain;  // tiles are read both plainly and transposed
   constexpr bool kPrefetch = DR <= 128;
@@ -505,7 +519,7 @@ __global__ void __launch_bounds__(256) dkdv_anyd_kernel(const Params p) {
 
 // ---- backward 3: dQ ---------------------------------------------------------------------------------
 template <typename T, int DR, bool Drop>
-__global__ void __launch_bounds__(256) dq_anyd_kernel(const Params p) {
+__global__ void __launch_bounds__(256, DR <= 96 ? 2 : 1) dq_anyd_kernel(const Params p) {
   using vec8 = typename Traits<T>::vec8;
   constexpr int KS = Pad<DR>::kPlain;  // K tile: plain and transposed reads
   constexpr int VS = Pad<DR>::kPlain;  // V tile: plain reads only
