@@ -253,6 +253,30 @@ def test_strided_tensors(case, code):
         assert err <= ATOL, (name, float(err))
 
 
+@pytest.mark.parametrize("case,p_drop", [
+    ((2, 700, 700, 8, 2, 64, (-1, 0)), 0.0),     # tuned kernels, grouped heads
+    ((1, 300, 2500, 4, 4, 128, (-1, -1)), 0.0),  # forward split over workgroups and merged
+    ((2, 2, 5000, 8, 2, 128, (-1, -1)), 0.0),    # decode kernel, several chunks per head
+    ((1, 333, 400, 2, 2, 80, (50, 10)), 0.0),    # generic kernels
+    ((1, 400, 400, 4, 2, 64, (-1, 0)), 0.2),     # dropout
+])
+def test_results_do_not_depend_on_the_run(case, p_drop):
+    """No atomics and a fixed merge order: a second call on the same inputs gives the same bits
+    (the reference accumulates dQ with float atomics, flash_bwd_kernel.h:663, and does not)."""
+    from byteir_amd import ops
+    b, sq, sk, h, h_k, d, window = case
+    q, k, v, do = (dev(x) for x in make_inputs(case, oracle.BF16, seed=11))
+    rng = ops.rng_state_tensor(1234, 5678, "cuda") if p_drop else None
+    runs = []
+    for _ in range(2):
+        o, lse = ops.flash_attn_fwd(q, k, v, 0.2, window, p_dropout=p_drop, rng_state=rng)
+        dq, dk, dv = ops.flash_attn_bwd(do, q, k, v, o, lse, 0.2, window, p_dropout=p_drop, rng_state=rng)
+        runs.append([host(t).copy() for t in (o, lse, dq, dk, dv)])
+        torch.randn((1 << 22,), device="cuda")  # other work in between
+    for a, c in zip(*runs):
+        assert np.array_equal(a, c, equal_nan=True)
+
+
 def test_unsupported_arguments_are_reported_not_run():
     import ctypes
     from byteir_amd import _lib, ops
