@@ -77,7 +77,7 @@ __global__ void __launch_bounds__(kDecWaves * 64, D <= 128 ? 2 : 1) decode_kerne
     const T *qg = static_cast<const T *>(p.q) + bi * p.q_bs + (int64_t)qi * p.q_rs + hq * p.q_hs;
 #pragma unroll
     for (int ks = 0; ks < D / 16; ++ks)
-      qf[ks] = col_ok ? *reinterpret_cast<const vec8 *>(qg + ks * 16 + g * 8) : vec8{0};
+      qf[ks] = (col_ok && ks * 16 + g * 8 < p.d) ? *reinterpret_cast<const vec8 *>(qg + ks * 16 + g * 8) : vec8{0};
   }
 
   T *Kt = reinterpret_cast<T *>(lds[wave]), *Vt = Kt + kUnit * KS;
@@ -94,7 +94,7 @@ __global__ void __launch_bounds__(kDecWaves * 64, D <= 128 ? 2 : 1) decode_kerne
 #pragma unroll
     for (int s = 0; s < NPV; ++s) {
       const int key = c0 + j * kUnit + s * RPP + v_r;
-      if (key < c1) {
+      if (key < c1 && v_c * 8 < p.d) {  // columns from head_dim up to D stay zero
         const bool fresh = key >= new0;
         T *kc_row = const_cast<T *>(kg) + (int64_t)key * p.k_rs + v_c * 8;
         T *vc_row = const_cast<T *>(vg) + (int64_t)key * p.v_rs + v_c * 8;
@@ -219,8 +219,8 @@ __global__ void __launch_bounds__(kDecWaves * 64, D <= 128 ? 2 : 1) decode_kerne
 #pragma unroll
     for (int w = 0; w < kDecWaves; ++w) acc += wgt[w] * reinterpret_cast<const float *>(lds[w])[dcol * 32 + n];
     if (out_ok) {
-      if (final_pass) og[dcol] = (T)(acc * inv);
-      else a.o_part[prow * D + dcol] = acc;
+      if (!final_pass) a.o_part[prow * D + dcol] = acc;
+      else if (dcol < p.d) og[dcol] = (T)(acc * inv);
     }
   }
   if (out_ok && slice == 0) {
@@ -257,7 +257,7 @@ __global__ void __launch_bounds__(D < 64 ? 64 : D) decode_merge_kernel(const Par
   const bool empty = l_all == 0.f || l_all != l_all;
   const int qi = (int)(row % p.sq), hq = (int)((row / p.sq) % p.h), bi = (int)(row / ((int64_t)p.sq * p.h));
   T *og = static_cast<T *>(p.o_w) + bi * p.o_bs + (int64_t)qi * p.o_rs + hq * p.o_hs;
-  if (threadIdx.x < D) og[dcol] = (T)(empty ? 0.f : acc / l_all);
+  if (threadIdx.x < p.d) og[dcol] = (T)(empty ? 0.f : acc / l_all);
   if (threadIdx.x == 0) p.lse[row] = empty ? INFINITY : m_all * p.scale + log2_fast(l_all) * kLn2;
 }
 
@@ -318,7 +318,7 @@ hipError_t launch_split_merge(const Params &p, int dtype, hipStream_t stream) {
 }
 
 bool decode_eligible(const Params &p) {
-  return (p.d == 32 || p.d == 64 || p.d == 128 || p.d == 256) && p.sq > 0 && (p.h / p.h_k) * p.sq <= 32 && p.sk >= 1 && !p.drop;
+  return p.d <= 256 && p.sq > 0 && (p.h / p.h_k) * p.sq <= 32 && p.sk >= 1 && !p.drop;
 }
 
 // The decode kernel can do the append itself when every appended row is certain to be loaded by
@@ -329,10 +329,12 @@ bool decode_can_append(const Params &p) {
 
 hipError_t launch_decode(Params &p, int dtype, hipStream_t stream) {
   if (p.b * p.h == 0 || p.sq == 0) return hipSuccess;
-  if (p.d == 32) return dtype == 1 ? decode_td<_Float16, 32>(p, stream) : decode_td<__bf16, 32>(p, stream);
-  if (p.d == 64) return dtype == 1 ? decode_td<_Float16, 64>(p, stream) : decode_td<__bf16, 64>(p, stream);
-  if (p.d == 256) return dtype == 1 ? decode_td<_Float16, 256>(p, stream) : decode_td<__bf16, 256>(p, stream);
-  return dtype == 1 ? decode_td<_Float16, 128>(p, stream) : decode_td<__bf16, 128>(p, stream);
+  // D is the tile width: the smallest of 32, 64, 128, 256 that holds head_dim (a multiple of 8);
+  // the columns between head_dim and D are zero in the tiles and never loaded or stored
+  if (p.d <= 32) return dtype == 1 ? decode_td<_Float16, 32>(p, stream) : decode_td<__bf16, 32>(p, stream);
+  if (p.d <= 64) return dtype == 1 ? decode_td<_Float16, 64>(p, stream) : decode_td<__bf16, 64>(p, stream);
+  if (p.d <= 128) return dtype == 1 ? decode_td<_Float16, 128>(p, stream) : decode_td<__bf16, 128>(p, stream);
+  return dtype == 1 ? decode_td<_Float16, 256>(p, stream) : decode_td<__bf16, 256>(p, stream);
 }
 
 }  // namespace fa

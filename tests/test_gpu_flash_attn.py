@@ -92,6 +92,10 @@ CASES = [
     (1, 32, 40, 2, 2, 64, (-1, 0)),        # all 32 columns are rows of one head
     (2, 7, 5, 4, 1, 128, (-1, 0)),         # causal with sq > sk: leading rows keep no key
     (1, 3, 600, 6, 2, 128, (-1, 5)),       # right window only
+    (2, 1, 1500, 8, 2, 80, (-1, -1)),      # decode kernel with a tile wider than head_dim
+    (1, 3, 700, 4, 4, 24, (-1, 0)),
+    (1, 2, 3000, 6, 2, 192, (-1, -1)),
+    (1, 1, 2600, 2, 2, 104, (300, 0)),
     # few query blocks against many keys: the key axis is split over workgroups and merged
     (1, 300, 2000, 2, 2, 64, (-1, 0)),
     (1, 256, 4096, 4, 1, 128, (-1, -1)),
@@ -394,6 +398,10 @@ KV_CASES = [
     (2, 3, 4, 2, 96, 260, 3, [250, 17], (-1, 0), True),         # head dimensions without a tuned kernel
     (1, 1, 2, 2, 256, 300, 1, [299], (-1, -1), True),
     (2, 4, 2, 2, 80, 128, 0, [128, 5], (-1, -1), False),
+    (2, 1, 8, 1, 40, 4000, 1, [3999, 1234], (-1, -1), True),    # decode kernel, tile wider than head_dim
+    (1, 2, 6, 2, 192, 2500, 2, [2498], (-1, 0), True),
+    (3, 1, 2, 2, 8, 90, 1, [0, 89, 31], (-1, -1), True),
+    (1, 4, 4, 2, 160, 700, 4, [650], (-1, 0), True),
 ]
 
 
