@@ -33,7 +33,10 @@ def run_case(shape, code, seed=0, sigma=2.0):
 
 @pytest.mark.parametrize("code", [oracle.F32, oracle.F16, oracle.BF16])
 @pytest.mark.parametrize("shape", [(10, 128), (8 * 12, 256, 256), (3, 1), (5, 4097), (7, 8), (33, 4096), (2, 8192),
-                                   (2, 20000), (1, 100003), (129, 520)])
+                                   (2, 20000), (1, 100003), (129, 520),
+                                   # rows held in LDS (odd lengths shift every row off 16-byte alignment),
+                                   # the longest that fit, and rows streamed twice
+                                   (6, 50257), (3, 32000), (2, 39900), (3, 40000), (2, 79800), (2, 80100), (5, 8200)])
 def test_softmax_matches_oracle(shape, code):
     run_case(shape, code)
 
@@ -64,6 +67,44 @@ def test_softmax_inner_axis_with_infinities():
     ok = ~np.isnan(want)
     assert np.abs(y[ok] - want[ok]).max() <= 1e-5
     assert np.all(y[0, :3, 5] == 0)
+
+
+@pytest.mark.parametrize("code", [oracle.F32, oracle.BF16])
+@pytest.mark.parametrize("cols", [9001, 30000, 90000])
+def test_long_rows_from_an_unaligned_view_leave_their_neighbours_alone(cols, code):
+    """Input and output start 1 element (f32: 4 bytes, bf16: 2 bytes) into a 16-byte granule: the
+    kernels read whole granules around the rows and must write the rows only."""
+    from byteir_amd import ops
+    rows = 3
+    x32 = (np.random.default_rng(cols).standard_normal((rows, cols)) * 2.0).astype(np.float32)
+    xs = oracle.from_f32(x32, code)
+    tdt = torch.float32 if code == oracle.F32 else torch.bfloat16
+    buf_in = torch.zeros(rows * cols + 16, dtype=tdt, device="cuda")
+    buf_out = torch.full((rows * cols + 16,), 7.0, dtype=tdt, device="cuda")
+    xin = buf_in[1:1 + rows * cols].view(rows, cols)
+    xin.copy_(dev(xs))
+    yout = buf_out[1:1 + rows * cols].view(rows, cols)
+    ops.softmax(xin, yout)
+    got = oracle.to_f32(host(yout))
+    want = sp_softmax(oracle.to_f32(xs).astype(np.float64), axis=-1).astype(np.float32)
+    rel, ab = TOL[code]
+    assert np.all(np.abs(got - want) <= rel * np.abs(want) + ab)
+    assert float(buf_out[0]) == 7.0 and torch.all(buf_out[1 + rows * cols:] == 7.0)
+
+
+@pytest.mark.parametrize("cols", [20000, 120000])
+def test_long_rows_in_place_nan_and_infinities(cols):
+    from byteir_amd import ops
+    x = torch.randn((4, cols), device="cuda")
+    x[1, cols // 3] = float("nan")
+    x[2, :] = -float("inf")
+    x[3, : cols - 5] = -float("inf")   # every lane but a few sees only -inf
+    want = oracle.softmax(host(x))
+    y = host(ops.softmax(x, x))        # in place
+    assert np.all(np.isnan(y[1])) and np.all(np.isnan(y[2]))
+    assert np.array_equal(np.isnan(y), np.isnan(want))
+    assert np.abs(y[0] - want[0]).max() <= 1e-5 * want[0].max() + 1e-10
+    assert np.all(y[3, : cols - 5] == 0) and abs(float(y[3].sum()) - 1.0) < 1e-5
 
 
 def test_softmax_properties_f32():
