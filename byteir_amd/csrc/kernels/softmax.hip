@@ -1,9 +1,9 @@
 // Fused row softmax for gfx950: y = exp(x - max(x)) / sum(exp(x - max(x))) over the last
 // axis of a dense [rows, cols] tensor, float internals, one rounding at the store.
 //
-// (A softmax over an inner axis, [A, B, C] over B with C > 1, takes softmax_inner_kernel: lanes
-// along the contiguous C axis, one online max/sum pass over B and a second pass that re-reads
-// the tile -- mostly from L2 -- and writes.)
+// (A softmax over an inner axis, [A, B, C] over B with C > 1, takes softmax_inner_kernel: a
+// workgroup per column tile, lanes along the contiguous C axis with 128-bit accesses, row lanes
+// along B; one online max/sum pass and a second pass that re-reads the tile and writes.)
 //
 // softmax_wave_kernel keeps a whole row in the registers of one wave (NV 128-bit vectors per
 // lane), so a row is read from HBM once and written once; max and sum are wave64 shuffle
@@ -299,52 +299,179 @@ softmax_stream_kernel(const T *in, T *out, uint64_t cols) {
     sp.each(raw, j, [&](float v) { vm = fmaxf(vm, v); });
     if (vm > m) { s *= fast_exp(m - vm); m = vm; }  // exp(-inf - vm) = 0 for the first finite value
     if (m != -INFINITY) sp.each(raw, j, [&](float v) { s += fast_exp(v - m); });
+    else sp.each(raw, j, [&](float v) { if (v != v) s = v; });  // only -inf so far: s stays 0, or NaN after a NaN
   }
   const float m_all = block_all<THREADS>(m, sm, true);
-  s = (m == -INFINITY) ? 0.f : s * fast_exp(m - m_all);  // a lane that saw only -inf adds nothing
+  s = (m == -INFINITY) ? s : s * fast_exp(m - m_all);  // a lane that saw only -inf (and NaN) adds 0 (NaN)
   s = block_all<THREADS>(s, sm, false);
   const float inv = 1.0f / s;
 #pragma unroll 4
   for (uint64_t j = threadIdx.x; j < sp.nvec; j += THREADS) sp.finish(load_stream(sp.src + j), j, m_all, inv);
 }
 
-// Softmax over the middle axis of a dense [A, B, C] tensor: one thread per (a, c) column, lanes
-// along c.  Pass 1 keeps a running maximum and a sum rescaled on the fly (so the column is read
-// once for both), pass 2 re-reads and writes.
-template <typename T>
+// Softmax over the middle axis of a dense [A, B, C] tensor.  A workgroup owns TX * VEC adjacent
+// columns of one a: lane (tx, ty) owns VEC columns (one 128-bit load per row when VEC > 1) and
+// walks rows ty, ty + TY, ...  Pass 1 keeps a running maximum and a sum rescaled on the fly per
+// column (one read for both); the TY partials of a column meet in LDS; pass 2 reads the tile
+// again (from the caches when they hold it) and writes.
+// Few columns and a long B would leave most of the chip idle, so B can be cut into S segments
+// over workgroups: MODE 1 runs pass 1 on a segment and writes the column's (maximum, sum) to
+// part[a][segment][c][2]; MODE 2 folds the S partials of its columns and runs pass 2 on its
+// segment.  MODE 0 is both passes in one workgroup (S = 1).
+template <typename T, int VEC, int TX, int MODE>
 __global__ void __launch_bounds__(kBlock)
-softmax_inner_kernel(const T *__restrict__ in, T *__restrict__ out, uint64_t B, uint64_t C) {
-  const uint64_t c = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (c >= C) return;
-  const T *x = in + (uint64_t)blockIdx.y * B * C + c;
-  T *y = out + (uint64_t)blockIdx.y * B * C + c;
-  float m = -INFINITY, s = 0.f;
-  for (uint64_t b = 0; b < B; ++b) {
-    const float v = Elem<T>::get(x[b * C]);
-    const float m_new = fmaxf(m, v);
-    // exp(-inf - -inf) would be NaN: a column that is -inf so far keeps s = 0 (if it stays
-    // -inf to the end, pass 2 produces the NaN the two-pass definition gives)
-    s = m_new == -INFINITY ? 0.f : s * fast_exp(m - m_new) + fast_exp(v - m_new);
-    m = m_new;
+softmax_inner_kernel(const T *__restrict__ in, T *__restrict__ out, uint64_t B, uint64_t C, uint32_t col_tiles,
+                     uint32_t S, uint64_t seg_rows, float *__restrict__ part) {
+  constexpr int TY = kBlock / TX;
+  __shared__ float pm[TY][TX * VEC + 1], ps[TY][TX * VEC + 1];
+  const int tx = threadIdx.x % TX, ty = threadIdx.x / TX;
+  const uint32_t tile = blockIdx.x % col_tiles;
+  const uint32_t seg = (blockIdx.x / col_tiles) % S;
+  const uint64_t a = blockIdx.x / ((uint64_t)col_tiles * S);
+  const uint64_t b0 = (uint64_t)seg * seg_rows, b1 = b0 + seg_rows < B ? b0 + seg_rows : B;
+  const uint64_t c = ((uint64_t)tile * TX + tx) * VEC;
+  const bool ok = c < C;  // C is a multiple of VEC
+  const T *x = in + a * B * C + c;
+  T *y = out + a * B * C + c;
+  auto load = [&](uint64_t b, float (&v)[VEC]) {
+    if constexpr (VEC > 1) {
+      const uint4 raw = *reinterpret_cast<const uint4 *>(x + b * C);
+      const T *e = reinterpret_cast<const T *>(&raw);
+#pragma unroll
+      for (int k = 0; k < VEC; ++k) v[k] = Elem<T>::get(e[k]);
+    } else {
+      v[0] = Elem<T>::get(x[b * C]);
+    }
+  };
+  float m[VEC], s[VEC];
+#pragma unroll
+  for (int k = 0; k < VEC; ++k) { m[k] = -INFINITY; s[k] = 0.f; }
+  if (MODE != 2 && ok) {
+#pragma unroll 8
+    for (uint64_t b = b0 + ty; b < b1; b += TY) {
+      float v[VEC];
+      load(b, v);
+#pragma unroll
+      for (int k = 0; k < VEC; ++k) {
+        const float m_new = fmaxf(m[k], v[k]);
+        // exp(-inf - -inf) would be NaN: a column that is -inf so far keeps its s, which is 0,
+        // or NaN once a NaN has been seen (the maximum skips NaN, the sum must not); if the
+        // column stays -inf to the end, pass 2 produces the NaN the two-pass definition gives
+        // One exponential serves both cases: a new maximum rescales the sum by exp(m - v) and adds
+        // 1, otherwise exp(v - m) is added.  (m = -inf: e = 0, s becomes 1; v = -inf: e = 0.)
+        const float d = v[k] - m[k];
+        const float e = fast_exp(-fabsf(d));
+        s[k] = m_new == -INFINITY ? (v[k] != v[k] ? v[k] : s[k]) : (d > 0.f ? fmaf(s[k], e, 1.f) : s[k] + e);
+        m[k] = m_new;
+      }
+    }
   }
-  const float inv = 1.0f / s;
-  for (uint64_t b = 0; b < B; ++b) y[b * C] = Elem<T>::make(fast_exp(Elem<T>::get(x[b * C]) - m) * inv);
+  if (MODE == 2 && ok) {  // the segments' partials of this lane's columns, shared out over the row lanes
+    const float *pp = part + (a * S * C + c) * 2;
+    for (uint32_t r = ty; r < S; r += TY)
+#pragma unroll
+      for (int k = 0; k < VEC; ++k) {
+        const float mr = pp[((uint64_t)r * C + k) * 2], sr = pp[((uint64_t)r * C + k) * 2 + 1];
+        const float m_new = fmaxf(m[k], mr);
+        // a side that saw only -inf (and NaN) adds its s as it is: 0, or NaN
+        s[k] = (m[k] == -INFINITY ? s[k] : s[k] * fast_exp(m[k] - m_new)) + (mr == -INFINITY ? sr : sr * fast_exp(mr - m_new));
+        m[k] = m_new;
+      }
+  }
+  // the TY partials of every column meet in LDS
+#pragma unroll
+  for (int k = 0; k < VEC; ++k) { pm[ty][tx * VEC + k] = m[k]; ps[ty][tx * VEC + k] = s[k]; }
+  __syncthreads();
+  float inv[VEC];
+#pragma unroll
+  for (int k = 0; k < VEC; ++k) {
+    float mm = -INFINITY, ss = 0.f;
+#pragma unroll 4
+    for (int r = 0; r < TY; ++r) mm = fmaxf(mm, pm[r][tx * VEC + k]);
+#pragma unroll 4
+    for (int r = 0; r < TY; ++r) {
+      const float mr = pm[r][tx * VEC + k];
+      ss += mr == -INFINITY ? ps[r][tx * VEC + k] : ps[r][tx * VEC + k] * fast_exp(mr - mm);
+    }
+    m[k] = mm;
+    inv[k] = 1.0f / ss;
+    s[k] = ss;
+  }
+  if constexpr (MODE == 1) {
+    if (ok && ty == 0) {
+      float *o = part + ((a * S + seg) * C + c) * 2;
+#pragma unroll
+      for (int k = 0; k < VEC; ++k) { o[2 * k] = m[k]; o[2 * k + 1] = s[k]; }
+    }
+    return;
+  }
+  if (!ok) return;
+#pragma unroll 8
+  for (uint64_t b = b0 + ty; b < b1; b += TY) {
+    float v[VEC];
+    load(b, v);
+    if constexpr (VEC > 1) {
+      uint4 o;
+      T *oe = reinterpret_cast<T *>(&o);
+#pragma unroll
+      for (int k = 0; k < VEC; ++k) oe[k] = Elem<T>::make(fast_exp(v[k] - m[k]) * inv[k]);
+      store_stream(reinterpret_cast<uint4 *>(y + b * C), o);
+    } else {
+      y[b * C] = Elem<T>::make(fast_exp(v[0] - m[0]) * inv[0]);
+    }
+  }
 }
 
 template <typename T>
 hipError_t run_inner(const T *in, T *out, uint64_t A, uint64_t B, uint64_t C, hipStream_t stream) {
-  const uint64_t bx = (C + kBlock - 1) / kBlock;
-  if (bx > 0x7fffffffull || A > 65535) {
-    // the grid's y extent is 16 bits: fold batches into several launches
-    for (uint64_t a0 = 0; a0 < A; a0 += 65535) {
-      const uint64_t na = A - a0 < 65535 ? A - a0 : 65535;
-      if (bx > 0x7fffffffull) return hipErrorInvalidValue;
-      softmax_inner_kernel<T><<<dim3((unsigned)bx, (unsigned)na), dim3(kBlock), 0, stream>>>(in + a0 * B * C, out + a0 * B * C, B, C);
-    }
-    return hipGetLastError();
+  constexpr int EPV = Elem<T>::EPV;
+  const bool vec = C % EPV == 0 && ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15u) == 0;
+  const uint64_t ncolv = vec ? C / EPV : C;
+  // narrower tiles (more row lanes) while the grid would not fill the chip: measured faster than
+  // wide tiles with the axis cut into segments ([4096, 65536] f32 over axis 0: 3.4 against 2.6 TB/s)
+  int tx = 256;
+  while (tx > 16 && (ncolv < (uint64_t)tx || A * ((ncolv + tx - 1) / tx) < 512)) tx /= 4;
+  const uint64_t col_tiles = (ncolv + tx - 1) / tx;
+  const int ty = kBlock / tx;
+  // segments of B over workgroups when the column tiles alone leave the chip idle (at least
+  // eight rows per lane and segment); the partials live in a stream-ordered allocation
+  uint64_t S = 1;
+  if (A * col_tiles < 512 && B >= (uint64_t)ty * 16) {
+    S = (512 + A * col_tiles - 1) / (A * col_tiles);
+    const uint64_t room = B / ((uint64_t)ty * 8);
+    if (S > room) S = room;
+    if (S > 1024) S = 1024;
   }
-  softmax_inner_kernel<T><<<dim3((unsigned)bx, (unsigned)A), dim3(kBlock), 0, stream>>>(in, out, B, C);
-  return hipGetLastError();
+  uint64_t seg_rows = ((B + S - 1) / S + ty - 1) / ty * ty;
+  S = (B + seg_rows - 1) / seg_rows;
+  float *part = nullptr;
+  if (S > 1 && hipMallocAsync(reinterpret_cast<void **>(&part), A * S * C * 2 * sizeof(float), stream) != hipSuccess) {
+    (void)hipGetLastError();  // no workspace: one workgroup per column tile
+    part = nullptr;
+    S = 1;
+    seg_rows = B;
+  }
+  if (col_tiles > 0xffffffffull || A * col_tiles * S > 0x7fffffffull) return hipErrorInvalidValue;
+  const dim3 grid((unsigned)(A * col_tiles * S)), block(kBlock);
+#define INNER(V, X, M) softmax_inner_kernel<T, V, X, M><<<grid, block, 0, stream>>>(in, out, B, C, (uint32_t)col_tiles, (uint32_t)S, seg_rows, part)
+#define INNER_TX(V, M) do { if (tx == 256) INNER(V, 256, M); else if (tx == 64) INNER(V, 64, M); else INNER(V, 16, M); } while (0)
+  hipError_t e = hipSuccess;
+  if (S == 1) {
+    if (vec) INNER_TX(EPV, 0); else INNER_TX(1, 0);
+    e = hipGetLastError();
+  } else {
+    if (vec) INNER_TX(EPV, 1); else INNER_TX(1, 1);
+    e = hipGetLastError();
+    if (e == hipSuccess) {
+      if (vec) INNER_TX(EPV, 2); else INNER_TX(1, 2);
+      e = hipGetLastError();
+    }
+    const hipError_t f = hipFreeAsync(part, stream);
+    if (e == hipSuccess) e = f;
+  }
+#undef INNER_TX
+#undef INNER
+  return e;
 }
 
 template <typename T>

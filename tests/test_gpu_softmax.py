@@ -43,21 +43,28 @@ def test_softmax_matches_oracle(shape, code):
 
 @pytest.mark.parametrize("code", [oracle.F32, oracle.F16, oracle.BF16])
 @pytest.mark.parametrize("shape,axis", [((4, 33, 70), 1), ((2, 3, 5, 7), 2), ((129, 1000), 0), ((3, 260, 2), 1),
-                                        ((2, 1, 300), 1), ((5, 64, 64), -2)])
+                                        ((2, 1, 300), 1), ((5, 64, 64), -2),
+                                        # few columns, long axis: the axis is cut into segments over workgroups
+                                        ((1, 5000, 100), 1), ((2, 3000, 24), 1), ((3, 2000, 7), 1), ((40000, 16), 0),
+                                        # wide: 128-bit column groups, one workgroup per column tile
+                                        ((3, 300, 2048), 1), ((600, 4100), 0)])
 def test_softmax_over_an_inner_axis(shape, axis, code):
     from byteir_amd import ops
     x32 = (np.random.default_rng(sum(shape)).standard_normal(shape) * 2.0).astype(np.float32)
     xs = oracle.from_f32(x32, code)
     got = oracle.to_f32(host(ops.softmax(dev(xs), axis=axis)))
     want = oracle.to_f32(oracle.softmax(xs, axis=axis))
+    if code == oracle.F32 and shape[axis] > 2048:  # the oracle's float chain drifts; fp64 closed form instead
+        want = sp_softmax(x32.astype(np.float64), axis=axis).astype(np.float32)
     rel, ab = TOL[code]
     assert np.all(np.abs(got - want) <= rel * np.abs(want) + ab), float(np.abs(got - want).max())
     np.testing.assert_allclose(got.sum(axis=axis), 1.0, atol=2e-2 if code != oracle.F32 else 1e-5)
 
 
-def test_softmax_inner_axis_with_infinities():
+@pytest.mark.parametrize("rows", [6, 4000])
+def test_softmax_inner_axis_with_infinities(rows):
     from byteir_amd import ops
-    x = torch.randn((2, 6, 130), device="cuda")
+    x = torch.randn((2, rows, 130), device="cuda")
     x[0, :3, 5] = -float("inf")          # the column starts with -inf values
     x[1, :, 7] = -float("inf")           # a column of -inf only: NaN, as exp(-inf - -inf) / 0 in the reference lowering
     x[1, 2, 9] = float("nan")
@@ -99,9 +106,11 @@ def test_long_rows_in_place_nan_and_infinities(cols):
     x[1, cols // 3] = float("nan")
     x[2, :] = -float("inf")
     x[3, : cols - 5] = -float("inf")   # every lane but a few sees only -inf
+    x = torch.cat([x, x[3:4].clone()])
+    x[4, 8:16] = float("nan")          # a lane that sees nothing but -inf and NaN must still pass the NaN on
     want = oracle.softmax(host(x))
     y = host(ops.softmax(x, x))        # in place
-    assert np.all(np.isnan(y[1])) and np.all(np.isnan(y[2]))
+    assert np.all(np.isnan(y[1])) and np.all(np.isnan(y[2])) and np.all(np.isnan(y[4]))
     assert np.array_equal(np.isnan(y), np.isnan(want))
     assert np.abs(y[0] - want[0]).max() <= 1e-5 * want[0].max() + 1e-10
     assert np.all(y[3, : cols - 5] == 0) and abs(float(y[3].sum()) - 1.0) < 1e-5
