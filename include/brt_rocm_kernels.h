@@ -112,14 +112,19 @@ int brt_rocm_reduce_ex(int op, int dtype, const void *input, void *output, size_
  * [rows, cols] tensor; float internals for every storage type, one rounding at the store.
  * The reference runtime has no softmax kernel; the arithmetic contract is the compiler's
  * linalg_ext.softmax lowering (compiler/lib/Conversion/ToLinalg/LinalgExtToLinalg.cpp:286-410).
- * dtype: BRT_ROCM_F32, BRT_ROCM_F16 or BRT_ROCM_BF16.  In-place (output == input) is allowed. */
+ * dtype: BRT_ROCM_F32, BRT_ROCM_F16 or BRT_ROCM_BF16.  In-place (output == input) is allowed.
+ * Rows of any length and alignment; rows that do not start on 16 bytes are processed through
+ * the 16-byte granules that cover them (bytes of the neighbouring rows in the first and last
+ * granule are read and never written). */
 int brt_rocm_softmax(int dtype, const void *input, void *output, size_t rows, size_t cols,
                      void *stream);
 
 /* The same over the middle axis of a dense row-major [A, B, C] tensor (byteir.softmax with an
  * `axis` that is not the last one, compiler/lib/Conversion/ToLinalg/HloToLinalg.cpp:393-467:
  * A = product of the dimensions before the axis, C = product of those after).  C == 1 is the
- * row softmax above. */
+ * row softmax above.  With few columns and a long axis the call takes a stream-ordered scratch
+ * allocation (hipMallocAsync / hipFreeAsync on `stream`, 8 * A * segments * C bytes) and falls
+ * back to one workgroup per column tile if that fails. */
 int brt_rocm_softmax_axis(int dtype, const void *input, void *output, size_t A, size_t B, size_t C,
                           void *stream);
 
