@@ -92,6 +92,7 @@ template <> struct Loader<float, 4> {
 };
 template <> struct Loader<float, 1> {
   static __device__ __forceinline__ void load(const float *p, float (&v)[1]) { v[0] = *p; }
+  static __device__ __forceinline__ float get(const float *p) { return *p; }
 };
 template <> struct Loader<__half, 8> {
   static __device__ __forceinline__ void load(const __half *p, float (&v)[8]) {
@@ -106,6 +107,7 @@ template <> struct Loader<__half, 8> {
 };
 template <> struct Loader<__half, 1> {
   static __device__ __forceinline__ void load(const __half *p, float (&v)[1]) { v[0] = __half2float(*p); }
+  static __device__ __forceinline__ float get(const __half *p) { return __half2float(*p); }
 };
 
 template <typename TO> __device__ __forceinline__ TO to_out(float v);
@@ -121,7 +123,10 @@ template <int OP> __device__ __forceinline__ float wave_fold(float r, int width)
 
 // ---- rows: C == 1 -----------------------------------------------------------------------
 // unit = a * S + s; G lanes fold in[a, s*seg_len : min(B, (s+1)*seg_len)] into out[unit].
-template <typename T, typename TO, int OP, int VEC, int G>
+// PEEL: the segment may start and end anywhere (a row length that is no multiple of the vector,
+// or an unaligned tensor): the elements before the first 16-byte boundary and after the last
+// are folded one by one, the aligned body with the same 128-bit loads.
+template <typename T, typename TO, int OP, int VEC, int G, bool PEEL>
 __global__ void __launch_bounds__(kBlock)
 reduce_row_kernel(const T *__restrict__ in, TO *__restrict__ out, uint64_t units, uint64_t B,
                   uint32_t S, uint64_t seg_len, float len) {
@@ -132,7 +137,7 @@ reduce_row_kernel(const T *__restrict__ in, TO *__restrict__ out, uint64_t units
   const bool valid = unit < units;
   if (!valid) unit = units - 1;  // surplus groups redo the last unit so shuffles stay whole
   const uint64_t a = unit / S, s = unit % S;
-  const uint64_t begin = s * seg_len;
+  uint64_t begin = s * seg_len;
   uint64_t end = begin + seg_len;
   if (end > B) end = B;
   const T *row = in + a * B;
@@ -140,6 +145,16 @@ reduce_row_kernel(const T *__restrict__ in, TO *__restrict__ out, uint64_t units
   float acc[U];
 #pragma unroll
   for (int u = 0; u < U; ++u) acc[u] = Fold<OP>::init();
+  if constexpr (PEEL) {
+    const uint64_t n = end - begin;
+    uint64_t head = ((16 - (reinterpret_cast<uintptr_t>(row + begin) & 15)) & 15) / sizeof(T);
+    if (head > n) head = n;
+    const uint64_t tail = (n - head) % VEC;
+    for (uint64_t e = lane; e < head; e += G) acc[0] = Fold<OP>::apply(acc[0], Fold<OP>::map(Loader<T, 1>::get(row + begin + e)));
+    for (uint64_t e = lane; e < tail; e += G) acc[1] = Fold<OP>::apply(acc[1], Fold<OP>::map(Loader<T, 1>::get(row + end - tail + e)));
+    begin += head;
+    end -= tail;
+  }
   const uint64_t step = (uint64_t)G * VEC;
   uint64_t i = begin + (uint64_t)lane * VEC;
   for (; i + (U - 1) * step < end; i += U * step) {
@@ -181,7 +196,7 @@ __global__ void __launch_bounds__(kBlock)
 reduce_col_kernel(const T *__restrict__ in, TO *__restrict__ out, uint64_t B, uint64_t C,
                   uint32_t S, uint64_t seg_rows, uint32_t col_tiles, float len) {
   constexpr int TY = kBlock / TX;
-  constexpr int U = kColU;
+  constexpr int U = VEC == 1 ? 4 * kColU : kColU;  // scalar loads: as many bytes in flight as with vectors
   __shared__ float part[TY][TX * VEC + 1];
   const int tx = threadIdx.x % TX, ty = threadIdx.x / TX;
   uint64_t bid = blockIdx.x;
@@ -324,8 +339,8 @@ Plan make_plan(int dtype, uint64_t A, uint64_t B, uint64_t C, bool allow_split) 
   const int vec_full = dtype == BRT_ROCM_F32 ? 4 : 8;
   if (C == 1) {
     p.kind = 1;
-    p.vec = (B % vec_full == 0) ? vec_full : 1;
-    const uint64_t nvec = ceil_div(B, p.vec);
+    p.vec = (B % vec_full == 0) ? vec_full : 1;  // 1: rows start off the 16-byte grid, peeled kernel
+    const uint64_t nvec = ceil_div(B, vec_full);
     p.g = nvec >= 2048 ? 256 : nvec >= 96 ? 64 : nvec >= 24 ? 16 : 4;
     uint64_t S = 1;
     if (allow_split && A * p.g < kFillThreads) {
@@ -385,8 +400,8 @@ hipError_t launch(const Plan &p, const T *in, TO *out, uint64_t A, uint64_t B, u
     if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
     const dim3 grid((unsigned)blocks), block(kBlock);
 #define ROW(G)                                                                                   \
-  if (vec) reduce_row_kernel<T, TO, OP, VF, G><<<grid, block, 0, stream>>>(in, out, units, B, p.S, p.seg, len); \
-  else reduce_row_kernel<T, TO, OP, 1, G><<<grid, block, 0, stream>>>(in, out, units, B, p.S, p.seg, len)
+  if (vec) reduce_row_kernel<T, TO, OP, VF, G, false><<<grid, block, 0, stream>>>(in, out, units, B, p.S, p.seg, len); \
+  else reduce_row_kernel<T, TO, OP, VF, G, true><<<grid, block, 0, stream>>>(in, out, units, B, p.S, p.seg, len)
     switch (p.g) {
     case 4: ROW(4); break;
     case 16: ROW(16); break;
