@@ -311,6 +311,10 @@ __global__ void __launch_bounds__(NW * 64, NW * QB >= 16 ? 2 : (QB == 2 ? 1 : 2)
   }
 
   // epilogue: normalise, write O and LSE
+  // D = 128, one workgroup per CU: nothing else hides the store latency, so O goes through LDS
+  // and leaves as whole rows (measured 3 % on causal and full b4 h32 s2048); with two workgroups
+  // per CU (D <= 64) the direct 8-byte stores are faster (8 % on b2 h16 s8192 d64).
+  constexpr bool kStageO = D == 128;
 #pragma unroll
   for (int qb = 0; qb < QB; ++qb) {
     const float l_tot = l_run[qb] + partner32(l_run[qb]);
@@ -330,7 +334,33 @@ __global__ void __launch_bounds__(NW * 64, NW * QB >= 16 ? 2 : (QB == 2 ? 1 : 2)
       }
       continue;
     }
-    if (qrow[qb] < p.sq) {
+    if constexpr (kStageO) {
+      // O^T in the accumulators -> the wave's own [32][D] tile in the (now idle) K/V ring ->
+      // whole 2*D-byte rows to global memory, 16 bytes per lane
+      constexpr int OS = D + 8;
+      static_assert(!kStageO || (NW / 2 * 32 * OS <= kStages * kBN * KS && NW / 2 * 32 * OS <= kStages * kBN * VS), "O staging must fit the ring");
+      if (qb == 0) __syncthreads();  // every wave has left the last K/V tile
+      T *Ot = (wave < NW / 2 ? &Ks[0][0] : &Vs[0][0]) + (wave % (NW / 2)) * 32 * OS;
+#pragma unroll
+      for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+        for (int i4 = 0; i4 < 4; ++i4) {
+          typedef T vec4 __attribute__((ext_vector_type(4)));
+          vec4 v;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) v[j] = (T)(o_acc[qb][db][i4 * 4 + j] * inv);
+          *reinterpret_cast<vec4 *>(&Ot[r32 * OS + db * 32 + i4 * 8 + g * 4]) = v;
+        }
+      constexpr int CPRO = D / 8, RPI = 64 / CPRO;  // 16-byte chunks per row, rows per store instruction
+      const int oc = lane % CPRO, orow = lane / CPRO;
+#pragma unroll
+      for (int it = 0; it < 32 / RPI; ++it) {
+        const int r = it * RPI + orow, q = wq0 + qb * 32 + r;
+        const uint4 v = *reinterpret_cast<const uint4 *>(&Ot[r * OS + oc * 8]);
+        if (q < p.sq)
+          *reinterpret_cast<uint4 *>(static_cast<T *>(p.o_w) + bi * p.o_bs + (int64_t)q * p.o_rs + hi * p.o_hs + oc * 8) = v;
+      }
+    } else if (qrow[qb] < p.sq) {
       T *og = static_cast<T *>(p.o_w) + bi * p.o_bs + (int64_t)qrow[qb] * p.o_rs + hi * p.o_hs;
 #pragma unroll
       for (int db = 0; db < D / 32; ++db)
@@ -342,6 +372,8 @@ __global__ void __launch_bounds__(NW * 64, NW * QB >= 16 ? 2 : (QB == 2 ? 1 : 2)
           for (int j = 0; j < 4; ++j) v[j] = (T)(o_acc[qb][db][i4 * 4 + j] * inv);
           *reinterpret_cast<vec4 *>(og + db * 32 + i4 * 8 + g * 4) = v;
         }
+    }
+    if (qrow[qb] < p.sq) {
       if (g == 0)
         p.lse[((int64_t)bi * p.h + hi) * p.sq + qrow[qb]] =
             empty ? INFINITY : m_run[qb] * p.scale + log2_fast(l_tot) * kLn2;
