@@ -312,7 +312,7 @@ __global__ void __launch_bounds__(NW * 64, NW * QB >= 16 ? 2 : (QB == 2 ? 1 : 2)
 
   // epilogue: normalise, write O and LSE
   // D = 128, one workgroup per CU: nothing else hides the store latency, so O goes through LDS
-  // and leaves as whole rows (measured 3 % on causal and full b4 h32 s2048); with two workgroups
+  // and leaves as whole rows (measured 3 % on causal b4 h32 s2048); with two workgroups
   // per CU (D <= 64) the direct 8-byte stores are faster (8 % on b2 h16 s8192 d64).
   constexpr bool kStageO = D == 128;
 #pragma unroll
