@@ -208,6 +208,43 @@ def test_backward_matches_oracle(case, code):
         assert np.all(err <= ATOL + ulp * np.abs(w32)), (name, float(err.max()))
 
 
+@pytest.mark.parametrize("code", [oracle.F16, oracle.BF16])
+@pytest.mark.parametrize("shape", [(1, 300, 900, 2, 2, 64), (1, 300, 900, 4, 2, 128), (1, 200, 700, 2, 2, 80),
+                                   (1, 2, 3000, 4, 2, 128), (1, 128, 4096, 2, 2, 64)])
+@pytest.mark.parametrize("trend", ["rising", "falling"])
+def test_large_and_drifting_scores(shape, trend, code):
+    """Scores with a spread of hundreds (in exponent units) whose maximum keeps rising, or falls,
+    along the key axis: the running maximum is raised many times (rising) or the first keys
+    dominate and everything later underflows (falling).  Forward and backward against plain
+    float attention."""
+    from byteir_amd import ops
+    b, sq, sk, h, h_k, d = shape
+    rng = np.random.default_rng(sq + sk + d)
+    ramp = np.linspace(0.2, 6.0, sk, dtype=np.float32)
+    if trend == "falling":
+        ramp = ramp[::-1]
+    q32 = rng.standard_normal((b, sq, h, d)).astype(np.float32) * 2.0
+    k32 = rng.standard_normal((b, sk, h_k, d)).astype(np.float32) * ramp[None, :, None, None]
+    q, k = oracle.from_f32(q32, code), oracle.from_f32(k32, code)
+    v, do = (oracle.from_f32(rng.standard_normal(s_).astype(np.float32), code) for s_ in ((b, sk, h_k, d), (b, sq, h, d)))
+    scale, window = 1.0 / np.sqrt(d), (-1, -1)
+    dq_, dk_, dv_, do_ = (dev(t) for t in (q, k, v, do))
+    o, lse = ops.flash_attn_fwd(dq_, dk_, dv_, scale, window)
+    o_ref, lse_ref, o32 = oracle.flash_fwd(q, k, v, scale, window, round_p=False)
+    assert np.abs(oracle.to_f32(host(o)) - o32).max() <= ATOL
+    assert np.abs(host(lse) - lse_ref).max() <= ATOL + 1e-6 * np.abs(lse_ref).max()
+    dq, dk, dv = ops.flash_attn_bwd(do_, dq_, dk_, dv_, o, lse, scale, window)
+    rq, rk, rv, _ = oracle.flash_bwd(do, q, k, v, host(o), host(lse), scale, window, round_p=False)
+    # P and dS are rounded to the storage type before their GEMMs (the reference's rounding
+    # points), so the error of a gradient element scales with the terms that are summed, not
+    # with the element itself: two storage ulps of the tensor's largest magnitude
+    ulp = 2.0 ** -10 if code == oracle.F16 else 2.0 ** -7
+    for name, got, want in (("dq", dq, rq), ("dk", dk, rk), ("dv", dv, rv)):
+        w32 = oracle.to_f32(want)
+        err = np.abs(oracle.to_f32(host(got)) - w32)
+        assert err.max() <= ATOL + 2 * ulp * np.abs(w32).max(), (name, float(err.max()), float(np.abs(w32).max()))
+
+
 STRIDED_CASES = [
     # layout, b, sq, sk, h, h_k, d, window
     ("packed_qkv", 2, 192, 192, 4, 4, 64, (-1, 0)),       # q, k, v are slices of one [b, s, 3, h, d] tensor
