@@ -82,6 +82,22 @@ struct TileLoader {
     ptr += tile_stride;
     row += ROWS;
   }
+  // the next tile into a register set of the caller's (two tiles in flight at a workgroup's start)
+  __device__ __forceinline__ void gload_into(uint4 (&r)[NP]) {
+#pragma unroll
+    for (int s = 0; s < NP; ++s) {
+      if (row + s * RPP < n_rows) r[s] = *reinterpret_cast<const uint4 *>(ptr + s * pass_stride);
+      else r[s] = uint4{0, 0, 0, 0};
+    }
+    ptr += tile_stride;
+    row += ROWS;
+  }
+  __device__ __forceinline__ void lstore_swz_from(T *tile, const uint4 (&rr)[NP]) const {
+    const int c = threadIdx.x % CPR, r = threadIdx.x / CPR;
+#pragma unroll
+    for (int s = 0; s < NP; ++s)
+      *reinterpret_cast<uint4 *>(&tile[Swz<D>::off(s * RPP + r, c)]) = rr[s];
+  }
   __device__ __forceinline__ void lstore(T *tile, int stride) const {
     const int c = threadIdx.x % CPR, r = threadIdx.x / CPR;
 #pragma unroll
@@ -179,11 +195,19 @@ __global__ void __launch_bounds__(256, (D <= 64 && KB == 1) ? 2 : 1) dkdv_kernel
       }
     }
   }
+  // head_dim 128 leaves room for one wave per SIMD, i.e. one workgroup per CU, so nothing covers
+  // a workgroup's start and end: the first two Q / dO tiles then travel together with the K / V
+  // fragments (a second register set, free at this occupancy), and dK / dV leave through LDS
+  // as whole rows.  A round of 256 workgroups costs 13.7 us + 2.26 us per tile without this.
+  constexpr bool kLean = D == 128;
   // consume the fragments once so that the wait for their loads sits here, not inside the loop
+  auto consume_kv = [&]() {
 #pragma unroll
-  for (int kb = 0; kb < KB; ++kb)
+    for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
-    for (int ks = 0; ks < D / 16; ++ks) asm volatile("" : "+v"(kf[kb][ks]), "+v"(vf[kb][ks]));
+      for (int ks = 0; ks < D / 16; ++ks) asm volatile("" : "+v"(kf[kb][ks]), "+v"(vf[kb][ks]));
+  };
+  if constexpr (!kLean) consume_kv();
   float16v dk_acc[KB][D / 32], dv_acc[KB][D / 32];
 #pragma unroll
   for (int kb = 0; kb < KB; ++kb)
@@ -352,7 +376,31 @@ __global__ void __launch_bounds__(256, (D <= 64 && KB == 1) ? 2 : 1) dkdv_kernel
       for (int w = 0; w < 2; ++w) { pb[kb][w] = vec8{0}; dsb[kb][w] = vec8{0}; }
   }
   // prologue: tiles m_min and m_min+1 into the ring, tile m_min+2 into registers
-  if (n_tiles > 0) {
+  if constexpr (kLean) {
+    uint4 q1[TileLoader<T, D, kQTile>::NP], do1[TileLoader<T, D, kQTile>::NP];
+    float lse1 = 0.f, dsm1 = 0.f;
+    if (n_tiles > 0) gload();
+    if (n_tiles > 1) {  // tile m_min+1 in flight together with tile m_min
+      lq.gload_into(q1);
+      ldo.gload_into(do1);
+      if (tid < kQTile) {
+        lse1 = q_next < p.sq ? lse_g[q_next] : INFINITY;
+        dsm1 = q_next < p.sq ? dsm_g[q_next] : 0.f;
+      }
+      q_next += kQTile;
+    }
+    if (gq == 0) consume_kv();
+    if (n_tiles > 0) {
+      lstore(0);
+      if (n_tiles > 1) {
+        lq.lstore_swz_from(Qs[1], q1);
+        ldo.lstore_swz_from(dOs[1], do1);
+        if (tid < kQTile) { lse_s[1][tid] = lse1 * kLog2e; dsm_s[1][tid] = -dsm1; }
+      }
+      if (n_tiles > 2) gload();
+      __syncthreads();
+    }
+  } else if (n_tiles > 0) {
     gload();
     lstore(0);
     if (n_tiles > 1) { gload(); lstore(1); }
@@ -391,6 +439,40 @@ __global__ void __launch_bounds__(256, (D <= 64 && KB == 1) ? 2 : 1) dkdv_kernel
   for (; m < m_max; ++m) idle_tile();
   }
 
+  if constexpr (kLean) {
+    // the wave's dK and dV rows -> its own [32][D] tiles in the idle Q and dO rings -> whole rows
+    static_assert(KB == 1, "one key block per wave");
+    constexpr int OS = D + 8, CPRO = D / 8, RPI = 64 / CPRO;
+    static_assert(!kLean || 4 * 32 * OS <= kRing * kQTile * QS, "staging must fit the ring");
+    __syncthreads();  // every wave has left the last Q / dO tile
+    T *Kt = &Qs[0][0] + wave * 32 * OS, *Vt = &dOs[0][0] + wave * 32 * OS;
+    typedef T vec4 __attribute__((ext_vector_type(4)));
+#pragma unroll
+    for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+      for (int i4 = 0; i4 < 4; ++i4) {
+        vec4 a, b;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          a[j] = (T)(dk_acc[0][db][i4 * 4 + j] * p.scale);
+          b[j] = (T)(dv_acc[0][db][i4 * 4 + j]);
+        }
+        *reinterpret_cast<vec4 *>(&Kt[r32 * OS + db * 32 + i4 * 8 + g * 4]) = a;
+        *reinterpret_cast<vec4 *>(&Vt[r32 * OS + db * 32 + i4 * 8 + g * 4]) = b;
+      }
+    const int oc = lane % CPRO, orow = lane / CPRO;
+#pragma unroll
+    for (int it = 0; it < 32 / RPI; ++it) {
+      const int r = it * RPI + orow, kv = wkv0 + r;
+      const uint4 a = *reinterpret_cast<const uint4 *>(&Kt[r * OS + oc * 8]);
+      const uint4 b = *reinterpret_cast<const uint4 *>(&Vt[r * OS + oc * 8]);
+      if (kv < p.sk) {
+        *reinterpret_cast<uint4 *>(static_cast<T *>(p.dk) + bi * p.k_bs + (int64_t)kv * p.k_rs + hk * p.k_hs + oc * 8) = a;
+        *reinterpret_cast<uint4 *>(static_cast<T *>(p.dv) + bi * p.v_bs + (int64_t)kv * p.v_rs + hk * p.v_hs + oc * 8) = b;
+      }
+    }
+    return;
+  }
 #pragma unroll
   for (int kb = 0; kb < KB; ++kb) {
     if (kvcol[kb] < p.sk) {
@@ -659,11 +741,18 @@ hipError_t launch_bwd_td(const Params &p, hipStream_t stream) {
   pk.xcd_remap = ((p.b * p.h_k) % 8 == 0) ? (p.wr >= 0 ? 2 : 1) : (p.wr >= 0 ? 3 : 0);
   if (pk.n_nblocks > 0)
     dkdv_kernel<T, D, KB><<<dim3((unsigned)(pk.n_nblocks * p.b * p.h_k)), dim3(256), 0, stream>>>(pk);
-  Params pq = p;
-  pq.n_mblocks = (p.sq + kQBlock - 1) / kQBlock;
-  if (pq.n_mblocks > 0)
-    dq_kernel<T, D><<<dim3((unsigned)(pq.n_mblocks * p.b * p.h)), dim3(256), 0, stream>>>(pq);
-  return hipGetLastError();
+  if constexpr (D == 128) {
+    // dq_kernel needs a whole SIMD per wave at this head dimension; the generic dQ kernel fits
+    // two and is faster
+    const hipError_t e = hipGetLastError();
+    return e != hipSuccess ? e : launch_dq_anyd128(p, std::is_same<T, _Float16>::value ? 1 : 2, stream);
+  } else {
+    Params pq = p;
+    pq.n_mblocks = (p.sq + kQBlock - 1) / kQBlock;
+    if (pq.n_mblocks > 0)
+      dq_kernel<T, D><<<dim3((unsigned)(pq.n_mblocks * p.b * p.h)), dim3(256), 0, stream>>>(pq);
+    return hipGetLastError();
+  }
 }
 
 template <typename T>

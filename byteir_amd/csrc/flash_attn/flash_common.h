@@ -192,6 +192,7 @@ __device__ __forceinline__ void row_limits(const Params &p, int q, int &lo, int 
 // have set everything in `p` but the block counts.
 hipError_t launch_fwd_anyd(Params &p, int dtype, hipStream_t stream);
 hipError_t launch_bwd_anyd(Params &p, int dtype, hipStream_t stream);
+hipError_t launch_dq_anyd128(const Params &p, int dtype, hipStream_t stream);
 
 // A few query rows against a long key sequence (flash_decode.hip): all query heads of a
 // key/value head times all query rows must fit the 32 columns of one score tile.
