@@ -24,7 +24,8 @@
  * [batch, heads, seqlen_q] float.
  *
  * Supported here: head_dim a multiple of 8 up to 256 (the reference's range; 32, 64 and 128
- * have tuned kernels), 0 <= p_dropout < 1, any seqlen, h % h_k == 0
+ * have tuned kernels), 0 <= p_dropout < 1, any seqlen including 0 (tensors of a side without rows
+ * may be NULL), h % h_k == 0
  * (backward with h_k < h: dK, dV of a key/value head are the sums over its query heads -- the
  * gradient; the reference's own addressing of dK / dV is only right for h == h_k).  Anything else is reported on stderr and the process aborts, since
  * the ABI has no error channel; the *_checked variants return an error code instead.
@@ -70,7 +71,8 @@ void run_flash_attn_bwd_bf16(void **tensors, void *extra_args, void *stream);
  * First k_new / v_new are written into the caches at rows seqlens_k[b] .. +seqlen_knew (in
  * place), then q attends to rows [0, seqlens_k[b] + seqlen_knew) of its batch, with the window
  * aligned to the end of that range (block_info.h:27-37, mask.h:160-200).  No rotary embedding
- * (the reference sets rotary_dim = 0), one split.  k_new / v_new may both be NULL (no append);
+ * (the reference sets rotary_dim = 0; it also fixes one split, whereas here the key axis is
+ * split over workgroups when that fills the chip).  k_new / v_new may both be NULL (no append);
  * seqlens_k may be NULL only then (all seqlen_k rows are attended).
  * extra_args (244 bytes): i64 q,k,v,knew,vnew,o batch_stride; the same six row_strides; the
  * same six head_strides; i64 b, h, h_k, d, d_rounded, seqlen_knew; f32 softmax_scale;
