@@ -143,7 +143,7 @@ private:
 
 // ---- byteir.softmax -----------------------------------------------------------------------------------
 // A new op kernel (the reference runtime has none): operands (input, output), attribute `axis`,
-// which must name the last axis; element type f32, f16 or bf16.
+// (any axis of the tensor, the last one by default); element type f32, f16 or bf16.
 class SoftmaxOpKernel : public OpKernel {
 public:
   explicit SoftmaxOpKernel(const OpKernelInfo &info) : OpKernel(info) {
