@@ -612,6 +612,48 @@ def test_decode_call_inside_a_hip_graph():
         assert torch.equal(kc_graph, kc), step
 
 
+@pytest.mark.parametrize("d,p_drop", [(64, 0.0), (128, 0.0), (80, 0.0), (64, 0.1)])
+def test_training_step_inside_a_hip_graph(d, p_drop):
+    """Forward and backward captured together (no call on this path allocates); replays with new
+    inputs, with eager work in between, must match the eager calls bit for bit."""
+    from byteir_amd import ops
+    b, s, h, h_k = 2, 700, 4, 2
+    gen = torch.Generator(device="cuda").manual_seed(d)
+    mk = lambda *sh: torch.randn(sh, generator=gen, device="cuda").bfloat16()
+    q, k, v, do = mk(b, s, h, d), mk(b, s, h_k, d), mk(b, s, h_k, d), mk(b, s, h, d)
+    rng = ops.rng_state_tensor(11, 22, "cuda")
+    scale, win = 1.0 / np.sqrt(d), (-1, 0)
+    o = torch.empty_like(q)
+    lse = torch.empty((b, h, s), dtype=torch.float32, device="cuda")
+    bufs = ops.flash_attn_bwd_buffers(q, k, v)
+
+    def step(stream):
+        ops.flash_attn_fwd(q, k, v, scale, win, stream=stream, out=(o, lse, rng), p_dropout=p_drop, rng_state=rng)
+        ops.flash_attn_bwd(do, q, k, v, o, lse, scale, win, stream=stream, out=bufs, p_dropout=p_drop, rng_state=rng)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step(side)  # warm-up outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        step(side)
+    for it in range(3):
+        for t in (q, k, v, do):
+            t.copy_(mk(*t.shape))
+        rng.copy_(ops.rng_state_tensor(100 + it, 7 * it, "cuda"))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in (o, lse, *bufs[:3])]
+        o2, lse2 = ops.flash_attn_fwd(q, k, v, scale, win, p_dropout=p_drop, rng_state=rng)
+        dq2, dk2, dv2 = ops.flash_attn_bwd(do, q, k, v, o2, lse2, scale, win, p_dropout=p_drop, rng_state=rng)
+        torch.cuda.synchronize()
+        for a, c in zip(got, (o2, lse2, dq2, dk2, dv2)):
+            assert torch.equal(a, c), it
+
+
 def test_decode_benchmark_size_sampled_heads():
     """The benchmark's decode call (fp16, 64 sequences with up to 8192 cached keys, 32 query heads on
     8 key/value heads of 128, one new token): ragged lengths, the appended rows land in the caches
