@@ -425,3 +425,38 @@ def test_intermediates_live_in_one_arena_per_frame():
     assert torch.equal(y, x.amax(dim=1))
     req.close()
     s.close()
+
+
+def test_op_kernels_on_two_streams_at_once():
+    """Nothing in the kernel libraries is shared between calls (workspaces are per call or
+    stream-ordered): the same work issued on two streams at once gives the serial results."""
+    from byteir_amd import ops, _lib
+    gen = torch.Generator(device="cuda").manual_seed(3)
+    work = []
+    for i in range(2):
+        x = torch.randn((4096, 2048), generator=gen, device="cuda")
+        q = torch.randn((1, 64, 8, 128), generator=gen, device="cuda").half()      # few query blocks, many keys:
+        k = torch.randn((1, 5000, 2, 128), generator=gen, device="cuda").half()    # key axis split, scratch allocation
+        v = torch.randn_like(k)
+        xs = torch.randn((1, 9000, 24), generator=gen, device="cuda")              # segmented inner-axis softmax
+        work.append((x, q, k, v, xs))
+
+    def run(i, stream):
+        x, q, k, v, xs = work[i]
+        r = ops.reduce(_lib.REDUCE_SUM, x, (0,), stream=stream)
+        o, lse = ops.flash_attn_fwd(q, k, v, 0.1, (-1, 0), stream=stream)
+        y = ops.softmax(xs, stream=stream, axis=1)
+        return r, o, lse, y
+
+    serial = [run(i, None) for i in range(2)]
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    for _ in range(3):
+        both = []
+        for i, s in enumerate(streams):
+            with torch.cuda.stream(s):
+                both.append(run(i, s))
+        torch.cuda.synchronize()
+        for got, want in zip(both, serial):
+            for a, c in zip(got, want):
+                assert torch.equal(a, c)
