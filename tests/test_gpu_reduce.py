@@ -241,3 +241,36 @@ def test_baseline_config2_full_size():
     s1 = ops.reduce(oracle.SUM, dx, (0,))
     s2 = ops.reduce(oracle.SUM, dx * 2, (0,))
     assert torch.equal(s2, s1 * 2)
+
+
+def test_random_shapes_sweep():
+    """Forty seeded random [A, B, C] views (odd extents, tiny and long axes, both storage types,
+    unaligned base pointers): sum within the documented tolerance, max and min bit-exact."""
+    from byteir_amd import ops
+    rng = np.random.default_rng(2024)
+    for case in range(40):
+        A = int(rng.choice([1, 2, 3, 7, 64, 300]))
+        B = int(rng.choice([1, 2, 5, 33, 127, 1000, 4099, 70001]))
+        C = int(rng.choice([1, 1, 1, 2, 3, 8, 33, 260, 1027]))
+        while A * B * C > 3_000_000:
+            if A > 1: A //= 2
+            elif C > 1: C //= 2
+            else: B //= 2
+        dtype = np.float16 if case % 3 == 2 else np.float32
+        off = int(rng.integers(0, 4))  # elements into the allocation: 16-byte alignment is not a given
+        x = rng.standard_normal(A * B * C).astype(dtype)
+        buf = torch.zeros(A * B * C + 8, dtype=torch.float16 if dtype == np.float16 else torch.float32, device="cuda")
+        view = buf[off:off + A * B * C]
+        view.copy_(dev(x))
+        for op in (oracle.SUM, oracle.MAX, oracle.MIN):
+            out = torch.empty(A * C, dtype=view.dtype, device="cuda")
+            ops.reduce_abc(op, view, out, A, B, C)
+            got = host(out)
+            want = oracle.reduce_abc(op, x, A, B, C)
+            if op == oracle.SUM:
+                x64 = x.astype(np.float64).reshape(A, B, C)
+                s64, sabs = x64.sum(axis=1).reshape(-1), np.abs(x64).sum(axis=1).reshape(-1)
+                tol = (2.0 ** -10 * np.abs(s64) + 1e-6 * sabs + 1e-7) if dtype == np.float16 else (1e-5 * np.maximum(np.abs(s64), 1e-2 * sabs) + 1e-30)
+                assert np.all(np.abs(got.astype(np.float64) - s64) <= tol), (case, A, B, C, dtype, off)
+            else:
+                assert np.array_equal(got, want), (case, op, A, B, C, dtype, off)

@@ -158,3 +158,25 @@ def test_baseline_config3_full_size():
     assert (got == want).mean() > 0.98
     sums = y.float().sum(dim=-1, dtype=torch.float64)
     assert float((sums - 1).abs().max()) < 4096 * 2.0 ** -9 * 0.05 + 1e-2
+
+
+def test_random_shapes_sweep():
+    """Thirty seeded random [A, B, C] softmaxes over B (C = 1: rows of any length and alignment;
+    C > 1: an inner axis), all storage types, against the fp64 closed form."""
+    from byteir_amd import ops
+    rng = np.random.default_rng(77)
+    for case in range(30):
+        A = int(rng.choice([1, 2, 5, 40]))
+        B = int(rng.choice([1, 3, 17, 130, 1000, 4097, 9001, 33000, 70003]))
+        C = int(rng.choice([1, 1, 1, 2, 7, 24, 128, 1030]))
+        while A * B * C > 2_000_000:
+            if A > 1: A //= 2
+            elif C > 1: C //= 2
+            else: B //= 2
+        code = [oracle.F32, oracle.F16, oracle.BF16][case % 3]
+        x32 = (rng.standard_normal((A, B, C)) * 2.0).astype(np.float32)
+        xs = oracle.from_f32(x32, code)
+        got = oracle.to_f32(host(ops.softmax(dev(xs), axis=1)))
+        want = sp_softmax(oracle.to_f32(xs).astype(np.float64), axis=1).astype(np.float32)
+        rel, ab = TOL[code]
+        assert np.all(np.abs(got - want) <= rel * np.abs(want) + ab), (case, A, B, C, code)
