@@ -245,6 +245,44 @@ def test_large_and_drifting_scores(shape, trend, code):
         assert err.max() <= ATOL + 2 * ulp * np.abs(w32).max(), (name, float(err.max()), float(np.abs(w32).max()))
 
 
+def test_random_cases_sweep():
+    """Thirty seeded random calls (sequence lengths, grouped heads, head dimensions, windows on
+    either or both sides, both storage types): forward and backward against plain float attention."""
+    from byteir_amd import ops
+    rng = np.random.default_rng(31337)
+    for case in range(30):
+        d = int(rng.choice([32, 64, 128, 128, 64, 40, 96, 256]))
+        h_k = int(rng.choice([1, 2, 3]))
+        h = h_k * int(rng.choice([1, 1, 2, 4]))
+        b = int(rng.choice([1, 2]))
+        sq = int(rng.choice([1, 3, 31, 64, 129, 300, 517]))
+        sk = int(rng.choice([1, 33, 64, 200, 517, 1100, 2600]))
+        while b * h * sq * sk * d > 1.5e8:
+            if sk > 600: sk //= 2
+            elif b > 1: b = 1
+            else: sq = max(1, sq // 2)
+        wl = int(rng.choice([-1, -1, 0, 17, 200]))
+        wr = int(rng.choice([-1, 0, 0, 5, 64]))
+        code = oracle.F16 if case % 2 else oracle.BF16
+        shape = (b, sq, sk, h, h_k, d, (wl, wr))
+        q, k, v, do = make_inputs(shape, code, seed=case)
+        scale = 1.0 / np.sqrt(d)
+        dq_, dk_, dv_, do_ = (dev(t) for t in (q, k, v, do))
+        o, lse = ops.flash_attn_fwd(dq_, dk_, dv_, scale, (wl, wr))
+        o_ref, lse_ref, o32 = oracle.flash_fwd(q, k, v, scale, (wl, wr), round_p=False)
+        assert np.abs(oracle.to_f32(host(o)) - o32).max() <= ATOL, shape
+        got_lse, inf = host(lse), np.isposinf(lse_ref)
+        assert np.array_equal(np.isposinf(got_lse), inf), shape
+        assert (~inf).sum() == 0 or np.abs(got_lse[~inf] - lse_ref[~inf]).max() <= ATOL, shape
+        dq, dk, dv = ops.flash_attn_bwd(do_, dq_, dk_, dv_, o, lse, scale, (wl, wr))
+        rq, rk, rv, _ = oracle.flash_bwd(do, q, k, v, host(o), host(lse), scale, (wl, wr), round_p=False)
+        ulp = 2.0 ** -10 if code == oracle.F16 else 2.0 ** -7
+        for name, got, want in (("dq", dq, rq), ("dk", dk, rk), ("dv", dv, rv)):
+            w32 = oracle.to_f32(want)
+            err = np.abs(oracle.to_f32(host(got)) - w32)
+            assert np.all(err <= ATOL + ulp * np.abs(w32)), (name, shape, float(err.max()))
+
+
 STRIDED_CASES = [
     # layout, b, sq, sk, h, h_k, d, window
     ("packed_qkv", 2, 192, 192, 4, 4, 64, (-1, 0)),       # q, k, v are slices of one [b, s, 3, h, d] tensor
