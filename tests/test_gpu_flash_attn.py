@@ -505,6 +505,45 @@ def test_kvcache_matches_oracle(case, code):
     np.testing.assert_allclose(host(lse), lse_ref, atol=2e-3, rtol=1e-4)
 
 
+def test_kvcache_random_cases_sweep():
+    """Thirty seeded random cache calls: query rows, grouped heads, head dimensions, capacities,
+    per-batch lengths (including empty and full), appends of several rows, windows."""
+    from byteir_amd import ops
+    rng = np.random.default_rng(4242)
+    for case in range(30):
+        d = int(rng.choice([32, 64, 128, 128, 80, 256]))
+        h_k = int(rng.choice([1, 2, 4]))
+        h = h_k * int(rng.choice([1, 2, 4, 8]))
+        b = int(rng.choice([1, 2, 3]))
+        sq = int(rng.choice([1, 1, 2, 5, 40, 130]))
+        cap = int(rng.choice([64, 200, 1000, 3000, 7000]))
+        append = bool(rng.integers(0, 4) > 0)
+        n_new = sq if append else 0
+        while b * h * sq * cap * d > 1.2e8:
+            if cap > 500: cap //= 2
+            elif b > 1: b -= 1
+            else: sq = max(1, sq // 2); n_new = sq if append else 0
+        lens = [int(rng.choice([0, 1, max(0, cap - n_new), int(rng.integers(0, cap - n_new + 1))])) for _ in range(b)]
+        window = (int(rng.choice([-1, -1, 50, 300])), int(rng.choice([-1, 0, 0])))
+        code = oracle.F16 if case % 2 else oracle.BF16
+        mk = lambda *sh: oracle.from_f32(rng.standard_normal(sh).astype(np.float32), code)
+        q, kc, vc = mk(b, sq, h, d), mk(b, cap, h_k, d), mk(b, cap, h_k, d)
+        kn, vn = (mk(b, n_new, h_k, d), mk(b, n_new, h_k, d)) if append else (None, None)
+        lens_a = np.array(lens, dtype=np.int32)
+        scale = 1.0 / np.sqrt(d)
+        dkc, dvc = dev(kc), dev(vc)
+        o, lse = ops.flash_attn_kvcache(dev(q), dkc, dvc, dev(kn) if append else None, dev(vn) if append else None,
+                                        dev(lens_a), scale, window)
+        o_ref, lse_ref, kc_ref, vc_ref = oracle.flash_kvcache(q, kc, vc, kn, vn, lens_a, scale, window)
+        o32, _, _, _ = oracle.flash_kvcache(q, kc, vc, kn, vn, lens_a, scale, window, round_p=False)
+        what = (case, b, sq, h, h_k, d, cap, lens, window, append)
+        assert np.array_equal(host(dkc), kc_ref) and np.array_equal(host(dvc), vc_ref), what
+        assert np.abs(oracle.to_f32(host(o)) - oracle.to_f32(o32)).max() <= ATOL, what
+        got_lse, inf = host(lse), np.isposinf(lse_ref)
+        assert np.array_equal(np.isposinf(got_lse), inf), what
+        assert (~inf).sum() == 0 or np.abs(got_lse[~inf] - lse_ref[~inf]).max() <= 2e-3 + 1e-4 * np.abs(lse_ref[~inf]).max(), what
+
+
 def test_kvcache_unsupported_arguments_are_reported_not_run():
     import ctypes
     from byteir_amd import _lib, ops
