@@ -49,8 +49,30 @@ int brt_rocm_memcpy_d2h(void *dst, const void *src, size_t bytes, void *stream) 
 int brt_rocm_memcpy_d2d(void *dst, const void *src, size_t bytes, void *stream) {
   return hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, static_cast<hipStream_t>(stream));
 }
+// A fill kernel instead of hipMemsetAsync: a caller may capture the call in a HIP graph, and
+// memset nodes have given wrong results on replays after the first on these machines.  Bytes
+// before the first and after the last 16-byte boundary are written one by one.
+__global__ void __launch_bounds__(256) fill_bytes_kernel(unsigned char *dst, unsigned value, size_t bytes) {
+  size_t head = (16 - (reinterpret_cast<uintptr_t>(dst) & 15)) & 15;
+  if (head > bytes) head = bytes;
+  const size_t body = (bytes - head) / 16, tail = bytes - head - body * 16;
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x, stride = (size_t)gridDim.x * 256;
+  const unsigned w = value * 0x01010101u;
+  for (size_t i = idx; i < head; i += stride) dst[i] = (unsigned char)value;
+  uint4 *mid = reinterpret_cast<uint4 *>(dst + head);
+  for (size_t i = idx; i < body; i += stride) mid[i] = uint4{w, w, w, w};
+  for (size_t i = idx; i < tail; i += stride) dst[head + body * 16 + i] = (unsigned char)value;
+}
+
 int brt_rocm_memset(void *dst, int value, size_t bytes, void *stream) {
-  return hipMemsetAsync(dst, value, bytes, static_cast<hipStream_t>(stream));
+  if (bytes == 0) return hipSuccess;
+  if (!dst) return hipErrorInvalidValue;
+  size_t blocks = (bytes / 16 + 255) / 256;
+  if (blocks < 1) blocks = 1;
+  if (blocks > 8192) blocks = 8192;
+  fill_bytes_kernel<<<dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(
+      static_cast<unsigned char *>(dst), (unsigned)value & 0xffu, bytes);
+  return hipGetLastError();
 }
 
 int brt_rocm_stream_create(void **stream) {

@@ -61,7 +61,7 @@ int brt_rocm_host_free(void *ptr);
 int brt_rocm_memcpy_h2d(void *dst, const void *src, size_t bytes, void *stream);
 int brt_rocm_memcpy_d2h(void *dst, const void *src, size_t bytes, void *stream);
 int brt_rocm_memcpy_d2d(void *dst, const void *src, size_t bytes, void *stream);
-int brt_rocm_memset(void *dst, int value, size_t bytes, void *stream);
+int brt_rocm_memset(void *dst, int value, size_t bytes, void *stream); /* a fill kernel, safe to capture in a HIP graph */
 /* device-to-device copy done by a plain compute kernel (128-bit loads and stores) rather than
  * a DMA engine: the cuda2cuda copy of runtime/lib/backends/cuda/providers/default/copy/copy.cc
  * for buffers that are multiples of 16 bytes and 16-byte aligned, and the known-traffic

@@ -460,3 +460,31 @@ def test_op_kernels_on_two_streams_at_once():
         for got, want in zip(both, serial):
             for a, c in zip(got, want):
                 assert torch.equal(a, c)
+
+
+def test_device_memset_any_alignment_and_inside_a_graph():
+    """brt_rocm_memset (the DeviceAPI memset of cuda_device_api.cc:29-55) is a fill kernel: every
+    byte of the range and none outside it, for any alignment and length; replays of a captured
+    call keep working."""
+    import ctypes
+    from byteir_amd import _lib
+    K = _lib.kernels()
+    buf = torch.zeros(5000, dtype=torch.uint8, device="cuda")
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    for off, n, val in ((0, 5000, 7), (1, 4998, 200), (13, 3, 9), (16, 16, 1), (31, 1000, 255), (5, 0, 3)):
+        buf.fill_(0x55)
+        _lib.check(K.brt_rocm_memset(ctypes.c_void_p(buf.data_ptr() + off), val, n, st), "memset")
+        h = buf.cpu().numpy()
+        assert np.all(h[off:off + n] == val) and np.all(h[:off] == 0x55) and np.all(h[off + n:] == 0x55), (off, n)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        _lib.check(K.brt_rocm_memset(ctypes.c_void_p(buf.data_ptr() + 3), 0, 4001, ctypes.c_void_p(side.cuda_stream)), "memset")
+    for _ in range(3):
+        buf.fill_(0x77)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        h = buf.cpu().numpy()
+        assert np.all(h[3:4004] == 0) and np.all(h[:3] == 0x77) and np.all(h[4004:] == 0x77)
