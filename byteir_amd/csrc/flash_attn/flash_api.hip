@@ -166,6 +166,8 @@ int flash_attn_bwd_checked(void **tensors, const void *extra_args, int dtype, vo
   p.rng_state = static_cast<const uint64_t *>(tensors[6]);
   p.dq = tensors[7]; p.dk = tensors[8]; p.dv = tensors[9];
   p.dsoftmax = static_cast<float *>(tensors[10]);
+  p.dq_accum = tensors[11];
+  p.dq_accum_bytes = p.dq_accum ? (size_t)a.b * (size_t)a.seqlen_q_rounded * (size_t)a.h * (size_t)a.d_rounded * sizeof(float) : 0;
   if (p.b == 0) return 0;
   if (p.drop && !p.rng_state) return fail("p_dropout > 0 needs the rng_state tensor {seed, offset}");
   // a side without rows (seqlen_q == 0 or seqlen_k == 0) may come as null pointers

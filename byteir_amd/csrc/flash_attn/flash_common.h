@@ -146,6 +146,14 @@ struct Params {
   float *lse;                         // [b, h, sq]
   void *dq, *dk, *dv;
   float *dsoftmax;                    // [b, h, sq_rounded]
+  void *dq_accum;                     // the caller's [b, sq_rounded, h, d_rounded] float scratch (may be null)
+  size_t dq_accum_bytes;
+  // dK/dV only: where a workgroup writes its rows (dk / dv with the strides of k / v, or partial
+  // buffers), and, when the query heads of a key/value head are shared out over `gsplit`
+  // workgroups, the factor by which h_k has been multiplied (K and V of virtual head hk are
+  // those of head hk / gsplit)
+  int64_t dk_bs, dk_rs, dk_hs, dv_bs, dv_rs, dv_hs;
+  int gsplit;
   int64_t q_bs, k_bs, v_bs, o_bs;     // batch strides (elements)
   int64_t q_rs, k_rs, v_rs, o_rs;     // row strides
   int64_t q_hs, k_hs, v_hs, o_hs;     // head strides

@@ -53,8 +53,10 @@ void run_flash_attn_fwd(void **tensors, void *extra_args, void *stream);
 /* tensors: {dout, q, k, v, out, softmax_lse, rng_state, dq, dk, dv, d_softmax, dq_accum}
  * (flash_api.cu:696-725).  fp16 storage.  d_softmax is [b, h, seqlen_q_rounded] float scratch
  * that receives rowsum(dout * out) (times 1 - p_dropout, as in the reference); rng_state must
- * hold what the forward call used; dq_accum is accepted and left untouched (dQ is
- * accumulated without atomics by a pass that is parallel over query blocks). */
+ * hold what the forward call used; dq_accum ([b, seqlen_q_rounded, h, d_rounded] float, may be
+ * NULL) is scratch: dQ is accumulated without atomics by a pass that is parallel over query
+ * blocks, and with grouped heads and few key blocks the buffer holds partial dK / dV of the
+ * group's query heads (a stream-ordered allocation supplies what it cannot hold). */
 void run_flash_attn_bwd(void **tensors, void *extra_args, void *stream);
 
 /* The same two entry points for bfloat16 storage.  The reference library is fp16 only
