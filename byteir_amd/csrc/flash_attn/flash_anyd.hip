@@ -389,8 +389,9 @@ __global__ void __launch_bounds__(256, DR <= 64 ? 2 : 1) dkdv_anyd_kernel(const 
 
   const T *qg = nullptr, *dog = nullptr;  // of the query head being streamed (set per head below)
   const float *lse_g = nullptr, *dsm_g = nullptr;
-  const T *kg = static_cast<const T *>(p.k) + bi * p.k_bs + (int64_t)kvcol * p.k_rs + hk * p.k_hs;
-  const T *vg = static_cast<const T *>(p.v) + bi * p.v_bs + (int64_t)kvcol * p.v_rs + hk * p.v_hs;
+  const int hkv = hk / p.gsplit;  // the key/value head whose query heads this workgroup takes a share of
+  const T *kg = static_cast<const T *>(p.k) + bi * p.k_bs + (int64_t)kvcol * p.k_rs + hkv * p.k_hs;
+  const T *vg = static_cast<const T *>(p.v) + bi * p.v_bs + (int64_t)kvcol * p.v_rs + hkv * p.v_hs;
 
   vec8 kf[DR / 16], vf[DR / 16];
 #pragma unroll
@@ -507,12 +508,23 @@ __global__ void __launch_bounds__(256, DR <= 64 ? 2 : 1) dkdv_anyd_kernel(const 
 
   }
   if (kvcol < p.sk) {
-    T *dkg = static_cast<T *>(p.dk) + bi * p.k_bs + (int64_t)kvcol * p.k_rs + hk * p.k_hs;
-    T *dvg = static_cast<T *>(p.dv) + bi * p.v_bs + (int64_t)kvcol * p.v_rs + hk * p.v_hs;
+    const float mk = Drop ? p.scale * p.rp_keep : p.scale, mv = Drop ? p.rp_keep : 1.f;
+    if (p.gsplit > 1) {  // a share of the group's query heads: float partials [b, sk, h_k * gsplit, d]
+      float *dkp = static_cast<float *>(p.dk) + bi * p.dk_bs + (int64_t)kvcol * p.dk_rs + hk * p.dk_hs;
+      float *dvp = static_cast<float *>(p.dv) + bi * p.dv_bs + (int64_t)kvcol * p.dv_rs + hk * p.dv_hs;
 #pragma unroll
-    for (int db = 0; db < DR / 32; ++db) {
-      store_acc<T>(dkg, dk_acc[db], db, g, Drop ? p.scale * p.rp_keep : p.scale, p.d);
-      store_acc<T>(dvg, dv_acc[db], db, g, Drop ? p.rp_keep : 1.f, p.d);
+      for (int db = 0; db < DR / 32; ++db) {
+        store_acc<float>(dkp, dk_acc[db], db, g, mk, p.d);
+        store_acc<float>(dvp, dv_acc[db], db, g, mv, p.d);
+      }
+    } else {
+      T *dkg = static_cast<T *>(p.dk) + bi * p.dk_bs + (int64_t)kvcol * p.dk_rs + hk * p.dk_hs;
+      T *dvg = static_cast<T *>(p.dv) + bi * p.dv_bs + (int64_t)kvcol * p.dv_rs + hk * p.dv_hs;
+#pragma unroll
+      for (int db = 0; db < DR / 32; ++db) {
+        store_acc<T>(dkg, dk_acc[db], db, g, mk, p.d);
+        store_acc<T>(dvg, dv_acc[db], db, g, mv, p.d);
+      }
     }
   }
 }
@@ -659,10 +671,19 @@ template <typename T, int DR>
 hipError_t bwd_anyd_d(const Params &p, hipStream_t stream) {
   const dim3 gk((unsigned)(p.n_nblocks * p.b * p.h_k)), gq((unsigned)(p.n_mblocks * p.b * p.h)), block(256);
   if (p.n_nblocks > 0) {
-    Params pk = p;  // the dK/dV grid runs over key/value heads
-    pk.xcd_remap = ((p.b * p.h_k) % 8 == 0) ? (p.wr >= 0 ? 2 : 1) : (p.wr >= 0 ? 3 : 0);
-    if (p.drop) dkdv_anyd_kernel<T, DR, true><<<gk, block, 0, stream>>>(pk);
-    else dkdv_anyd_kernel<T, DR, false><<<gk, block, 0, stream>>>(pk);
+    Params pk = p;  // the dK/dV grid runs over key/value heads (or shares of their groups)
+    pk.dk_bs = p.k_bs; pk.dk_rs = p.k_rs; pk.dk_hs = p.k_hs;
+    pk.dv_bs = p.v_bs; pk.dv_rs = p.v_rs; pk.dv_hs = p.v_hs;
+    const GroupSplit split = plan_group_split(p, (int64_t)p.n_nblocks * p.b * p.h_k, 256 * (DR <= 64 ? 2 : 1), p.d, stream);
+    apply_group_split(pk, p, split, p.d);
+    pk.xcd_remap = ((p.b * pk.h_k) % 8 == 0) ? (p.wr >= 0 ? 2 : 1) : (p.wr >= 0 ? 3 : 0);
+    const dim3 gks((unsigned)(p.n_nblocks * p.b * pk.h_k));
+    if (p.drop) dkdv_anyd_kernel<T, DR, true><<<gks, block, 0, stream>>>(pk);
+    else dkdv_anyd_kernel<T, DR, false><<<gks, block, 0, stream>>>(pk);
+    if (split.gs > 1) {
+      const hipError_t e = launch_group_sum(p, split, p.d, std::is_same<T, _Float16>::value ? 1 : 2, stream);
+      if (e != hipSuccess) return e;
+    }
   }
   if (p.n_mblocks > 0) {
     if (p.drop) dq_anyd_kernel<T, DR, true><<<gq, block, 0, stream>>>(p);

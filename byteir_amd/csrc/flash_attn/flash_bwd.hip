@@ -745,24 +745,24 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) dq_kernel(const Params p
 }
 
 // dk, dv = sums over the `gs` partial heads per key/value head; partials are float
-// [b, sk, h_k*gs, D], one thread per 16 bytes of output, one rounding.
-template <typename T, int D>
-__global__ void __launch_bounds__(256) group_sum_kernel(const Params p, const void *dk_part, const void *dv_part, int gs) {
-  constexpr int CPR = D / 8;
+// [b, sk, h_k*gs, row] (row = head_dim), one thread per 16 bytes of output, one rounding.
+template <typename T>
+__global__ void __launch_bounds__(256) group_sum_kernel(const Params p, const void *dk_part, const void *dv_part, int gs, int row) {
+  const int cpr = row / 8;
   const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  const int64_t chunks = (int64_t)p.b * p.sk * p.h_k * CPR;
+  const int64_t chunks = (int64_t)p.b * p.sk * p.h_k * cpr;
   if (idx >= chunks) return;
-  const int c = (int)(idx % CPR);
-  const int hk = (int)((idx / CPR) % p.h_k);
-  const int64_t row = idx / ((int64_t)CPR * p.h_k);  // batch * sk + key
-  const int kv = (int)(row % p.sk), bi = (int)(row / p.sk);
-  const int64_t src = ((row * p.h_k + hk) * gs) * D + c * 8;
+  const int c = (int)(idx % cpr);
+  const int hk = (int)((idx / cpr) % p.h_k);
+  const int64_t r = idx / ((int64_t)cpr * p.h_k);  // batch * sk + key
+  const int kv = (int)(r % p.sk), bi = (int)(r / p.sk);
+  const int64_t src = ((r * p.h_k + hk) * gs) * row + c * 8;
   float ak[8], av[8];
 #pragma unroll
   for (int j = 0; j < 8; ++j) { ak[j] = 0.f; av[j] = 0.f; }
   for (int s = 0; s < gs; ++s) {
-    const float4 *rk = reinterpret_cast<const float4 *>(static_cast<const float *>(dk_part) + src + (int64_t)s * D);
-    const float4 *rv = reinterpret_cast<const float4 *>(static_cast<const float *>(dv_part) + src + (int64_t)s * D);
+    const float4 *rk = reinterpret_cast<const float4 *>(static_cast<const float *>(dk_part) + src + (int64_t)s * row);
+    const float4 *rv = reinterpret_cast<const float4 *>(static_cast<const float *>(dv_part) + src + (int64_t)s * row);
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
       const float4 k4 = rk[half], v4 = rv[half];
@@ -777,12 +777,6 @@ __global__ void __launch_bounds__(256) group_sum_kernel(const Params p, const vo
   *reinterpret_cast<uint4 *>(static_cast<T *>(p.dk) + bi * p.k_bs + (int64_t)kv * p.k_rs + hk * p.k_hs + c * 8) = ok;
   *reinterpret_cast<uint4 *>(static_cast<T *>(p.dv) + bi * p.v_bs + (int64_t)kv * p.v_rs + hk * p.v_hs + c * 8) = ov;
 }
-
-// Rounds of dK/dV workgroups wanted when a window makes them unequal.  Measured (bf16, causal,
-// 32 query heads on 8; one / two / four rounds): D = 64 b1 s8192 1235 / 1083 / 1050 us,
-// b4 s4096 h16/4 637 / 571 / 570, b8 s2048 615 / 604 / 652; D = 128 b1 s4096 h32/4
-// 838 / 626 / 626, b4 s2048 626 / 628 / 681.
-constexpr int kGroupRounds = 2;
 
 template <typename T, int D>
 hipError_t launch_bwd_td(const Params &p, hipStream_t stream) {
@@ -801,55 +795,15 @@ hipError_t launch_bwd_td(const Params &p, hipStream_t stream) {
   pk.dk_bs = p.k_bs; pk.dk_rs = p.k_rs; pk.dk_hs = p.k_hs;
   pk.dv_bs = p.v_bs; pk.dv_rs = p.v_rs; pk.dv_hs = p.v_hs;
   pk.gsplit = 1;
-  // Grouped heads with few key blocks (one or two sequences per GPU): a workgroup per key/value
-  // head and key block leaves most CUs idle, so the query heads of a group are shared out over
-  // `gsplit` workgroups that write float partials of dK / dV, summed over the group (and
-  // rounded once) by a second kernel.  The partials take the caller's dq_accum scratch as far
-  // as it reaches, a stream-ordered allocation for the rest.
-  const int group = p.h / p.h_k;
-  const int64_t base_wg = (int64_t)pk.n_nblocks * p.b * p.h_k;
-  void *ws = nullptr;
-  bool ws_owned = false;
-  // wanted: one round of workgroups over the chip's slots (256 CUs, two workgroups each up to
-  // head_dim 64); more rounds when a window makes them unequal, so that the longest-first
-  // order can even them out
-  const int64_t want_wg = (int64_t)(256 * (D <= 64 ? 2 : 1)) * ((p.wr >= 0 || p.wl >= 0) ? kGroupRounds : 1);
-  if (group > 1 && base_wg > 0 && base_wg < want_wg) {
-    int gs = group;
-    for (int c = 2; c <= group; ++c)
-      if (group % c == 0 && base_wg * c >= want_wg) { gs = c; break; }
-    const size_t one = (size_t)p.b * p.sk * p.h_k * gs * D * sizeof(float);
-    const bool aligned = (reinterpret_cast<uintptr_t>(p.dq_accum) & 15) == 0;
-    void *dk_p = nullptr, *dv_p = nullptr;
-    if (p.dq_accum && aligned && p.dq_accum_bytes >= 2 * one) {
-      dk_p = p.dq_accum;
-      dv_p = static_cast<char *>(p.dq_accum) + one;
-    } else if (p.dq_accum && aligned && p.dq_accum_bytes >= one) {
-      if (hipMallocAsync(&ws, one, stream) == hipSuccess) { ws_owned = true; dk_p = p.dq_accum; dv_p = ws; }
-    } else if (hipMallocAsync(&ws, 2 * one, stream) == hipSuccess) {
-      ws_owned = true; dk_p = ws; dv_p = static_cast<char *>(ws) + one;
-    }
-    if (!dk_p) (void)hipGetLastError();  // no scratch: one workgroup per key/value head as before
-    if (dk_p) {
-      pk.gsplit = gs;
-      pk.h_k = p.h_k * gs;
-      pk.dk = dk_p;
-      pk.dv = dv_p;
-      pk.dk_hs = pk.dv_hs = D;
-      pk.dk_rs = pk.dv_rs = (int64_t)pk.h_k * D;
-      pk.dk_bs = pk.dv_bs = (int64_t)p.sk * pk.h_k * D;
-    }
-  }
+  // chip slots for this kernel: 256 CUs, two workgroups each up to head_dim 64
+  const GroupSplit split = plan_group_split(p, (int64_t)pk.n_nblocks * p.b * p.h_k, 256 * (D <= 64 ? 2 : 1), D, stream);
+  apply_group_split(pk, p, split, D);
   pk.xcd_remap = ((p.b * pk.h_k) % 8 == 0) ? (p.wr >= 0 ? 2 : 1) : (p.wr >= 0 ? 3 : 0);
   if (pk.n_nblocks > 0)
     dkdv_kernel<T, D, KB><<<dim3((unsigned)(pk.n_nblocks * p.b * pk.h_k)), dim3(256), 0, stream>>>(pk);
-  if (pk.gsplit > 1) {
-    const int64_t chunks = (int64_t)p.b * p.sk * p.h_k * (D / 8);
-    group_sum_kernel<T, D><<<dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, stream>>>(p, pk.dk, pk.dv, pk.gsplit);
-    if (ws_owned) {
-      const hipError_t f = hipFreeAsync(ws, stream);
-      if (f != hipSuccess) return f;
-    }
+  if (split.gs > 1) {
+    const hipError_t e = launch_group_sum(p, split, D, std::is_same<T, _Float16>::value ? 1 : 2, stream);
+    if (e != hipSuccess) return e;
   }
   if constexpr (D == 128) {
     // dq_kernel needs a whole SIMD per wave at this head dimension; the generic dQ kernel fits
@@ -873,6 +827,22 @@ hipError_t launch_bwd_t(const Params &p, hipStream_t stream) {
   case 128: return launch_bwd_td<T, 128>(p, stream);
   default: return hipErrorInvalidValue;
   }
+}
+
+hipError_t launch_group_sum(const Params &p, const GroupSplit &s, int row, int dtype, hipStream_t stream) {
+  const int64_t chunks = (int64_t)p.b * p.sk * p.h_k * (row / 8);
+  hipError_t e = hipSuccess;
+  if (chunks > 0) {
+    const dim3 grid((unsigned)((chunks + 255) / 256)), block(256);
+    if (dtype == 1) group_sum_kernel<_Float16><<<grid, block, 0, stream>>>(p, s.dk, s.dv, s.gs, row);
+    else group_sum_kernel<__bf16><<<grid, block, 0, stream>>>(p, s.dk, s.dv, s.gs, row);
+    e = hipGetLastError();
+  }
+  if (s.owned) {
+    const hipError_t f = hipFreeAsync(s.owned, stream);
+    if (e == hipSuccess) e = f;
+  }
+  return e;
 }
 
 hipError_t launch_bwd(Params &p, int dtype, hipStream_t stream) {

@@ -202,6 +202,59 @@ hipError_t launch_fwd_anyd(Params &p, int dtype, hipStream_t stream);
 hipError_t launch_bwd_anyd(Params &p, int dtype, hipStream_t stream);
 hipError_t launch_dq_anyd128(const Params &p, int dtype, hipStream_t stream);
 
+// Grouped heads with few key blocks (one or two sequences per GPU): a dK/dV workgroup per
+// key/value head and key block leaves most CUs idle, so the query heads of a group are shared
+// out over `gs` workgroups that write float partials [b, sk, h_k * gs, row] of dK / dV, which
+// launch_group_sum adds (and rounds once).  The partials take the caller's dq_accum scratch as
+// far as it reaches, a stream-ordered allocation for the rest.
+struct GroupSplit {
+  int gs = 1;             // 1: no split
+  void *dk = nullptr, *dv = nullptr;
+  void *owned = nullptr;  // to be released with hipFreeAsync after the sum
+};
+// Rounds of dK/dV workgroups wanted when a window makes them unequal.  Measured (bf16, causal,
+// 32 query heads on 8; one / two / four rounds): D = 64 b1 s8192 1235 / 1083 / 1050 us,
+// b4 s4096 h16/4 637 / 571 / 570, b8 s2048 615 / 604 / 652; D = 128 b1 s4096 h32/4
+// 838 / 626 / 626, b4 s2048 626 / 628 / 681.
+constexpr int kGroupRounds = 2;
+inline GroupSplit plan_group_split(const Params &p, int64_t base_wg, int slots, int row, hipStream_t stream) {
+  GroupSplit r;
+  const int group = p.h / p.h_k;
+  // wanted: one round of workgroups over the chip's slots; more when a window makes them
+  // unequal, so that the longest-first order can even them out
+  const int64_t want_wg = (int64_t)slots * ((p.wr >= 0 || p.wl >= 0) ? kGroupRounds : 1);
+  if (group <= 1 || base_wg <= 0 || base_wg >= want_wg) return r;
+  int gs = group;
+  for (int c = 2; c <= group; ++c)
+    if (group % c == 0 && base_wg * c >= want_wg) { gs = c; break; }
+  const size_t one = (size_t)p.b * p.sk * p.h_k * gs * row * sizeof(float);
+  const bool usable = p.dq_accum && (reinterpret_cast<uintptr_t>(p.dq_accum) & 15) == 0;
+  if (usable && p.dq_accum_bytes >= 2 * one) {
+    r.dk = p.dq_accum;
+    r.dv = static_cast<char *>(p.dq_accum) + one;
+  } else if (usable && p.dq_accum_bytes >= one) {
+    if (hipMallocAsync(&r.owned, one, stream) == hipSuccess) { r.dk = p.dq_accum; r.dv = r.owned; }
+  } else if (hipMallocAsync(&r.owned, 2 * one, stream) == hipSuccess) {
+    r.dk = r.owned;
+    r.dv = static_cast<char *>(r.owned) + one;
+  }
+  if (!r.dk) { (void)hipGetLastError(); r.owned = nullptr; return r; }  // no scratch: no split
+  r.gs = gs;
+  return r;
+}
+// the Params of the dK/dV launch for a split: virtual key/value heads, partial outputs
+inline void apply_group_split(Params &pk, const Params &p, const GroupSplit &s, int row) {
+  pk.gsplit = s.gs;
+  if (s.gs == 1) return;
+  pk.h_k = p.h_k * s.gs;
+  pk.dk = s.dk;
+  pk.dv = s.dv;
+  pk.dk_hs = pk.dv_hs = row;
+  pk.dk_rs = pk.dv_rs = (int64_t)pk.h_k * row;
+  pk.dk_bs = pk.dv_bs = (int64_t)p.sk * pk.h_k * row;
+}
+hipError_t launch_group_sum(const Params &p, const GroupSplit &s, int row, int dtype, hipStream_t stream);
+
 // A few query rows against a long key sequence (flash_decode.hip): all query heads of a
 // key/value head times all query rows must fit the 32 columns of one score tile.
 // merges p.n_splits partials (p.o_part, p.ml_part) into p.o_w and p.lse

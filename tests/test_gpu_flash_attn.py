@@ -629,6 +629,28 @@ def test_dropout_forward_and_backward_match_oracle(case, code):
         assert err <= ATOL, (name, float(err))
 
 
+@pytest.mark.parametrize("d", [64, 128, 96])
+def test_dropout_with_grouped_heads_matches_oracle(d):
+    """Dropout streams are per query head; dK / dV of a key/value head sum over its group (here
+    through the partial buffers, the grid being small)."""
+    from byteir_amd import ops
+    b, s, h, h_k, window, p_drop, code = 1, 300, 8, 2, (-1, 0), 0.15, oracle.BF16
+    q, k, v, do = make_inputs((b, s, s, h, h_k, d, window), code, seed=d)
+    scale = 1.0 / np.sqrt(d)
+    rs = ops.rng_state_tensor(*RNG_STATE, "cuda")
+    dq_, dk_, dv_, do_ = (dev(t) for t in (q, k, v, do))
+    o, lse = ops.flash_attn_fwd(dq_, dk_, dv_, scale, window, p_dropout=p_drop, rng_state=rs)
+    _, lse_ref, o32 = oracle.flash_fwd(q, k, v, scale, window, round_p=False, p_dropout=p_drop, rng_state=RNG_STATE)
+    assert np.abs(oracle.to_f32(host(o)) - o32).max() <= ATOL
+    dq, dk, dv = ops.flash_attn_bwd(do_, dq_, dk_, dv_, o, lse, scale, window, p_dropout=p_drop, rng_state=rs)
+    rq, rk, rv, _ = oracle.flash_bwd(do, q, k, v, host(o), host(lse), scale, window, round_p=False,
+                                     p_dropout=p_drop, rng_state=RNG_STATE)
+    for name, got, want in (("dq", dq, rq), ("dk", dk, rk), ("dv", dv, rv)):
+        w32 = oracle.to_f32(want)
+        err = np.abs(oracle.to_f32(host(got)) - w32)
+        assert np.all(err <= ATOL + 2.0 ** -7 * np.abs(w32)), (name, float(err.max()))
+
+
 def test_dropout_without_rng_state_is_reported():
     import ctypes
     from byteir_amd import _lib, ops
