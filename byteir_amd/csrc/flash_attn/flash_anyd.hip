@@ -382,7 +382,9 @@ __global__ void __launch_bounds__(256, DR <= 64 ? 2 : 1) dkdv_anyd_kernel(const 
   int n_block, bh;
   block_of(p, p.n_nblocks, false, n_block, bh, p.b * p.h_k);
   // a workgroup belongs to a key/value head; its dK, dV sum over the query heads of the group
-  const int bi = bh / p.h_k, hk = bh % p.h_k, group = p.h / p.h_k;
+  // (with shares: bh runs over virtual heads; hk = key/value head * gsplit + group share)
+  const int bi = bh / p.h_k, vh = bh % p.h_k, hk = vh / p.qsplit, q_share = vh % p.qsplit;
+  const int group = p.h / (p.h_k / p.qsplit);
   const int kvb0 = n_block * kRows;
   const int kvcol = kvb0 + wave * 32 + r32;  // the key this lane owns
   const int off = p.sk - p.sq;
@@ -407,8 +409,13 @@ __global__ void __launch_bounds__(256, DR <= 64 ? 2 : 1) dkdv_anyd_kernel(const 
   int q_lo = 0, q_hi = p.sq;
   if (p.wr >= 0) q_lo = max(0, kvb0 - off - p.wr);              // hi(q) = q+1+off+wr > kvb0
   if (p.wl >= 0) q_hi = min(p.sq, kvb0 + kRows - off + p.wl);   // lo(q) = q+off-wl < kvb0+128
-  const int m_min = q_lo / kTile;
-  const int m_max = q_hi > 0 ? (q_hi + kTile - 1) / kTile : 0;
+  int m_min = q_lo / kTile;
+  int m_max = q_hi > 0 ? (q_hi + kTile - 1) / kTile : 0;
+  if (p.qsplit > 1) {  // this workgroup's share of the visible query tiles
+    const int per = (max(m_max - m_min, 0) + p.qsplit - 1) / p.qsplit;
+    m_min += q_share * per;
+    m_max = min(m_max, m_min + per);
+  }
   const float c = p.scale_log2;
   DropCtx drop;
 
@@ -509,9 +516,9 @@ __global__ void __launch_bounds__(256, DR <= 64 ? 2 : 1) dkdv_anyd_kernel(const 
   }
   if (kvcol < p.sk) {
     const float mk = Drop ? p.scale * p.rp_keep : p.scale, mv = Drop ? p.rp_keep : 1.f;
-    if (p.gsplit > 1) {  // a share of the group's query heads: float partials [b, sk, h_k * gsplit, d]
-      float *dkp = static_cast<float *>(p.dk) + bi * p.dk_bs + (int64_t)kvcol * p.dk_rs + hk * p.dk_hs;
-      float *dvp = static_cast<float *>(p.dv) + bi * p.dv_bs + (int64_t)kvcol * p.dv_rs + hk * p.dv_hs;
+    if (p.gsplit * p.qsplit > 1) {  // a share of the work of a key/value head: float partials [b, sk, virtual heads, d]
+      float *dkp = static_cast<float *>(p.dk) + bi * p.dk_bs + (int64_t)kvcol * p.dk_rs + vh * p.dk_hs;
+      float *dvp = static_cast<float *>(p.dv) + bi * p.dv_bs + (int64_t)kvcol * p.dv_rs + vh * p.dv_hs;
 #pragma unroll
       for (int db = 0; db < DR / 32; ++db) {
         store_acc<float>(dkp, dk_acc[db], db, g, mk, p.d);
@@ -674,13 +681,14 @@ hipError_t bwd_anyd_d(const Params &p, hipStream_t stream) {
     Params pk = p;  // the dK/dV grid runs over key/value heads (or shares of their groups)
     pk.dk_bs = p.k_bs; pk.dk_rs = p.k_rs; pk.dk_hs = p.k_hs;
     pk.dv_bs = p.v_bs; pk.dv_rs = p.v_rs; pk.dv_hs = p.v_hs;
-    const GroupSplit split = plan_group_split(p, (int64_t)p.n_nblocks * p.b * p.h_k, 256 * (DR <= 64 ? 2 : 1), p.d, stream);
+    pk.gsplit = pk.qsplit = 1;
+    const GroupSplit split = plan_group_split(p, (int64_t)p.n_nblocks * p.b * p.h_k, 256 * (DR <= 64 ? 2 : 1), p.d, kTile, stream);
     apply_group_split(pk, p, split, p.d);
     pk.xcd_remap = ((p.b * pk.h_k) % 8 == 0) ? (p.wr >= 0 ? 2 : 1) : (p.wr >= 0 ? 3 : 0);
     const dim3 gks((unsigned)(p.n_nblocks * p.b * pk.h_k));
     if (p.drop) dkdv_anyd_kernel<T, DR, true><<<gks, block, 0, stream>>>(pk);
     else dkdv_anyd_kernel<T, DR, false><<<gks, block, 0, stream>>>(pk);
-    if (split.gs > 1) {
+    if (split.gs * split.qs > 1) {
       const hipError_t e = launch_group_sum(p, split, p.d, std::is_same<T, _Float16>::value ? 1 : 2, stream);
       if (e != hipSuccess) return e;
     }

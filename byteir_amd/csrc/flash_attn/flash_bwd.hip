@@ -167,7 +167,9 @@ __global__ void __launch_bounds__(256, (D <= 64 && KB == 1) ? 2 : 1) dkdv_kernel
     }
   }
   // a workgroup belongs to a key/value head; its dK, dV sum over the query heads of the group
-  const int bi = bh / p.h_k, hk = bh % p.h_k, group = p.h / p.h_k;
+  // (with shares: bh runs over virtual heads; hk = key/value head * gsplit + group share)
+  const int bi = bh / p.h_k, vh = bh % p.h_k, hk = vh / p.qsplit, q_share = vh % p.qsplit;
+  const int group = p.h / (p.h_k / p.qsplit);
   constexpr int kKeys = kKvBlock * KB;
   const int kvb0 = n_block * kKeys;
   const int wkv0 = kvb0 + wave * 32 * KB;  // first key of the wave
@@ -219,8 +221,13 @@ __global__ void __launch_bounds__(256, (D <= 64 && KB == 1) ? 2 : 1) dkdv_kernel
   int q_lo = 0, q_hi = p.sq;
   if (p.wr >= 0) q_lo = max(0, kvb0 - off - p.wr);                 // hi(q) = q+1+off+wr > kvb0
   if (p.wl >= 0) q_hi = min(p.sq, kvb0 + kKeys - off + p.wl);      // lo(q) = q+off-wl < kvb0+kKeys
-  const int m_min = q_lo / kQTile;
-  const int m_max = q_hi > 0 ? (q_hi + kQTile - 1) / kQTile : 0;
+  int m_min = q_lo / kQTile;
+  int m_max = q_hi > 0 ? (q_hi + kQTile - 1) / kQTile : 0;
+  if (p.qsplit > 1) {  // this workgroup's share of the visible query tiles
+    const int per = (max(m_max - m_min, 0) + p.qsplit - 1) / p.qsplit;
+    m_min += q_share * per;
+    m_max = min(m_max, m_min + per);
+  }
   // the same for the wave's own keys [wkv0, wkv0 + 32*KB)
   int qw_lo = 0, qw_hi = p.sq;
   if (p.wr >= 0) qw_lo = max(0, wkv0 - off - p.wr);
@@ -440,12 +447,12 @@ __global__ void __launch_bounds__(256, (D <= 64 && KB == 1) ? 2 : 1) dkdv_kernel
   for (; m < m_max; ++m) idle_tile();
   }
 
-  if (p.gsplit > 1) {  // a share of the group's query heads: float partials [b, sk, h_k * gsplit, D]
+  if (p.gsplit * p.qsplit > 1) {  // a share of the work of a key/value head: float partials [b, sk, virtual heads, D]
 #pragma unroll
     for (int kb = 0; kb < KB; ++kb) {
       if (kvcol[kb] < p.sk) {
-        float *dkp = static_cast<float *>(p.dk) + bi * p.dk_bs + (int64_t)kvcol[kb] * p.dk_rs + hk * p.dk_hs;
-        float *dvp = static_cast<float *>(p.dv) + bi * p.dv_bs + (int64_t)kvcol[kb] * p.dv_rs + hk * p.dv_hs;
+        float *dkp = static_cast<float *>(p.dk) + bi * p.dk_bs + (int64_t)kvcol[kb] * p.dk_rs + vh * p.dk_hs;
+        float *dvp = static_cast<float *>(p.dv) + bi * p.dv_bs + (int64_t)kvcol[kb] * p.dv_rs + vh * p.dv_hs;
 #pragma unroll
         for (int db = 0; db < D / 32; ++db)
 #pragma unroll
@@ -794,29 +801,32 @@ hipError_t launch_bwd_td(const Params &p, hipStream_t stream) {
   pk.n_nblocks = (p.sk + kKvBlock * KB - 1) / (kKvBlock * KB);
   pk.dk_bs = p.k_bs; pk.dk_rs = p.k_rs; pk.dk_hs = p.k_hs;
   pk.dv_bs = p.v_bs; pk.dv_rs = p.v_rs; pk.dv_hs = p.v_hs;
-  pk.gsplit = 1;
+  pk.gsplit = pk.qsplit = 1;
   // chip slots for this kernel: 256 CUs, two workgroups each up to head_dim 64
-  const GroupSplit split = plan_group_split(p, (int64_t)pk.n_nblocks * p.b * p.h_k, 256 * (D <= 64 ? 2 : 1), D, stream);
+  const GroupSplit split = plan_group_split(p, (int64_t)pk.n_nblocks * p.b * p.h_k, 256 * (D <= 64 ? 2 : 1), D, kQTile, stream);
   apply_group_split(pk, p, split, D);
   pk.xcd_remap = ((p.b * pk.h_k) % 8 == 0) ? (p.wr >= 0 ? 2 : 1) : (p.wr >= 0 ? 3 : 0);
   if (pk.n_nblocks > 0)
     dkdv_kernel<T, D, KB><<<dim3((unsigned)(pk.n_nblocks * p.b * pk.h_k)), dim3(256), 0, stream>>>(pk);
-  if (split.gs > 1) {
+  if (split.gs * split.qs > 1) {
     const hipError_t e = launch_group_sum(p, split, D, std::is_same<T, _Float16>::value ? 1 : 2, stream);
     if (e != hipSuccess) return e;
   }
+  Params pq = p;
+  pq.n_mblocks = (p.sq + kQBlock - 1) / kQBlock;
   if constexpr (D == 128) {
     // dq_kernel needs a whole SIMD per wave at this head dimension; the generic dQ kernel fits
-    // two and is faster
-    const hipError_t e = hipGetLastError();
-    return e != hipSuccess ? e : launch_dq_anyd128(p, std::is_same<T, _Float16>::value ? 1 : 2, stream);
-  } else {
-    Params pq = p;
-    pq.n_mblocks = (p.sq + kQBlock - 1) / kQBlock;
-    if (pq.n_mblocks > 0)
-      dq_kernel<T, D><<<dim3((unsigned)(pq.n_mblocks * p.b * p.h)), dim3(256), 0, stream>>>(pq);
-    return hipGetLastError();
+    // two, and once there are two workgroups for every CU they overlap each other and it is
+    // the faster one (3-8 %); on a smaller grid the one-wave kernel's deeper pipeline wins
+    // (b1 h16 s1024 causal backward: 87 against 106 us)
+    if ((int64_t)pq.n_mblocks * p.b * p.h >= 512) {
+      const hipError_t e = hipGetLastError();
+      return e != hipSuccess ? e : launch_dq_anyd128(p, std::is_same<T, _Float16>::value ? 1 : 2, stream);
+    }
   }
+  if (pq.n_mblocks > 0)
+    dq_kernel<T, D><<<dim3((unsigned)(pq.n_mblocks * p.b * p.h)), dim3(256), 0, stream>>>(pq);
+  return hipGetLastError();
 }
 
 template <typename T>
@@ -834,8 +844,8 @@ hipError_t launch_group_sum(const Params &p, const GroupSplit &s, int row, int d
   hipError_t e = hipSuccess;
   if (chunks > 0) {
     const dim3 grid((unsigned)((chunks + 255) / 256)), block(256);
-    if (dtype == 1) group_sum_kernel<_Float16><<<grid, block, 0, stream>>>(p, s.dk, s.dv, s.gs, row);
-    else group_sum_kernel<__bf16><<<grid, block, 0, stream>>>(p, s.dk, s.dv, s.gs, row);
+    if (dtype == 1) group_sum_kernel<_Float16><<<grid, block, 0, stream>>>(p, s.dk, s.dv, s.gs * s.qs, row);
+    else group_sum_kernel<__bf16><<<grid, block, 0, stream>>>(p, s.dk, s.dv, s.gs * s.qs, row);
     e = hipGetLastError();
   }
   if (s.owned) {

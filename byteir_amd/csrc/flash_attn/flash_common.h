@@ -154,6 +154,9 @@ struct Params {
   // those of head hk / gsplit)
   int64_t dk_bs, dk_rs, dk_hs, dv_bs, dv_rs, dv_hs;
   int gsplit;
+  // ... and the number of shares the visible query tiles of a key block are cut into on top of
+  // that (virtual head = (key/value head * gsplit + group share) * qsplit + query share)
+  int qsplit;
   int64_t q_bs, k_bs, v_bs, o_bs;     // batch strides (elements)
   int64_t q_rs, k_rs, v_rs, o_rs;     // row strides
   int64_t q_hs, k_hs, v_hs, o_hs;     // head strides
@@ -208,7 +211,8 @@ hipError_t launch_dq_anyd128(const Params &p, int dtype, hipStream_t stream);
 // launch_group_sum adds (and rounds once).  The partials take the caller's dq_accum scratch as
 // far as it reaches, a stream-ordered allocation for the rest.
 struct GroupSplit {
-  int gs = 1;             // 1: no split
+  int gs = 1;             // shares of a group's query heads; 1: no split
+  int qs = 1;             // shares of a key block's query tiles on top of that
   void *dk = nullptr, *dv = nullptr;
   void *owned = nullptr;  // to be released with hipFreeAsync after the sum
 };
@@ -217,17 +221,33 @@ struct GroupSplit {
 // b4 s4096 h16/4 637 / 571 / 570, b8 s2048 615 / 604 / 652; D = 128 b1 s4096 h32/4
 // 838 / 626 / 626, b4 s2048 626 / 628 / 681.
 constexpr int kGroupRounds = 2;
-inline GroupSplit plan_group_split(const Params &p, int64_t base_wg, int slots, int row, hipStream_t stream) {
+inline GroupSplit plan_group_split(const Params &p, int64_t base_wg, int slots, int row, int q_tile, hipStream_t stream) {
   GroupSplit r;
   const int group = p.h / p.h_k;
   // wanted: one round of workgroups over the chip's slots; more when a window makes them
   // unequal, so that the longest-first order can even them out
   const int64_t want_wg = (int64_t)slots * ((p.wr >= 0 || p.wl >= 0) ? kGroupRounds : 1);
-  if (group <= 1 || base_wg <= 0 || base_wg >= want_wg) return r;
-  int gs = group;
-  for (int c = 2; c <= group; ++c)
-    if (group % c == 0 && base_wg * c >= want_wg) { gs = c; break; }
-  const size_t one = (size_t)p.b * p.sk * p.h_k * gs * row * sizeof(float);
+  if (base_wg <= 0 || base_wg >= want_wg) return r;
+  int gs = 1;
+  if (group > 1) {
+    gs = group;
+    for (int c = 2; c <= group; ++c)
+      if (group % c == 0 && base_wg * c >= want_wg) { gs = c; break; }
+  }
+  // still short: cut the query axis too, at least sixteen tiles per share, at most eight shares
+  // (bf16 backward, with / without: b1 h8 s4096 D=128 causal 242 / 270 us, b1 h4 s2048 D=64
+  // causal 71 / 88, b2 h8 on 2 s2048 D=128 causal 147 / 164; with eight tiles per share
+  // b1 h16 s1024 D=128 causal lost 6 %)
+  int qs = 1;
+  if (base_wg * gs < want_wg) {
+    const int64_t n_q_tiles = (p.sq + q_tile - 1) / q_tile;
+    qs = (int)((want_wg + base_wg * gs - 1) / (base_wg * gs));
+    if (qs > n_q_tiles / 16) qs = (int)(n_q_tiles / 16);
+    if (qs > 8) qs = 8;
+    if (qs < 1) qs = 1;
+  }
+  if (gs * qs == 1) return r;
+  const size_t one = (size_t)p.b * p.sk * p.h_k * gs * qs * row * sizeof(float);
   const bool usable = p.dq_accum && (reinterpret_cast<uintptr_t>(p.dq_accum) & 15) == 0;
   if (usable && p.dq_accum_bytes >= 2 * one) {
     r.dk = p.dq_accum;
@@ -240,13 +260,15 @@ inline GroupSplit plan_group_split(const Params &p, int64_t base_wg, int slots, 
   }
   if (!r.dk) { (void)hipGetLastError(); r.owned = nullptr; return r; }  // no scratch: no split
   r.gs = gs;
+  r.qs = qs;
   return r;
 }
 // the Params of the dK/dV launch for a split: virtual key/value heads, partial outputs
 inline void apply_group_split(Params &pk, const Params &p, const GroupSplit &s, int row) {
   pk.gsplit = s.gs;
-  if (s.gs == 1) return;
-  pk.h_k = p.h_k * s.gs;
+  pk.qsplit = s.qs;
+  if (s.gs * s.qs == 1) return;
+  pk.h_k = p.h_k * s.gs * s.qs;
   pk.dk = s.dk;
   pk.dv = s.dv;
   pk.dk_hs = pk.dv_hs = row;

@@ -80,6 +80,11 @@ CASES = [
     (1, 1000, 1000, 4, 2, 64, (100, 60)),
     (1, 900, 1100, 2, 2, 128, (70, 0)),
     (1, 700, 700, 2, 1, 32, (0, 90)),
+    # long query axis, few heads: the backward cuts a key block's query tiles (and a head group)
+    # into shares over workgroups and sums float partials
+    (1, 2100, 2100, 2, 2, 64, (-1, 0)),
+    (1, 2304, 2304, 4, 2, 128, (-1, -1)),
+    (1, 2200, 2050, 2, 2, 80, (300, 0)),
     # few query rows: the decode kernel (all query heads of a key/value head in one score tile,
     # keys split over waves and, for long sequences, over workgroups)
     (2, 1, 1000, 8, 2, 128, (-1, -1)),
