@@ -31,7 +31,8 @@
  * the ABI has no error channel; the *_checked variants return an error code instead.
  * Calls with few query rows or few query blocks against many keys split the key axis over
  * workgroups and keep their partial results in a stream-ordered allocation
- * (hipMallocAsync / hipFreeAsync on `stream`); no other call allocates.
+ * (hipMallocAsync / hipFreeAsync on `stream`); the backward call does so for partial dK / dV on
+ * small grids when dq_accum cannot hold them; no other call allocates.
  */
 #ifndef BYTEIR_AMD_FLASH_API_H_
 #define BYTEIR_AMD_FLASH_API_H_
