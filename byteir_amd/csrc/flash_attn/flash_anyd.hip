@@ -733,7 +733,8 @@ hipError_t launch_fwd_anyd(Params &p, int dtype, hipStream_t stream) {
 
 // dQ alone, head_dim 128 without dropout, for the tuned backward: at two waves per SIMD (two
 // workgroups per CU, which overlap each other's start and end) this kernel is 3-8 % faster than
-// a kernel tuned for one wave per SIMD (b1 s1024...4096, causal and full).
+// a kernel tuned for one wave per SIMD once the grid has two workgroups for every CU (512...2048
+// heads x 1024...4096 keys, causal and full); the caller keeps the tuned kernel for smaller grids.
 hipError_t launch_dq_anyd128(const Params &p, int dtype, hipStream_t stream) {
   Params pq = p;
   pq.n_mblocks = (p.sq + kRows - 1) / kRows;
