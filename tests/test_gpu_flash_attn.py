@@ -288,6 +288,43 @@ def test_random_cases_sweep():
             assert np.all(err <= ATOL + ulp * np.abs(w32)), (name, shape, float(err.max()))
 
 
+@pytest.mark.parametrize("shape", [
+    (1, 4096, 4096, 16, 4, 128, True),    # grouped heads, shares over workgroups in the backward
+    (1, 4096, 4096, 8, 8, 128, True),     # few heads: query-range shares
+    (2, 3000, 3000, 8, 8, 64, False),
+    (1, 2048, 6000, 4, 2, 96, True),      # generic kernels, sq != sk
+])
+def test_large_shapes_against_float32_matmul_attention_on_the_gpu(shape):
+    """Sizes beyond what the CPU oracle finishes in seconds: the yardstick is plain float32
+    attention (matmul, softmax, matmul) with torch autograd on the same device; 2e-2 absolute
+    plus one storage ulp, as everywhere."""
+    from byteir_amd import ops
+    b, sq, sk, h, h_k, d, causal = shape
+    gen = torch.Generator(device="cuda").manual_seed(sq + h)
+    mk = lambda *sh: torch.randn(sh, generator=gen, device="cuda").bfloat16()
+    q, k, v, do = mk(b, sq, h, d), mk(b, sk, h_k, d), mk(b, sk, h_k, d), mk(b, sq, h, d)
+    scale = 1.0 / np.sqrt(d)
+    win = (-1, 0) if causal else (-1, -1)
+    o, lse = ops.flash_attn_fwd(q, k, v, scale, win)
+    dq, dk, dv = ops.flash_attn_bwd(do, q, k, v, o, lse, scale, win)
+    qf, kf, vf = (t.float().detach().requires_grad_(True) for t in (q, k, v))
+    g = h // h_k
+    kx, vx = kf.repeat_interleave(g, dim=2), vf.repeat_interleave(g, dim=2)
+    sc = torch.einsum("bqhd,bkhd->bhqk", qf, kx) * scale
+    if causal:
+        i = torch.arange(sq, device="cuda")[:, None] + (sk - sq)
+        sc = sc.masked_fill(torch.arange(sk, device="cuda")[None, :] > i, float("-inf"))
+    pr = torch.softmax(sc, dim=-1)
+    o_ref = torch.einsum("bhqk,bkhd->bqhd", pr, vx)
+    o_ref.backward(do.float())
+    ulp = 2.0 ** -7
+    for name, got, want in (("o", o, o_ref.detach()), ("dq", dq, qf.grad), ("dk", dk, kf.grad), ("dv", dv, vf.grad)):
+        err = (got.float() - want).abs()
+        assert bool(torch.all(err <= ATOL + ulp * want.abs())), (name, float(err.max()))
+    lse_ref = torch.logsumexp(sc.detach(), dim=-1)
+    assert float((lse - lse_ref).abs().max()) <= ATOL
+
+
 STRIDED_CASES = [
     # layout, b, sq, sk, h, h_k, d, window
     ("packed_qkv", 2, 192, 192, 4, 4, 64, (-1, 0)),       # q, k, v are slices of one [b, s, 3, h, d] tensor
