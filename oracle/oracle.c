@@ -30,9 +30,12 @@
  *       10-round generator (the library's 7-round call differs in the round count only).
  *   attention dropout                        : the arithmetic around the mask by its closed form
  *       on an explicit mask (tests build it element by element with oracle_dropout_keep) and by
- *       finite differences; the keep rate against the 8-bit threshold.  PARITY UNPINNED for the
- *       element-to-random-byte mapping of oracle_dropout_keep: no reference fixture exercises
- *       dropout and the CUDA kernels cannot be run here.
+ *       finite differences; the keep rate against the 8-bit threshold.  The element-to-random-byte
+ *       mapping of oracle_dropout_keep (no reference fixture exercises dropout) is pinned by a
+ *       thread-by-thread emulation of the reference's own loop nest, lib/dropout.h:26-84 on the
+ *       register fragment of every thread of a block, with the register-to-element map taken
+ *       from the reference's mask code (tests/test_oracle_dropout_layout.py, forward and
+ *       backward tilings, with negative controls).
  *   extra_args blob                          : byte-level known answer from the reference's
  *       fixture module runtime/test/test_files/flash_attn_fwd.mlir:9.
  */
@@ -422,8 +425,9 @@ void oracle_philox4x32(uint64_t seed, uint64_t subsequence, uint64_t offset, int
  * 8*tile + 2*(lane%4) [+1], four 8-column tiles): byte = 4*tile + 2*(row half) + (column & 1).
  * subsequence = (row block, column block) as (low, high) words, offset = rng_state[1] +
  * (batch*heads + head)*32 + lane, seed = rng_state[0]; kept iff byte <= floor(p_keep*255).
- * parity unpinned: no reference fixture exercises dropout, so the element-to-byte mapping above
- * is restated from the sources (and the accumulator layout of the m16n8k16 instruction) only. */
+ * Pinned by tests/test_oracle_dropout_layout.py: every thread of a block is walked through the
+ * loop nest of apply_dropout over its own register fragment, for the forward and the backward
+ * warp tilings; the closed form above must reproduce that bit for bit. */
 int oracle_dropout_keep(const uint64_t *rng_state, int64_t bh, int64_t row, int64_t col, uint8_t threshold) {
   const uint32_t lane = (uint32_t)((row % 8) * 4 + (col % 8) / 2);
   const uint64_t subseq = (uint64_t)(uint32_t)(row / 16) | ((uint64_t)(uint32_t)(col / 32) << 32);

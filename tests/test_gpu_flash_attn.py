@@ -620,7 +620,9 @@ RNG_STATE = (0x9E3779B97F4A7C15, 0x1_0000_0003)   # seed with the top bit set, o
 def test_dropout_mask_is_the_reference_function_of_position(code):
     """V = rows of the identity (head_dim = seqlen_k) makes O[i, :] = keep[i, :] * P[i, :] / p_keep,
     dO = rows of the identity (head_dim = seqlen_q) makes dV[j, :] = the same matrix transposed:
-    the kept set of the forward and of the dK/dV kernel must equal the oracle's mask bit for bit."""
+    the kept set of the forward and of the dK/dV kernel must equal the oracle's mask bit for bit.
+    This is kernel-against-oracle consistency; that the oracle's mask is the reference's function
+    of position is shown on the CPU by tests/test_oracle_dropout_layout.py."""
     from byteir_amd import ops
     b, h, n, p_drop = 2, 3, 256, 0.3
     rng = np.random.default_rng(11)
