@@ -8,6 +8,8 @@ LIB_DIR = os.path.join(_HERE, "lib")
 
 F32, F16, BF16 = 0, 1, 2
 REDUCE_SUM, REDUCE_MAX, REDUCE_MIN, REDUCE_PROD, REDUCE_MEAN, REDUCE_SUMSQR = range(6)
+REDUCE_STATIC_SCRATCH_BYTES = 8 << 20
+ERROR_STATIC_SCRATCH_TOO_SMALL = 20001
 
 
 class LibraryMissing(RuntimeError):
@@ -62,6 +64,7 @@ def kernels():
         L.brt_rocm_reduce_workspace_bytes.restype = sz
         L.brt_rocm_reduce.argtypes = [i32, i32, vp, vp, sz, sz, sz, vp, sz, vp]
         L.brt_rocm_reduce_ex.argtypes = [i32, i32, vp, vp, sz, sz, sz, vp, sz, vp, vp]
+        L.brt_rocm_reduce_static.argtypes = [i32, i32, vp, vp, sz, sz, sz, vp]
         L.brt_rocm_softmax.argtypes = [i32, vp, vp, sz, sz, vp]
         L.brt_rocm_softmax_axis.argtypes = [i32, vp, vp, sz, sz, sz, vp]
         _kernels = L

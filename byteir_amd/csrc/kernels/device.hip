@@ -31,7 +31,12 @@ int brt_rocm_copy_kernel(void *dst, const void *src, size_t bytes, void *stream)
 }
 
 const char *brt_rocm_version(void) { return "byteir-amd 0.1 (gfx950)"; }
-const char *brt_rocm_error_string(int err) { return hipGetErrorString(static_cast<hipError_t>(err)); }
+const char *brt_rocm_error_string(int err) {
+  if (err == BRT_ROCM_ERROR_STATIC_SCRATCH_TOO_SMALL)
+    return "brt_rocm_reduce_static: the split partials of this fold exceed the 8 MiB static scratch "
+           "(BRT_ROCM_REDUCE_STATIC_SCRATCH_BYTES); use brt_rocm_reduce with a caller workspace";
+  return hipGetErrorString(static_cast<hipError_t>(err));
+}
 
 int brt_rocm_device_count(int *count) { return hipGetDeviceCount(count); }
 int brt_rocm_set_device(int device_id) { return hipSetDevice(device_id); }

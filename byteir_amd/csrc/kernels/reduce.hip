@@ -20,6 +20,8 @@
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+
 #include <cstdint>
 #include <type_traits>
 
@@ -525,4 +527,48 @@ extern "C" int brt_rocm_reduce(int op, int dtype, const void *input, void *outpu
                                size_t B, size_t C, void *workspace, size_t workspace_bytes,
                                void *stream) {
   return brt_rocm_reduce_ex(op, dtype, input, output, A, B, C, workspace, workspace_bytes, stream, nullptr);
+}
+
+// ---- the call that allocates nothing ------------------------------------------------------
+// Partials of the split first pass live in a device array that is part of the code object, so
+// every GPU the library is loaded on holds its own copy for the life of the process.  In host
+// code the array's name is only a handle for hipGetSymbolAddress; kernels get the address that
+// call returns, looked up once per device and kept.
+namespace {
+static __device__ __align__(256) float scratch[BRT_ROCM_REDUCE_STATIC_SCRATCH_BYTES / sizeof(float)];
+constexpr int kMaxDevices = 64;
+std::atomic<float *> g_scratch_ptr[kMaxDevices];
+
+hipError_t static_scratch(float **ptr) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+  float *p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (p == nullptr) {
+    void *sym = nullptr;
+    e = hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch));  // address on the current device
+    if (e != hipSuccess) return e;
+    if (sym == nullptr) return hipErrorInvalidSymbol;
+    p = static_cast<float *>(sym);
+    g_scratch_ptr[dev].store(p, std::memory_order_release);  // racing first calls store the same value
+  }
+  *ptr = p;
+  return hipSuccess;
+}
+}  // namespace
+
+extern "C" int brt_rocm_reduce_static(int op, int dtype, const void *input, void *output, size_t A,
+                                      size_t B, size_t C, void *stream) {
+  if (dtype != BRT_ROCM_F32 && dtype != BRT_ROCM_F16) return hipErrorInvalidValue;
+  const size_t need = brt_rocm_reduce_workspace_bytes(dtype, A, B, C);
+  if (need > BRT_ROCM_REDUCE_STATIC_SCRATCH_BYTES) return BRT_ROCM_ERROR_STATIC_SCRATCH_TOO_SMALL;
+  float *ws = nullptr;
+  if (need) {
+    const hipError_t e = static_scratch(&ws);
+    if (e != hipSuccess) return e;
+  }
+  // Every partial the second pass reads is written by the first pass of the same call, so
+  // nothing in the array has to start at zero.
+  return brt_rocm_reduce_ex(op, dtype, input, output, A, B, C, ws, need, stream, nullptr);
 }

@@ -76,6 +76,14 @@ def reduce_abc(op, x, out, A, B, C, workspace=None, stream=None):
     return out
 
 
+def reduce_abc_static(op, x, out, A, B, C, stream=None):
+    """The same fold through brt_rocm_reduce_static: split partials in the library's own device
+    array, no allocation of any kind; raises when the fold needs more than that array holds."""
+    _lib.check(_lib.kernels().brt_rocm_reduce_static(op, _DT[x.dtype], _dev(x), _dev(out), A, B, C,
+                                                     _stream(stream)), "brt_rocm_reduce_static")
+    return out
+
+
 def reduce(op, x, dims, stream=None):
     """Reduce<Op>Op over `dims` of a dense tensor (op: _lib.REDUCE_SUM / MAX / MIN / PROD / MEAN /
     SUMSQR)."""

@@ -107,6 +107,23 @@ int brt_rocm_reduce_ex(int op, int dtype, const void *input, void *output, size_
                        size_t C, void *workspace, size_t workspace_bytes, void *stream,
                        void *first_pass_done);
 
+/* The same fold for callers that must not allocate and have no workspace to hand over (code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
+ * counterpart in the reference, whose ReduceImpl always takes its workspace from the frame's
+ * allocator (reduce_impl.h:76-79).  The partials of the split first pass go to a device array
+ * of BRT_ROCM_REDUCE_STATIC_SCRATCH_BYTES that is part of the library's code object (every GPU
+ * the library runs on holds one for the life of the process); the call makes no hipMalloc,
+ * hipFree or other allocating call.  A fold whose brt_rocm_reduce_workspace_bytes exceeds that
+ * size is refused with BRT_ROCM_ERROR_STATIC_SCRATCH_TOO_SMALL (brt_rocm_error_string names the
+ * limit) before anything is enqueued.  All calls on one GPU share the array: calls that can run
+ * at the same time on one GPU (different streams, different threads) race on it and must be
+ * ordered by the caller.  Nothing in the array needs clearing between calls.  The first call on
+ * a device looks the array's address up (hipGetSymbolAddress); make it outside graph capture. */
+#define BRT_ROCM_REDUCE_STATIC_SCRATCH_BYTES (8u << 20)
+#define BRT_ROCM_ERROR_STATIC_SCRATCH_TOO_SMALL 20001
+int brt_rocm_reduce_static(int op, int dtype, const void *input, void *output, size_t A, size_t B,
+                           size_t C, void *stream);
+
 /* ---- fused row softmax ----------------------------------------------------------- */
 /* y[r, :] = exp(x[r, :] - max_j x[r, j]) / sum_j exp(...) over the last axis of a dense
  * [rows, cols] tensor; float internals for every storage type, one rounding at the store.
