@@ -5,9 +5,11 @@
 // workgroup per column tile, lanes along the contiguous C axis with 128-bit accesses, row lanes
 // along B; one online max/sum pass and a second pass that re-reads the tile and writes.)
 //
-// softmax_wave_kernel keeps a whole row in the registers of one wave (NV 128-bit vectors per
-// lane), so a row is read from HBM once and written once; max and sum are wave64 shuffle
-// trees.  Longer rows, and rows that are not 16-byte aligned, take one workgroup each:
+// softmax_wave_kernel keeps a whole row of up to 128 vectors in the registers of one wave (one
+// or two 128-bit vectors per lane), softmax_split_kernel a row of up to 1024 vectors in those of
+// 2, 4 or 8 waves, so a row is read from HBM once and written once; max and sum are wave64
+// shuffle trees (plus one LDS hop between the waves of a row).  Longer rows, and rows that are
+// not 16-byte aligned, take one workgroup each:
 // softmax_regs_kernel holds the row in the workgroup's registers (up to 65536 elements: one HBM
 // read, one write), softmax_stream_kernel reads longer ones twice (online maximum and sum, then
 // the output pass); both use 128-bit accesses on the aligned span that covers the row.  softmax_block_kernel
@@ -30,21 +32,60 @@ namespace {
 constexpr int kBlock = 256;
 constexpr float kLog2e = 1.4426950408889634f;
 
+// get / make convert one element; unpack / pack convert a whole 128-bit vector held as four
+// 32-bit words (the form in which a vector stays between its load and its use).
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 template <typename T> struct Elem;
 template <> struct Elem<float> {
   static constexpr int EPV = 4;  // elements per 128-bit vector
   static __device__ __forceinline__ float get(const float &v) { return v; }
   static __device__ __forceinline__ float make(float v) { return v; }
+  static __device__ __forceinline__ void unpack(const uint4 &r, float *x) {
+    x[0] = __uint_as_float(r.x); x[1] = __uint_as_float(r.y); x[2] = __uint_as_float(r.z); x[3] = __uint_as_float(r.w);
+  }
+  static __device__ __forceinline__ uint4 pack(const float *x) {
+    return uint4{__float_as_uint(x[0]), __float_as_uint(x[1]), __float_as_uint(x[2]), __float_as_uint(x[3])};
+  }
 };
 template <> struct Elem<__half> {
   static constexpr int EPV = 8;
   static __device__ __forceinline__ float get(const __half &v) { return __half2float(v); }
   static __device__ __forceinline__ __half make(float v) { return __float2half_rn(v); }
+  static __device__ __forceinline__ void unpack(const uint4 &r, float *x) {
+    const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const f16x2 h = __builtin_bit_cast(f16x2, w[j]);
+      x[2 * j] = (float)h.x;
+      x[2 * j + 1] = (float)h.y;
+    }
+  }
+  static __device__ __forceinline__ uint4 pack(const float *x) {
+    uint32_t w[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) w[j] = __builtin_bit_cast(uint32_t, f16x2{(_Float16)x[2 * j], (_Float16)x[2 * j + 1]});  // RNE
+    return uint4{w[0], w[1], w[2], w[3]};
+  }
 };
 template <> struct Elem<__bf16> {
   static constexpr int EPV = 8;
   static __device__ __forceinline__ float get(const __bf16 &v) { return (float)v; }
   static __device__ __forceinline__ __bf16 make(float v) { return (__bf16)v; }  // RNE
+  static __device__ __forceinline__ void unpack(const uint4 &r, float *x) {
+    const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      x[2 * j] = __uint_as_float(w[j] << 16);  // a bf16 is the upper half of a float
+      x[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+    }
+  }
+  static __device__ __forceinline__ uint4 pack(const float *x) {
+    uint32_t w[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) w[j] = __builtin_bit_cast(uint32_t, bf16x2{(__bf16)x[2 * j], (__bf16)x[2 * j + 1]});  // RNE
+    return uint4{w[0], w[1], w[2], w[3]};
+  }
 };
 
 // the tensor is read once and written once: non-temporal accesses keep it out of the caches
@@ -81,21 +122,23 @@ softmax_wave_kernel(const T *__restrict__ in, T *__restrict__ out, uint64_t rows
   const uint4 *src = reinterpret_cast<const uint4 *>(in) + row * nvec;
   uint4 *dst = reinterpret_cast<uint4 *>(out) + row * nvec;
 
+  // Every load is issued unconditionally (a lane beyond the row re-reads the row's last vector
+  // and ignores it): a load under a branch would be waited for before the next one is issued.
   uint4 raw[NV];
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
     const uint32_t v = lane + 64u * i;
-    if (v < nvec) raw[i] = load_stream(src + v);
+    raw[i] = load_stream(src + (v < nvec ? v : nvec - 1));
   }
   float x[NV][EPV];
   float m = -INFINITY;
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
     const bool ok = lane + 64u * i < nvec;
-    const T *e = reinterpret_cast<const T *>(&raw[i]);
+    Elem<T>::unpack(raw[i], x[i]);
 #pragma unroll
     for (int k = 0; k < EPV; ++k) {
-      x[i][k] = ok ? Elem<T>::get(e[k]) : -INFINITY;
+      x[i][k] = ok ? x[i][k] : -INFINITY;
       m = fmaxf(m, x[i][k]);
     }
   }
@@ -114,12 +157,80 @@ softmax_wave_kernel(const T *__restrict__ in, T *__restrict__ out, uint64_t rows
   for (int i = 0; i < NV; ++i) {
     const uint32_t v = lane + 64u * i;
     if (v < nvec) {
-      uint4 o;
-      T *e = reinterpret_cast<T *>(&o);
 #pragma unroll
-      for (int k = 0; k < EPV; ++k) e[k] = Elem<T>::make(x[i][k] * inv);
-      store_stream(dst + v, o);
+      for (int k = 0; k < EPV; ++k) x[i][k] *= inv;
+      store_stream(dst + v, Elem<T>::pack(x[i]));
     }
+  }
+}
+
+// A row shared by RW waves of a 512-thread workgroup, two vectors per lane: the same single
+// read and single write per element as the wave kernel, but in 2 KiB pieces per wave with twice
+// the waves per SIMD.  On MI355X this moves a [32768, 4096] bf16 tensor as fast as a plain copy
+// kernel does (6.4-6.5 TB/s); one wave per 8 KiB row, 8 vectors per lane, reaches 6.1 TB/s, and
+// resident waves that walk the rows with the next row's loads in flight 5.8-6.0 TB/s.
+// FULL: every row is exactly RW * 128 vectors.  Workgroups hold 8 / RW rows; a workgroup's
+// rows beyond the tensor are computed on the last row and not stored (all waves meet the barriers).
+constexpr int kSplitWaves = 8;
+template <typename T, int RW, bool FULL>
+__global__ void __launch_bounds__(kSplitWaves * 64)
+softmax_split_kernel(const T *__restrict__ in, T *__restrict__ out, uint64_t rows, uint32_t nvec) {
+  constexpr int EPV = Elem<T>::EPV;
+  constexpr int NV = 2;
+  __shared__ float red[2][kSplitWaves];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int first = wave / RW * RW;  // first wave of this row
+  uint64_t row = (uint64_t)blockIdx.x * (kSplitWaves / RW) + wave / RW;
+  const bool row_ok = row < rows;
+  if (!row_ok) row = rows - 1;
+  const uint32_t base = (uint32_t)(wave % RW) * (NV * 64) + lane;
+  const uint4 *src = reinterpret_cast<const uint4 *>(in) + row * nvec;
+  uint4 *dst = reinterpret_cast<uint4 *>(out) + row * nvec;
+
+  uint4 raw[NV];
+  bool ok[NV];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const uint32_t v = base + 64u * i;
+    ok[i] = FULL || v < nvec;
+    raw[i] = load_stream(src + (ok[i] ? v : nvec - 1));  // never a load under a branch
+  }
+  float x[NV][EPV];
+  float m = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    Elem<T>::unpack(raw[i], x[i]);
+#pragma unroll
+    for (int k = 0; k < EPV; ++k) {
+      if (!FULL) x[i][k] = ok[i] ? x[i][k] : -INFINITY;
+      m = fmaxf(m, x[i][k]);
+    }
+  }
+  m = wave_max(m);
+  if (lane == 0) red[0][wave] = m;
+  __syncthreads();
+#pragma unroll
+  for (int r = 0; r < RW; ++r) m = fmaxf(m, red[0][first + r]);
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i)
+#pragma unroll
+    for (int k = 0; k < EPV; ++k) {
+      x[i][k] = fast_exp(x[i][k] - m);  // exp(-inf) = 0 for the padding
+      s += x[i][k];
+    }
+  s = wave_sum(s);
+  if (lane == 0) red[1][wave] = s;
+  __syncthreads();
+  s = 0.f;
+#pragma unroll
+  for (int r = 0; r < RW; ++r) s += red[1][first + r];
+  const float inv = 1.0f / s;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+#pragma unroll
+    for (int k = 0; k < EPV; ++k) x[i][k] *= inv;
+    if (row_ok && ok[i]) store_stream(dst + base + 64u * i, Elem<T>::pack(x[i]));
   }
 }
 
@@ -486,9 +597,19 @@ hipError_t run(const T *in, T *out, uint64_t rows, uint64_t cols, hipStream_t st
     const uint32_t nv = (uint32_t)nvec;
     if (nvec <= 64) softmax_wave_kernel<T, 1><<<grid, block, 0, stream>>>(in, out, rows, nv);
     else if (nvec <= 128) softmax_wave_kernel<T, 2><<<grid, block, 0, stream>>>(in, out, rows, nv);
-    else if (nvec <= 256) softmax_wave_kernel<T, 4><<<grid, block, 0, stream>>>(in, out, rows, nv);
-    else if (nvec <= 512) softmax_wave_kernel<T, 8><<<grid, block, 0, stream>>>(in, out, rows, nv);
-    else softmax_wave_kernel<T, 16><<<grid, block, 0, stream>>>(in, out, rows, nv);
+    else {
+      // longer rows: RW waves per row, two vectors per lane
+      const int rw = nvec <= 256 ? 2 : nvec <= 512 ? 4 : 8;
+      const bool full = nvec == (uint64_t)rw * 128;
+      const uint64_t rpb = kSplitWaves / rw, sblocks = (rows + rpb - 1) / rpb;
+      if (sblocks > 0x7fffffffull) return hipErrorInvalidValue;
+      const dim3 sgrid((unsigned)sblocks), sblock(kSplitWaves * 64);
+#define SPLIT(RW)                                                                                \
+  if (full) softmax_split_kernel<T, RW, true><<<sgrid, sblock, 0, stream>>>(in, out, rows, nv);  \
+  else softmax_split_kernel<T, RW, false><<<sgrid, sblock, 0, stream>>>(in, out, rows, nv)
+      if (rw == 2) { SPLIT(2); } else if (rw == 4) { SPLIT(4); } else { SPLIT(8); }
+#undef SPLIT
+    }
     return hipGetLastError();
   }
   if (rows > 0x7fffffffull) return hipErrorInvalidValue;
