@@ -133,24 +133,33 @@ __global__ void __launch_bounds__(NW * 64, NW * QB >= 16 ? 2 : (QB == 2 ? 1 : 2)
   const int ld_c = tid % CPR, ld_r = tid / CPR;
   const bool ld_on = RPP <= kBN || ld_r < kBN;     // narrow heads: surplus threads stay idle
   uint4 kreg[NP], vreg[NP];
-  // running pointers to this thread's first chunk of the next tile to fetch
-  const T *kp = kg + (int64_t)(n_min * kBN + ld_r) * p.k_rs + ld_c * 8;
-  const T *vp = vg + (int64_t)(n_min * kBN + ld_r) * p.v_rs + ld_c * 8;
-  const int64_t k_pass = (int64_t)RPP * p.k_rs, v_pass = (int64_t)RPP * p.v_rs;
-  const int64_t k_tile = (int64_t)kBN * p.k_rs, v_tile = (int64_t)kBN * p.v_rs;
-  int ld_kv = n_min * kBN + ld_r;  // key row of pass 0 of the next tile to fetch
+  // Buffer loads: the descriptors cover this head's rows [0, sk), so rows beyond the last key
+  // read as zeros without an address check (0 * finite stays finite in P V).  The tile offset
+  // is added to the per-thread offset (the vector offset is what the hardware checks against
+  // the descriptor's size); launch_fwd keeps head slices below 2 GiB so the sum cannot wrap.
+  typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+  constexpr unsigned kRsrcFlags = 0x00020000;  // raw buffer, 32-bit data format
+  const unsigned k_bytes = sk > 0 ? (unsigned)((((int64_t)sk - 1) * p.k_rs + D) * 2) : 0u;
+  const unsigned v_bytes = sk > 0 ? (unsigned)((((int64_t)sk - 1) * p.v_rs + D) * 2) : 0u;
+  const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(kg), 0, k_bytes, kRsrcFlags);
+  const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(vg), 0, v_bytes, kRsrcFlags);
+  unsigned k_vo[NP], v_vo[NP];
+#pragma unroll
+  for (int s = 0; s < NP; ++s) {  // surplus threads of a narrow head point beyond the buffer
+    k_vo[s] = ld_on ? (unsigned)(((int64_t)(ld_r + s * RPP) * p.k_rs + ld_c * 8) * 2) : 0xffffffffu;
+    v_vo[s] = ld_on ? (unsigned)(((int64_t)(ld_r + s * RPP) * p.v_rs + ld_c * 8) * 2) : 0xffffffffu;
+  }
+  const unsigned k_tile_b = (unsigned)(kBN * p.k_rs * 2), v_tile_b = (unsigned)(kBN * p.v_rs * 2);
+  unsigned k_so = (unsigned)n_min * k_tile_b, v_so = (unsigned)n_min * v_tile_b;  // byte offset of the next tile to fetch
   auto gload = [&]() {
 #pragma unroll
     for (int s = 0; s < NP; ++s) {
-      if (ld_on && ld_kv + s * RPP < sk) {
-        kreg[s] = *reinterpret_cast<const uint4 *>(kp + s * k_pass);
-        vreg[s] = *reinterpret_cast<const uint4 *>(vp + s * v_pass);
-      } else {  // zero rows: 0 * finite stays finite in P V
-        kreg[s] = uint4{0, 0, 0, 0};
-        vreg[s] = uint4{0, 0, 0, 0};
-      }
+      const u32x4 a = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, ld_on ? k_vo[s] + k_so : 0xffffffffu, 0, 0);
+      const u32x4 b = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, ld_on ? v_vo[s] + v_so : 0xffffffffu, 0, 0);
+      kreg[s] = uint4{a.x, a.y, a.z, a.w};
+      vreg[s] = uint4{b.x, b.y, b.z, b.w};
     }
-    kp += k_tile; vp += v_tile; ld_kv += kBN;
+    k_so += k_tile_b; v_so += v_tile_b;
   };
   const int st_off_k = ld_r * KS + ld_c * 8, st_off_v = ld_r * VS + ld_c * 8;
   auto lstore = [&](int buf) {
@@ -287,10 +296,28 @@ __global__ void __launch_bounds__(NW * 64, NW * QB >= 16 ? 2 : (QB == 2 ? 1 : 2)
   const int n_tiles = n_max > n_min ? n_max - n_min : 0;
   Unit ua, ub;  // S^T of the unit being consumed / being produced
   if (n_tiles > 0) {
+    // All three tiles are requested before the first is stored: one memory latency, not
+    // three.  (Tiles beyond the last one read rows that are in bounds or zeros, and stay unused.)
+    uint4 k1[NP], v1[NP], k2[NP], v2[NP];
     gload();
+#pragma unroll
+    for (int s = 0; s < NP; ++s) { k1[s] = kreg[s]; v1[s] = vreg[s]; }
+    gload();
+#pragma unroll
+    for (int s = 0; s < NP; ++s) { k2[s] = kreg[s]; v2[s] = vreg[s]; }
+    gload();
+#pragma unroll
+    for (int s = 0; s < NP; ++s) {  // kreg / vreg: tile n_min + 2, as the loop expects; k1: n_min, k2: n_min + 1
+      const uint4 a = kreg[s], b = vreg[s];
+      kreg[s] = k1[s]; vreg[s] = v1[s];
+      k1[s] = a; v1[s] = b;
+    }
     lstore(0);
-    if (n_tiles > 1) { gload(); lstore(1); }
-    if (n_tiles > 2) gload();
+#pragma unroll
+    for (int s = 0; s < NP; ++s) { kreg[s] = k2[s]; vreg[s] = v2[s]; }
+    lstore(1);
+#pragma unroll
+    for (int s = 0; s < NP; ++s) { kreg[s] = k1[s]; vreg[s] = v1[s]; }
     __syncthreads();
     if (!skipped(n_min * kBN)) qk(Ks[0], 0, ua);
   }
@@ -492,7 +519,9 @@ hipError_t launch_fwd(Params &p, int dtype, hipStream_t stream) {
   p.xcd_remap = ((p.b * p.h) % 8 == 0) ? (p.wr >= 0 ? 2 : 1) : (p.wr >= 0 ? 3 : 0);
   if (p.b * p.h == 0 || p.sq == 0) return hipSuccess;
   if (decode_eligible(p)) return launch_decode(p, dtype, stream);
-  if (p.drop || (p.d != 32 && p.d != 64 && p.d != 128)) return launch_fwd_anyd(p, dtype, stream);
+  // the tuned kernel addresses a head's K and V rows through 32-bit buffer offsets
+  const int64_t kv_span = 2 * ((int64_t)p.sk * std::max(p.k_rs, p.v_rs) + 256);
+  if (p.drop || (p.d != 32 && p.d != 64 && p.d != 128) || kv_span >= (int64_t(1) << 31)) return launch_fwd_anyd(p, dtype, stream);
   return dtype == 1 ? launch_fwd_t<_Float16>(p, stream) : launch_fwd_t<__bf16>(p, stream);
 }
 
