@@ -1,38 +1,51 @@
 #!/usr/bin/env python3
 """Benchmark of the op-kernel hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2] [--no-extras] [--pmc-probe]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2] [--no-extras] [--no-cpu] [--pmc-probe]
 
-Prints ONE JSON line.  The headline workload (`config.workload`) is the second of the benchmark configurations the repository's BASELINE.json lists:
-ReduceMaxOp_f32_f32 and ReduceSumOp_f32_f32 over axis 0 (column / two-pass split case) and over
-axis 1 of one [16384, 8192] float tensor; a "step" is those four op-kernel launches, `value` is
-the algorithmic bytes of a step divided by the step time, inputs resident in HBM.  The other
-listed configurations (row sum, fused softmax, flash-attention forward and backward) are
-timed in the same run and reported under `all_configs`, each with its own roofline fraction and
-a CPU figure.
+Prints ONE JSON line.  The headline workload (`config.workload`) is the second of the benchmark
+configurations the repository's BASELINE.json lists: ReduceMaxOp_f32_f32 and ReduceSumOp_f32_f32
+over axis 0 (column / two-pass split case) and over axis 1 of one [16384, 8192] float tensor; a
+"step" is those four op-kernel launches, `value` is the algorithmic bytes of a step divided by the
+step time, inputs resident in HBM.  The other listed configurations (row sum, fused softmax,
+flash-attention forward and backward) are timed in the same run and reported under `all_configs`,
+each with its own roofline fraction, the shader clock sampled while it ran, and CPU figures on
+one core and on all cores of this job's share.
+
+Inputs come from the library's counter-based generator (brt_rocm_fill: element i is a function
+of (seed, i) only), with one seed per tensor; the CPU side regenerates the same bits with
+oracle.fill instead of reading buffers back.  Every configuration passes a parity gate against the
+CPU oracle before it is timed; a failed gate ends the run.
 
 Timing: HIP events recorded on the stream the kernels are launched on (through the library's
 own C ABI, not torch's event wrapper), plus a host clock around the synchronised region.
-Everything is launched through the C ABI (libbrt_rocm_kernels.so / libflash_attn.so); torch is
-used for device memory, streams and random input only.
+`value` and every `us_per_op` come from ONE pair of events around all timed steps; `median_*`
+from a second pass with an event pair per step.  Everything is launched through the C ABI
+(libbrt_rocm_kernels.so / libflash_attn.so); torch is used for device memory and streams only.
 """
 import argparse
 import ctypes
+import glob
 import json
 import os
+import re
+import statistics
 import sys
+import threading
 import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E, published
-MFMA_PEAK_TFLOPS = 2500.0  # dense bf16 / fp16 MFMA, published
-
-# measured HBM bytes of one first-pass launch: 536 894 846 fetched + 4 194 304 written
-TRAFFIC_COL_FIRST_PASS = 541089150
+MFMA_PEAK_TFLOPS = 2500.0  # dense bf16 / fp16 MFMA, published (256 CUs x 4 SIMDs x 1024 FLOP/clk x 2.4 GHz)
+PEAK_CLOCK_MHZ = 2400.0
 
 METRIC = "reduce HBM GB/s + flash-attn fwd/bwd TFLOP/s, % of MI355X roofline, 1 GPU"
+
+# seeds of the synthetic tensors: one per tensor; rotating copies add their index << 32
+SEED = {"c1": 0xC1, "c2": 0xC2, "c3": 0xC3, "c4q": 0xC41, "c4k": 0xC42, "c4v": 0xC43,
+        "c5q": 0xC51, "c5k": 0xC52, "c5v": 0xC53, "c5do": 0xC54, "dec": 0xDC}
 
 
 class Events:
@@ -60,30 +73,78 @@ class Events:
             self.K.brt_rocm_event_destroy(e)
 
 
-def time_ops(ev, fns, steps, warmup):
+class ClockSampler:
+    """Samples the GPU's current shader clock (the starred level of pp_dpm_sclk) from a thread
+    while a timed region runs: the attention kernels do not hold the 2.4 GHz the published MFMA
+    peak assumes, and how far they fall depends on the data (zeros run faster than random
+    numbers), so a TFLOP/s figure is only comparable together with the clock it ran at."""
+
+    def __init__(self):
+        files = sorted(glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk"))
+        self.path = files[0] if files else None
+        self.samples, self._stop, self._t = [], None, None
+
+    def read(self):
+        if not self.path:
+            return None
+        try:
+            for line in open(self.path).read().splitlines():
+                if "*" in line:
+                    m = re.search(r"(\d+)\s*[Mm][Hh]z", line)
+                    return float(m.group(1)) if m else None
+        except OSError:
+            return None
+        return None
+
+    def __enter__(self):
+        self.samples, self._stop = [], threading.Event()
+
+        def run():
+            while not self._stop.is_set():
+                v = self.read()
+                if v:
+                    self.samples.append(v)
+                time.sleep(0.002)
+
+        self._t = threading.Thread(target=run, daemon=True)
+        self._t.start()
+        return self
+
+    def __exit__(self, *a):
+        self._stop.set()
+        self._t.join()
+
+    def summary(self):
+        s = [v for v in self.samples if v > 400]  # drop the idle level seen before the first launch lands
+        if not s:
+            return None
+        return {"mean_mhz": round(sum(s) / len(s), 0), "min_mhz": min(s), "max_mhz": max(s), "samples": len(s)}
+
+
+def time_ops(ev, fns, steps, warmup, clocks=None):
     """Run `fns` (a list of launch closures = one step) `warmup` + `steps` times.
-    -> (ms per step by events, [ms per launch of fns[i]], ms per step by host clock).
-    The step time comes from ONE pair of events around all `steps` steps (an event between every
-    two launches costs a few microseconds of idle GPU each); the per-launch breakdown is taken
-    in a second pass of the same length with an event after every launch."""
+    -> dict(ms: ms per step from one event pair around all steps, per: [ms per launch of fns[i]],
+    host_ms, median_ms: median over per-step event pairs of a second pass, clock: sampled MHz)."""
     import torch
     for _ in range(warmup):
         for f in fns:
             f()
     torch.cuda.synchronize()
     e0, e1 = ev.new(), ev.new()
-    t0 = time.perf_counter()
-    ev.record(e0)
-    for _ in range(steps):
-        for f in fns:
-            f()
-    ev.record(e1)
-    torch.cuda.synchronize()
-    host_ms = (time.perf_counter() - t0) * 1e3 / steps
+    sampler = clocks if clocks is not None else ClockSampler()
+    with sampler:
+        t0 = time.perf_counter()
+        ev.record(e0)
+        for _ in range(steps):
+            for f in fns:
+                f()
+        ev.record(e1)
+        torch.cuda.synchronize()
+        host_ms = (time.perf_counter() - t0) * 1e3 / steps
     total = ev.elapsed_ms(e0, e1) / steps
     ev.free([e0, e1])
-    if len(fns) == 1:
-        return total, [total], host_ms
+    # second pass: an event after every launch (each costs a few microseconds of idle GPU, so
+    # this pass feeds the per-launch breakdown and the median only)
     marks = [[ev.new() for _ in range(len(fns) + 1)] for _ in range(steps)]
     for s in range(steps):
         ev.record(marks[s][0])
@@ -91,17 +152,18 @@ def time_ops(ev, fns, steps, warmup):
             f()
             ev.record(marks[s][i + 1])
     torch.cuda.synchronize()
-    per = [sum(ev.elapsed_ms(marks[s][i], marks[s][i + 1]) for s in range(steps)) / steps
-           for i in range(len(fns))]
+    per = [sum(ev.elapsed_ms(marks[s][i], marks[s][i + 1]) for s in range(steps)) / steps for i in range(len(fns))]
+    med = statistics.median(ev.elapsed_ms(marks[s][0], marks[s][-1]) for s in range(steps))
     for m in marks:
         ev.free(m)
-    return total, per, host_ms
+    return {"ms": total, "per": per, "host_ms": host_ms, "median_ms": med, "clock": sampler.summary()}
 
 
-def prewarm(fn, seconds=0.08):
-    """Run `fn` back to back for about `seconds` of wall time.  After idle time (or after
-    memory-bound kernels) the matrix-heavy attention kernels run 15-20 % slower for their first
-    ~100 launches (~30 ms) while the clocks ramp; the timed region should see the steady state."""
+def prewarm(fn, seconds=0.5):
+    """Run `fn` back to back for about `seconds` of wall time.  After idle time (the parity gate's
+    CPU work) or after memory-bound kernels the matrix-heavy attention kernels run 10-20 % slower
+    for some tenths of a second while the clocks settle; the timed region should see the steady
+    state."""
     import torch
     t0 = time.perf_counter()
     while time.perf_counter() - t0 < seconds:
@@ -117,6 +179,50 @@ def cpu_time(fn, repeat=2):
         fn()
         best = min(best, time.perf_counter() - t)
     return best
+
+
+def cpu_both(oracle, fn, n_thr, repeat=2):
+    """Best-of-`repeat` seconds of `fn` on one core and with OpenMP on `n_thr` threads."""
+    oracle.set_threads(1)
+    t1 = cpu_time(fn, repeat)
+    oracle.set_threads(n_thr)
+    tn = cpu_time(fn, repeat)
+    oracle.set_threads(1)
+    return t1, tn
+
+
+def gate(ok, what):
+    if not ok:
+        sys.exit(f"bench.py: parity gate failed before timing: {what}")
+
+
+def measured_traffic(K, _lib, R, Cc):
+    """HBM bytes of one first-pass launch of the axis-0 fold, from the tracked counter profile
+    (FETCH_SIZE and WRITE_SIZE per dispatch, each scaled by the same counter's reading for a copy
+    kernel of known size).  The profile is only valid for the split it was measured with: the
+    workspace size it records must equal what the library plans today."""
+    path = os.path.join(ROOT, "profiles", "reduce_c2_hbm_traffic.txt")
+    if not os.path.exists(path):
+        return None, "profiles/reduce_c2_hbm_traffic.txt not present"
+    text = open(path).read()
+    vals = {"FETCH_SIZE": [], "WRITE_SIZE": []}
+    section = None
+    for line in text.splitlines():
+        for k in vals:
+            if line.startswith(k + ":"):
+                section = k
+        m = re.search(r"reduce_colwide_kernel<float, float, [01],.*scaled_bytes=\s*(\d+)", line)
+        if m and section:
+            vals[section].append(int(m.group(1)))
+    if not vals["FETCH_SIZE"] or not vals["WRITE_SIZE"]:
+        return None, "no reduce_colwide_kernel rows in the profile"
+    ws_now = K.brt_rocm_reduce_workspace_bytes(_lib.F32, 1, R, Cc)
+    ws_then = sum(vals["WRITE_SIZE"]) // len(vals["WRITE_SIZE"])  # the first pass writes exactly its partials
+    if ws_now != ws_then:
+        sys.exit(f"bench.py: the axis-0 split has changed (partials {ws_now} B now, {ws_then} B when "
+                 "profiles/reduce_c2_hbm_traffic.txt was measured): re-measure the traffic profile")
+    fetch = sum(vals["FETCH_SIZE"]) / len(vals["FETCH_SIZE"])
+    return int(round(fetch + ws_then)), "profiles/reduce_c2_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, copy-kernel scaled)"
 
 
 def main():
@@ -145,13 +251,12 @@ def main():
     stream = torch.cuda.current_stream()
     sp = ctypes.c_void_p(stream.cuda_stream)
     ev = Events(K, sp)
-    gen = torch.Generator(device="cuda")
+    import oracle  # the checker: parity gates and the cpu_baseline legs only
 
     # ---- headline: C2, [16384, 8192] f32 ~ U(-1, 1) --------------------------------------
     R, Cc = 16384, 8192
     NBUF = 3  # rotate inputs: 1.5 GiB between two touches of a buffer, beyond the 256 MB LLC
-    gen.manual_seed(0xC2)
-    xs = [torch.rand((R, Cc), generator=gen, device="cuda") * 2 - 1 for _ in range(NBUF)]
+    xs = [ops.fill(torch.empty((R, Cc), device="cuda"), _lib.FILL_UNIFORM, SEED["c2"] + (i << 32), -1.0, 1.0) for i in range(NBUF)]
     out_col = torch.empty(Cc, device="cuda")
     out_row = torch.empty(R, device="cuda")
     ws_col = torch.empty(max(1, ops.reduce_workspace_bytes(torch.float32, 1, R, Cc)), dtype=torch.uint8, device="cuda")
@@ -184,9 +289,8 @@ def main():
         # heads on 8 key/value heads of 128, fp16): 2 GiB of cache rows per call
         del dst
         b_, h_, hk_, sk_, d_ = 64, 32, 8, 8192, 128
-        qd = torch.randn((b_, 1, h_, d_), generator=gen, device="cuda").half()
-        kc, vc = (torch.randn((b_, sk_, hk_, d_), generator=gen, device="cuda").half() for _ in range(2))
-        kn, vn = (torch.randn((b_, 1, hk_, d_), generator=gen, device="cuda").half() for _ in range(2))
+        mk = lambda shape, j: ops.fill(torch.empty(shape, dtype=torch.float16, device="cuda"), _lib.FILL_NORMAL, SEED["dec"] + (j << 32), 0.0, 1.0)
+        qd, kc, vc, kn, vn = mk((b_, 1, h_, d_), 0), mk((b_, sk_, hk_, d_), 1), mk((b_, sk_, hk_, d_), 2), mk((b_, 1, hk_, d_), 3), mk((b_, 1, hk_, d_), 4)
         lens = torch.full((b_,), sk_ - 1, dtype=torch.int32, device="cuda")
         for _ in range(2):
             ops.flash_attn_kvcache(qd, kc, vc, kn, vn, lens, 1.0 / np.sqrt(d_), (-1, -1))
@@ -195,7 +299,23 @@ def main():
                           "decode_cache_bytes": 2 * b_ * sk_ * hk_ * d_ * 2}))
         return
 
-    ms_step, per, host_ms = time_ops(ev, c2_fns, args.steps, args.warmup)
+    # parity gate (and the CPU baseline's input): the host regenerates buffer 0 from its seed
+    n_thr = max(1, min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16"))))
+    xh = oracle.fill(0, oracle.UNIFORM, SEED["c2"], R * Cc, -1.0, 1.0).reshape(R, Cc)
+    gate(np.array_equal(xs[0][:64].cpu().numpy(), xh[:64]) and np.array_equal(xs[0][-1].cpu().numpy(), xh[-1]),
+         "GPU fill and host fill disagree")
+    oracle.set_threads(n_thr)
+    for dims, (A, B, C), o in (((0,), (1, R, Cc), out_col), ((1,), (R, Cc, 1), out_row)):
+        ops.reduce_abc(_lib.REDUCE_MAX, xs[0], o, A, B, C, workspace=ws_col if C > 1 else ws_row)
+        gate(np.array_equal(o.cpu().numpy(), oracle.reduce_abc(oracle.MAX, xh, A, B, C)), f"c2 ReduceMax dims={dims}")
+        ops.reduce_abc(_lib.REDUCE_SUM, xs[0], o, A, B, C, workspace=ws_col if C > 1 else ws_row)
+        s64, sabs = oracle.reduce_sum_f64(xh, A, B, C)
+        gate(np.all(np.abs(o.cpu().numpy().astype(np.float64) - s64) <= 1e-5 * np.maximum(np.abs(s64), 1e-2 * sabs)),
+             f"c2 ReduceSum dims={dims} (1e-5 relative against the float64 fold)")
+    oracle.set_threads(1)
+
+    r2 = time_ops(ev, c2_fns, args.steps, args.warmup)
+    ms_step, per, host_ms = r2["ms"], r2["per"], r2["host_ms"]
     value = step_bytes / (ms_step * 1e-3) / 1e9
     col_ms = (per[0] + per[1]) / 2
     row_ms = (per[2] + per[3]) / 2
@@ -216,29 +336,47 @@ def main():
     for t in triples:
         ev.free(t)
     col_gbs = bytes_col / (pass1_ms * 1e-3) / 1e9
+    traffic, traffic_src = measured_traffic(K, _lib, R, Cc)
     roofline = {
         "bound": "hbm", "kernel": "reduce_colwide_kernel<float, float, OP, 4, 2, 2> (first pass of the axis-0 split reduction)",
         "achieved": round(col_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": round(col_gbs / HBM_PEAK_GBS, 4),
         "algorithmic_bytes_per_launch": bytes_col, "avg_launch_us": round(pass1_ms * 1e3, 2),
         "op_us_including_combine_pass": round(col_ms * 1e3, 2), "combine_pass_us": round(p2_ms * 1e3, 2),
-        # FETCH_SIZE + WRITE_SIZE per first-pass dispatch from two rocprofv3 --pmc runs, each
-        # scaled by the same counter's reading for a 512 MiB copy kernel (profiles/)
-        "traffic": TRAFFIC_COL_FIRST_PASS,
+        "traffic": traffic, "traffic_source": traffic_src,
     }
     col_op_gbs = bytes_col / (col_ms * 1e-3) / 1e9
 
+    props = torch.cuda.get_device_properties(0)
+    max_sclk = None
+    try:
+        levels = [float(m) for m in re.findall(r"(\d+)\s*[Mm][Hh]z", open(ClockSampler().path).read())]
+        max_sclk = max(levels) if levels else None
+    except (OSError, TypeError):
+        pass
     result = {
         "metric": METRIC, "value": round(value, 1), "unit": "GB/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_step, 4),
+        "median_ms_per_step": round(r2["median_ms"], 4),
         "host_ms_per_step": round(host_ms, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": "c2: ReduceMaxOp_f32_f32 + ReduceSumOp_f32_f32 over axis 0 and over axis 1 "
                                "of [16384, 8192] f32 ~ U(-1,1) (4 op-kernel launches per step, "
                                f"{NBUF} rotating input buffers)",
-                   "algorithmic_bytes_per_step": step_bytes},
+                   "algorithmic_bytes_per_step": step_bytes,
+                   "generator": "brt_rocm_fill / oracle_fill: splitmix64 counter stream per tensor (uniform: 24 bits; "
+                                "normal: sum of twelve 16-bit fields), seeds " + json.dumps({k: hex(v) for k, v in SEED.items()})},
         "roofline": roofline,
+        "device": {"name": props.name, "compute_units": props.multi_processor_count,
+                   "max_shader_clock_mhz": max_sclk, "hbm_bytes": props.total_memory,
+                   "memory_clock_mhz": (getattr(props, "memory_clock_rate", 0) or 0) / 1e3 or None,
+                   "memory_bus_bits": getattr(props, "memory_bus_width", None),
+                   "published_peaks": {"hbm_GBs": HBM_PEAK_GBS, "mfma_f16_bf16_dense_TFLOPs": MFMA_PEAK_TFLOPS,
+                                       "at_shader_clock_mhz": PEAK_CLOCK_MHZ},
+                   # compute units x 4 SIMDs x 1024 FLOP per clock (one 32x32x16 MFMA per 32 clocks) x the top clock level
+                   "mfma_peak_from_device_TFLOPs": round(props.multi_processor_count * 4 * 1024 * max_sclk * 1e6 / 1e12, 1) if max_sclk else None,
+                   "shader_clock_during_c2": r2["clock"]},
     }
 
     all_cfg = {
@@ -252,56 +390,68 @@ def main():
 
     # ---- CPU baseline for the headline workload --------------------------------------------
     if not args.no_cpu:
-        import oracle
-        oracle.set_threads(1)
-        xh = xs[0].cpu().numpy()
-        t_cpu = cpu_time(lambda: (oracle.reduce_abc(oracle.MAX, xh, 1, R, Cc), oracle.reduce_abc(oracle.SUM, xh, 1, R, Cc),
-                                  oracle.reduce_abc(oracle.MAX, xh, R, Cc, 1), oracle.reduce_abc(oracle.SUM, xh, R, Cc, 1)),
-                         repeat=2)
+        step = lambda: (oracle.reduce_abc(oracle.MAX, xh, 1, R, Cc), oracle.reduce_abc(oracle.SUM, xh, 1, R, Cc),
+                        oracle.reduce_abc(oracle.MAX, xh, R, Cc, 1), oracle.reduce_abc(oracle.SUM, xh, R, Cc, 1))
+        t_cpu, t_par = cpu_both(oracle, step, n_thr)
         result["cpu_baseline"] = {
             "value": round(step_bytes / t_cpu / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
             "sample": "the full step (4 reductions of the [16384, 8192] tensor) run once per repeat, best of 2, "
                       "by the scalar loop-nest oracle (the reference's CPU path is single-threaded LLVM-JIT'ed "
                       "loop nests, which cannot be built here)",
             "seconds": round(t_cpu, 3), "host_cores_available": os.cpu_count(),
+            # the same loop nests with OpenMP over the independent outputs, on this job's CPU share
+            "openmp": {"value": round(step_bytes / t_par / 1e9, 3), "unit": "GB/s", "cores": n_thr, "seconds": round(t_par, 3)},
         }
-        # the same loop nests with OpenMP over the independent outputs, on this job's CPU share
-        n_thr = max(1, min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16"))))
-        oracle.set_threads(n_thr)
-        t_par = cpu_time(lambda: (oracle.reduce_abc(oracle.MAX, xh, 1, R, Cc), oracle.reduce_abc(oracle.SUM, xh, 1, R, Cc),
-                                  oracle.reduce_abc(oracle.MAX, xh, R, Cc, 1), oracle.reduce_abc(oracle.SUM, xh, R, Cc, 1)),
-                         repeat=2)
-        oracle.set_threads(1)
-        result["cpu_baseline"]["openmp"] = {"value": round(step_bytes / t_par / 1e9, 3), "unit": "GB/s", "cores": n_thr,
-                                            "seconds": round(t_par, 3)}
-        del xh
+        for key, (A, B, C), byt in (("c2a_col_max_sum_axis0", (1, R, Cc), bytes_col), ("c2b_row_max_sum_axis1", (R, Cc, 1), bytes_row)):
+            t1, tn = cpu_both(oracle, lambda: (oracle.reduce_abc(oracle.MAX, xh, A, B, C), oracle.reduce_abc(oracle.SUM, xh, A, B, C)), n_thr, 1)
+            all_cfg[key]["cpu_1core_GBs"] = round(2 * byt / t1 / 1e9, 3)
+            all_cfg[key]["cpu_allcore_GBs"] = round(2 * byt / tn / 1e9, 3)
+            all_cfg[key]["cpu_cores"] = n_thr
+    del xh
 
     if not args.no_extras:
-        extras(all_cfg, ev, ops, _lib, gen, args, np, torch)
+        extras(all_cfg, ev, ops, _lib, oracle, args, np, torch, n_thr)
     result["all_configs"] = all_cfg
     print(json.dumps(result))
 
 
-def extras(all_cfg, ev, ops, _lib, gen, args, np, torch):
-    """The remaining benchmark configurations, timed with the same event machinery."""
-    import oracle
+def with_clock(entry, r, peak, key):
+    """Adds the sampled shader clock and the fraction of the peak scaled to that clock."""
+    c = r["clock"]
+    entry["median_us_per_op"] = round(r["median_ms"] * 1e3 / r.get("ops_per_step", 1), 2)
+    if c:
+        entry["shader_clock_mhz"] = c
+        entry[key + "_at_sampled_clock"] = round(entry["value"] / (peak * c["mean_mhz"] / PEAK_CLOCK_MHZ), 4)
+    return entry
+
+
+def extras(all_cfg, ev, ops, _lib, oracle, args, np, torch, n_thr):
+    """The remaining benchmark configurations: parity gate, timing, CPU figures."""
     steps, warm = max(5, args.steps // 2), max(2, args.warmup // 2)
     do_cpu = not args.no_cpu
+    F, H, B16 = torch.float32, torch.float16, torch.bfloat16
+
+    def mk(shape, dtype, dist, seed, a, b):
+        return ops.fill(torch.empty(shape, dtype=dtype, device="cuda"), dist, seed, a, b)
 
     # c1: row ReduceSum f32 [4096, 1024] ~ N(0,1).  16 MiB: launch-bound; rotating 40 buffers
     # (640 MiB) keeps the input out of the 256 MB LLC ("cold"), one buffer gives the warm figure.
-    gen.manual_seed(0xC1)
-    bufs = [torch.randn((4096, 1024), generator=gen, device="cuda") for _ in range(40)]
+    bufs = [mk((4096, 1024), F, _lib.FILL_NORMAL, SEED["c1"] + (i << 32), 0.0, 1.0) for i in range(40)]
     o1 = torch.empty(4096, device="cuda")
     b1 = 4096 * 1024 * 4 + 4096 * 4
+    xh = oracle.fill(0, oracle.NORMAL, SEED["c1"], 4096 * 1024, 0.0, 1.0).reshape(4096, 1024)
+    ops.reduce_abc(_lib.REDUCE_SUM, bufs[0], o1, 4096, 1024, 1)
+    s64, sabs = oracle.reduce_sum_f64(xh, 4096, 1024, 1)
+    gate(np.all(np.abs(o1.cpu().numpy().astype(np.float64) - s64) <= 1e-5 * np.maximum(np.abs(s64), 1e-2 * sabs)), "c1 row ReduceSum")
     i = [0]
 
     def c1_cold():
         i[0] = (i[0] + 1) % len(bufs)
         ops.reduce_abc(_lib.REDUCE_SUM, bufs[i[0]], o1, 4096, 1024, 1)
 
-    ms_cold, _, _ = time_ops(ev, [c1_cold] * 10, steps, warm)
-    ms_warm, _, _ = time_ops(ev, [lambda: ops.reduce_abc(_lib.REDUCE_SUM, bufs[0], o1, 4096, 1024, 1)] * 10, steps, warm)
+    rc = time_ops(ev, [c1_cold] * 10, steps, warm)
+    rw = time_ops(ev, [lambda: ops.reduce_abc(_lib.REDUCE_SUM, bufs[0], o1, 4096, 1024, 1)] * 10, steps, warm)
+    ms_cold, ms_warm = rc["ms"], rw["ms"]
     # the same 40 cold launches captured once in a HIP graph: launch cost leaves the host
     side = torch.cuda.Stream()
     graph = torch.cuda.CUDAGraph()
@@ -313,103 +463,162 @@ def extras(all_cfg, ev, ops, _lib, gen, args, np, torch):
             for b in bufs:
                 ops.reduce_abc(_lib.REDUCE_SUM, b, o1, 4096, 1024, 1, stream=torch.cuda.current_stream())
     torch.cuda.synchronize()
-    ms_graph, _, _ = time_ops(ev, [graph.replay], steps, warm)
+    ms_graph = time_ops(ev, [graph.replay], steps, warm)["ms"]
     c1 = {"value": round(b1 / (ms_cold / 10 * 1e-3) / 1e9, 1), "unit": "GB/s", "us_per_op": round(ms_cold / 10 * 1e3, 2),
           "frac_of_hbm_peak": round(b1 / (ms_cold / 10 * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+          "median_us_per_op": round(rc["median_ms"] / 10 * 1e3, 2),
           "warm_cache_GBs": round(b1 / (ms_warm / 10 * 1e-3) / 1e9, 1), "warm_us_per_op": round(ms_warm / 10 * 1e3, 2),
           "graph_replay_GBs": round(b1 / (ms_graph / len(bufs) * 1e-3) / 1e9, 1),
           "graph_replay_us_per_op": round(ms_graph / len(bufs) * 1e3, 2),
           "note": "16 MiB per launch: bound by launch latency, not by HBM; value = back-to-back launches from the "
                   "host over 40 rotating buffers, graph_replay = the same 40 launches replayed from one HIP graph"}
     if do_cpu:
-        xh = bufs[0].cpu().numpy()
-        t = cpu_time(lambda: oracle.reduce_abc(oracle.SUM, xh, 4096, 1024, 1), 3)
-        c1["cpu_1core_GBs"] = round(b1 / t / 1e9, 3)
+        t1, tn = cpu_both(oracle, lambda: oracle.reduce_abc(oracle.SUM, xh, 4096, 1024, 1), n_thr, 3)
+        c1.update(cpu_1core_GBs=round(b1 / t1 / 1e9, 3), cpu_allcore_GBs=round(b1 / tn / 1e9, 3), cpu_cores=n_thr)
     all_cfg["c1_row_sum"] = c1
-    del bufs
+    del bufs, xh
 
     # c3: fused softmax bf16 [32768, 4096] ~ N(0, 4)
-    gen.manual_seed(0xC3)
-    xs = [(torch.randn((32768, 4096), generator=gen, device="cuda") * 2).bfloat16() for _ in range(3)]
+    xs = [mk((32768, 4096), B16, _lib.FILL_NORMAL, SEED["c3"] + (i << 32), 0.0, 2.0) for i in range(3)]
     ys = torch.empty_like(xs[0])
     b3 = 2 * 32768 * 4096 * 2
+    rows = 1024  # the oracle's share: 1024 of the 32768 rows (gate and CPU sample)
+    xh = oracle.fill(2, oracle.NORMAL, SEED["c3"], rows * 4096, 0.0, 2.0).reshape(rows, 4096)
+    ops.softmax(xs[0], out=ys)
+    got = oracle.from_bf16_bits(ys[:rows].view(torch.int16).cpu().numpy().view(np.uint16))
+    want = oracle.from_bf16_bits(oracle.softmax(xh))
+    gate(np.all(np.abs(got - want) <= 2.0 ** -7 * np.abs(want) + 1e-38), "c3 softmax (1 bf16 ulp against the float oracle)")
     j = [0]
 
     def c3():
         j[0] = (j[0] + 1) % 3
         ops.softmax(xs[j[0]], out=ys)
 
-    ms3, _, _ = time_ops(ev, [c3], steps, warm)
+    r3 = time_ops(ev, [c3], steps, warm)
+    ms3 = r3["ms"]
     c3r = {"value": round(b3 / (ms3 * 1e-3) / 1e9, 1), "unit": "GB/s", "us_per_op": round(ms3 * 1e3, 2),
-           "frac_of_hbm_peak": round(b3 / (ms3 * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+           "frac_of_hbm_peak": round(b3 / (ms3 * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+           "median_us_per_op": round(r3["median_ms"] * 1e3, 2),
+           "frac_of_copy_kernel_ceiling": round(b3 / (ms3 * 1e-3) / 1e9 / 6450.0, 4),
+           "note": "a plain copy of the same tensor (one 128-bit load and store per lane, non-temporal) tops out at "
+                   "6.43-6.50 TB/s on this part: equal parts of reads and writes do not reach the 7.0 TB/s of a pure read stream"}
     if do_cpu:
-        rows = 1024  # bounded sample: 1024 of the 32768 rows, scaled
-        xh = xs[0][:rows].view(torch.int16).cpu().numpy().view(np.uint16)
-        t = cpu_time(lambda: oracle.softmax(xh), 2)
-        c3r["cpu_1core_GBs"] = round(2 * rows * 4096 * 2 / t / 1e9, 3)
-        c3r["cpu_sample"] = "1024 rows"
+        t1, tn = cpu_both(oracle, lambda: oracle.softmax(xh), n_thr)
+        c3r.update(cpu_1core_GBs=round(2 * rows * 4096 * 2 / t1 / 1e9, 3), cpu_allcore_GBs=round(2 * rows * 4096 * 2 / tn / 1e9, 3),
+                   cpu_cores=n_thr, cpu_sample="1024 rows")
     all_cfg["c3_softmax_bf16"] = c3r
-    del xs, ys
+    del xs, ys, xh
+
+    def head_slice(code, seed, b, s, h, d, rows=None):
+        """Host copy of batch 0, head 0 of a [b, s, h, d] tensor (storage bits), rows = slice."""
+        t = oracle.fill(code, oracle.NORMAL, seed, s * h * d, 0.0, 1.0).reshape(1, s, h, d)[:, :, :1]
+        t = t.view(np.float16) if code == 1 else t
+        return np.ascontiguousarray(t if rows is None else t[:, rows])
 
     # c4: flash-attention forward fp16 causal b4 h32 s2048 d128
-    gen.manual_seed(0xC4)
-    q, k, v = (torch.randn((4, 2048, 32, 128), generator=gen, device="cuda").half() for _ in range(3))
+    q, k, v = (mk((4, 2048, 32, 128), H, _lib.FILL_NORMAL, SEED[n], 0.0, 1.0) for n in ("c4q", "c4k", "c4v"))
     sc4 = 1.0 / np.sqrt(128.0)
     fl4 = 4 * 4 * 32 * 2048 * 2048 * 128 // 2  # 137 438 953 472
     fwd_out = (torch.empty_like(q), torch.empty((4, 32, 2048), device="cuda"), torch.zeros(2, dtype=torch.int64, device="cuda"))
     c4_fwd = lambda: ops.flash_attn_fwd(q, k, v, sc4, (-1, 0), out=fwd_out)
+    # gate: batch 0, head 0, the last 64 query rows against the float oracle (2e-2 absolute)
+    c4_fwd()
+    qs, ks_, vs_ = (head_slice(1, SEED[n], 4, 2048, 32, 128) for n in ("c4q", "c4k", "c4v"))
+    oracle.set_threads(n_thr)
+    _, lse_ref, o32 = oracle.flash_fwd(qs[:, -64:], ks_, vs_, sc4, (-1, 0), round_p=False)
+    oracle.set_threads(1)
+    gate(np.abs(fwd_out[0][0, -64:, 0].float().cpu().numpy() - o32[0, :, 0]).max() <= 2e-2 and
+         np.abs(fwd_out[1][0, 0, -64:].cpu().numpy() - lse_ref[0, 0]).max() <= 2e-2, "c4 flash forward O / LSE (2e-2 absolute)")
     prewarm(c4_fwd)
-    ms4, _, _ = time_ops(ev, [c4_fwd], steps, warm)
-    c4 = {"value": round(fl4 / (ms4 * 1e-3) / 1e12, 1), "unit": "TFLOP/s", "us_per_op": round(ms4 * 1e3, 1),
-          "frac_of_mfma_peak": round(fl4 / (ms4 * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, 4), "flop": fl4}
+    r4 = time_ops(ev, [c4_fwd], steps, warm)
+    ms4 = r4["ms"]
+    c4 = with_clock({"value": round(fl4 / (ms4 * 1e-3) / 1e12, 1), "unit": "TFLOP/s", "us_per_op": round(ms4 * 1e3, 1),
+                     "frac_of_mfma_peak": round(fl4 / (ms4 * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, 4), "flop": fl4},
+                    r4, MFMA_PEAK_TFLOPS, "frac_of_mfma_peak")
     if do_cpu:
         # the reference has no CPU attention; the naive oracle on one (batch, head) with 256
         # query rows, scaled by the flop ratio
-        qs, ks_, vs_ = (t[:1, :, :1].cpu().numpy() for t in (q, k, v))
-        t = cpu_time(lambda: oracle.flash_fwd(qs[:, -256:], ks_, vs_, sc4, (-1, 0)), 1)
         fl_s = 4 * 256 * (2048 - 128) * 128  # rows 1792..2047 see ~1920 keys on average
-        c4["cpu_1core_TFLOPs"] = round(fl_s / t / 1e12, 6)
-        c4["cpu_sample"] = "1 batch x 1 head x last 256 query rows"
+        t1, tn = cpu_both(oracle, lambda: oracle.flash_fwd(qs[:, -256:], ks_, vs_, sc4, (-1, 0)), n_thr, 1)
+        c4.update(cpu_1core_TFLOPs=round(fl_s / t1 / 1e12, 6), cpu_allcore_TFLOPs=round(fl_s / tn / 1e12, 6), cpu_cores=n_thr,
+                  cpu_sample="naive oracle, 1 batch x 1 head x last 256 query rows, by flop count")
     all_cfg["c4_flash_fwd_fp16_causal"] = c4
-    del q, k, v
+    del q, k, v, qs, ks_, vs_
 
     # c5: flash-attention forward + backward bf16 non-causal b2 h16 s8192 d64
-    gen.manual_seed(0xC5)
-    q, k, v, do = (torch.randn((2, 8192, 16, 64), generator=gen, device="cuda").bfloat16() for _ in range(4))
+    q, k, v, do = (mk((2, 8192, 16, 64), B16, _lib.FILL_NORMAL, SEED[n], 0.0, 1.0) for n in ("c5q", "c5k", "c5v", "c5do"))
     fl5 = 4 * 2 * 16 * 8192 * 8192 * 64  # 549 755 813 888
     fwd_out = (torch.empty_like(q), torch.empty((2, 16, 8192), device="cuda"), torch.zeros(2, dtype=torch.int64, device="cuda"))
     c5_fwd = lambda: ops.flash_attn_fwd(q, k, v, 0.125, (-1, -1), out=fwd_out)
+    c5_fwd()
+    qs, ks_, vs_, dos = (head_slice(2, SEED[n], 2, 8192, 16, 64) for n in ("c5q", "c5k", "c5v", "c5do"))
+    rows5 = slice(4096, 4096 + 32)
+    oracle.set_threads(n_thr)
+    _, lse_ref, o32 = oracle.flash_fwd(qs[:, rows5], ks_, vs_, 0.125, (-1, -1), round_p=False)
+    gate(np.abs(fwd_out[0][0, rows5, 0].float().cpu().numpy() - o32[0, :, 0]).max() <= 2e-2 and
+         np.abs(fwd_out[1][0, 0, rows5].cpu().numpy() - lse_ref[0, 0]).max() <= 2e-2, "c5 flash forward O / LSE (2e-2 absolute)")
     prewarm(c5_fwd)
-    msf, _, _ = time_ops(ev, [c5_fwd], steps, warm)
+    rf = time_ops(ev, [c5_fwd], steps, warm)
+    msf = rf["ms"]
     o, lse = ops.flash_attn_fwd(q, k, v, 0.125, (-1, -1))
     bwd_out = ops.flash_attn_bwd_buffers(q, k, v)
     c5_bwd = lambda: ops.flash_attn_bwd(do, q, k, v, o, lse, 0.125, (-1, -1), out=bwd_out)
+    # gate for the backward kernels: the first 1024 positions of batch 0, head 0 as a problem of
+    # its own (same kernels, same head_dim and dtype; the full-size oracle would take minutes)
+    n5 = 1024
+    tq, tk, tv, tdo = (torch.from_numpy(np.ascontiguousarray(t[:, :n5]).view(np.int16)).cuda().view(torch.bfloat16) for t in (qs, ks_, vs_, dos))
+    to_, tlse = ops.flash_attn_fwd(tq, tk, tv, 0.125, (-1, -1))
+    gq, gk, gv = ops.flash_attn_bwd(tdo, tq, tk, tv, to_, tlse, 0.125, (-1, -1))
+    rq, rk, rv, _ = oracle.flash_bwd(dos[:, :n5], qs[:, :n5], ks_[:, :n5], vs_[:, :n5], to_.view(torch.int16).cpu().numpy().view(np.uint16),
+                                     tlse.cpu().numpy(), 0.125, (-1, -1), round_p=False)
+    oracle.set_threads(1)
+    worst, ok = {}, True
+    for n, g, r in (("dq", gq, rq), ("dk", gk, rk), ("dv", gv, rv)):
+        ref = oracle.to_f32(r)
+        worst[n] = float(np.abs(g.float().cpu().numpy() - ref).max())
+        ok = ok and worst[n] <= 2e-2 + 2.0 ** -8 * float(np.abs(ref).max())  # + 1 bf16 ulp of the largest value stored
+    gate(ok, f"c5 flash backward dq/dk/dv (2e-2 absolute + 1 bf16 ulp of the largest value): {worst}")
     prewarm(c5_bwd)
-    msb, _, _ = time_ops(ev, [c5_bwd], max(3, steps // 3), 2)
-    all_cfg["c5_flash_fwd_bf16"] = {
+    rb = time_ops(ev, [c5_bwd], max(3, steps // 3), 2)
+    msb = rb["ms"]
+    all_cfg["c5_flash_fwd_bf16"] = with_clock({
         "value": round(fl5 / (msf * 1e-3) / 1e12, 1), "unit": "TFLOP/s", "us_per_op": round(msf * 1e3, 1),
-        "frac_of_mfma_peak": round(fl5 / (msf * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, 4), "flop": fl5}
+        "frac_of_mfma_peak": round(fl5 / (msf * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, 4), "flop": fl5}, rf, MFMA_PEAK_TFLOPS, "frac_of_mfma_peak")
     flb = fl5 * 5 // 2
-    all_cfg["c5_flash_bwd_bf16"] = {
+    all_cfg["c5_flash_bwd_bf16"] = with_clock({
         "value": round(flb / (msb * 1e-3) / 1e12, 1), "unit": "TFLOP/s", "us_per_op": round(msb * 1e3, 1),
         "frac_of_mfma_peak": round(flb / (msb * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, 4), "flop": flb,
-        "note": "flop = 2.5 x forward (5 GEMMs); the kernels execute 7 (S and dP are recomputed by the dQ pass)"}
+        "gate_worst_abs_error": {n: round(e, 5) for n, e in worst.items()},
+        "note": "flop = 2.5 x forward (5 GEMMs); the kernels execute 7 (S and dP are recomputed by the dQ pass)"},
+        rb, MFMA_PEAK_TFLOPS, "frac_of_mfma_peak")
     all_cfg["c5_flash_fwd_bwd_bf16"] = {
         "value": round((fl5 + flb) / ((msf + msb) * 1e-3) / 1e12, 1), "unit": "TFLOP/s",
         "frac_of_mfma_peak": round((fl5 + flb) / ((msf + msb) * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, 4)}
+    if do_cpu:
+        # naive oracle on batch 0, head 0: 128 query rows against all 8192 keys, scaled by flops
+        r128 = slice(0, 128)
+        fl_s = 4 * 128 * 8192 * 64
+        t1, tn = cpu_both(oracle, lambda: oracle.flash_fwd(qs[:, r128], ks_, vs_, 0.125, (-1, -1)), n_thr, 1)
+        all_cfg["c5_flash_fwd_bf16"].update(cpu_1core_TFLOPs=round(fl_s / t1 / 1e12, 6), cpu_allcore_TFLOPs=round(fl_s / tn / 1e12, 6),
+                                            cpu_cores=n_thr, cpu_sample="naive oracle, 1 batch x 1 head x 128 query rows x 8192 keys, by flop count")
+        o_s = fwd_out[0][:1, r128, :1].contiguous().view(torch.int16).cpu().numpy().view(np.uint16)
+        lse_s = fwd_out[1][:1, :1, r128].contiguous().cpu().numpy()
+        bw = lambda: oracle.flash_bwd(dos[:, r128], qs[:, r128], ks_, vs_, o_s, lse_s, 0.125, (-1, -1))
+        t1, tn = cpu_both(oracle, bw, n_thr, 1)
+        all_cfg["c5_flash_bwd_bf16"].update(cpu_1core_TFLOPs=round(2.5 * fl_s / t1 / 1e12, 6), cpu_allcore_TFLOPs=round(2.5 * fl_s / tn / 1e12, 6),
+                                            cpu_cores=n_thr, cpu_sample="naive oracle backward, 1 batch x 1 head x 128 query rows x 8192 keys, by flop count")
     del q, k, v, do, o, lse, bwd_out, fwd_out
 
     # decode against a key/value cache (not a BASELINE configuration; the serving-side call of the
     # same library): one new token per sequence, fp16, 64 sequences x 8192 cached keys,
     # 32 query heads on 8 key/value heads of 128: the 2 GiB cache is read once per call
     b_, h_, hk_, sk_, d_ = 64, 32, 8, 8192, 128
-    gen.manual_seed(0xDC)
-    qd = torch.randn((b_, 1, h_, d_), generator=gen, device="cuda").half()
-    kc, vc = (torch.randn((b_, sk_, hk_, d_), generator=gen, device="cuda").half() for _ in range(2))
-    kn, vn = (torch.randn((b_, 1, hk_, d_), generator=gen, device="cuda").half() for _ in range(2))
+    mkd = lambda shape, jj: mk(shape, H, _lib.FILL_NORMAL, SEED["dec"] + (jj << 32), 0.0, 1.0)
+    qd, kc, vc, kn, vn = mkd((b_, 1, h_, d_), 0), mkd((b_, sk_, hk_, d_), 1), mkd((b_, sk_, hk_, d_), 2), mkd((b_, 1, hk_, d_), 3), mkd((b_, 1, hk_, d_), 4)
     lens = torch.full((b_,), sk_ - 1, dtype=torch.int32, device="cuda")
     dec = lambda: ops.flash_attn_kvcache(qd, kc, vc, kn, vn, lens, 1.0 / np.sqrt(d_), (-1, -1))
-    msd, _, _ = time_ops(ev, [dec], steps, warm)
+    rd = time_ops(ev, [dec], steps, warm)
+    msd = rd["ms"]
     byt = 2 * b_ * sk_ * hk_ * d_ * 2
     all_cfg["kvcache_decode_fp16"] = {
         "value": round(byt / (msd * 1e-3) / 1e9, 1), "unit": "GB/s", "us_per_op": round(msd * 1e3, 1),

@@ -8,6 +8,7 @@ LIB_DIR = os.path.join(_HERE, "lib")
 
 F32, F16, BF16 = 0, 1, 2
 REDUCE_SUM, REDUCE_MAX, REDUCE_MIN, REDUCE_PROD, REDUCE_MEAN, REDUCE_SUMSQR = range(6)
+FILL_UNIFORM, FILL_NORMAL = 0, 1
 REDUCE_STATIC_SCRATCH_BYTES = 8 << 20
 ERROR_STATIC_SCRATCH_TOO_SMALL = 20001
 
@@ -60,6 +61,7 @@ def kernels():
         L.brt_rocm_event_record.argtypes = [vp, vp]
         L.brt_rocm_event_synchronize.argtypes = [vp]
         L.brt_rocm_event_elapsed_ms.argtypes = [ctypes.POINTER(ctypes.c_float), vp, vp]
+        L.brt_rocm_fill.argtypes = [i32, i32, ctypes.c_uint64, vp, sz, ctypes.c_float, ctypes.c_float, vp]
         L.brt_rocm_reduce_workspace_bytes.argtypes = [i32, sz, sz, sz]
         L.brt_rocm_reduce_workspace_bytes.restype = sz
         L.brt_rocm_reduce.argtypes = [i32, i32, vp, vp, sz, sz, sz, vp, sz, vp]

@@ -28,6 +28,14 @@ def _dev(t):
     return ctypes.c_void_p(t.data_ptr())
 
 
+def fill(t, dist, seed, a=0.0, b=1.0, stream=None):
+    """Counter-based synthetic data in place (brt_rocm_fill): element i is a function of
+    (seed, i) only; dist = _lib.FILL_UNIFORM ([a, b)) or _lib.FILL_NORMAL (mean 0, sigma b)."""
+    _lib.check(_lib.kernels().brt_rocm_fill(_DT[t.dtype], dist, seed, _dev(t), t.numel(), a, b, _stream(stream)),
+               "brt_rocm_fill")
+    return t
+
+
 def deduce_output_shape(shape, dims):
     """reduction::DeduceOutputShape, runtime/lib/core/common/utils/math_helper.cc:145-159."""
     for d in dims:

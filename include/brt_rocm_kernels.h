@@ -78,6 +78,19 @@ int brt_rocm_event_record(void *event, void *stream);
 int brt_rocm_event_synchronize(void *event);
 int brt_rocm_event_elapsed_ms(float *ms, void *start, void *stop);
 
+/* ---- synthetic data -------------------------------------------------------------- */
+/* Fills `n` elements with a counter-based pseudo-random sequence: element i depends on
+ * (seed, i) only -- splitmix64 output number i (uniform) or 3i .. 3i + 2 (normal) -- through
+ * integer arithmetic and exact float operations, so a host restatement of the same lines gives
+ * the same bits (the benchmark's and the tests' CPU side generates its own copy instead of
+ * reading the buffer back).  BRT_ROCM_FILL_UNIFORM: x = fma(u, b - a, a), u = 24 random bits
+ * * 2^-24 in [0, 1).  BRT_ROCM_FILL_NORMAL: x = b * (sum of twelve 16-bit fields - 393210) *
+ * 2^-16, mean 0 and standard deviation b (twelve-term central limit, support +-6 b); a unused.
+ * Stored as f32 / f16 / bf16 with round-to-nearest-even.  The reference has no counterpart: its
+ * tests fill buffers on the host (runtime/test/include/brt/test/common/util.h). */
+enum { BRT_ROCM_FILL_UNIFORM = 0, BRT_ROCM_FILL_NORMAL = 1 };
+int brt_rocm_fill(int dtype, int dist, uint64_t seed, void *ptr, size_t n, float a, float b, void *stream);
+
 /* ---- reductions ------------------------------------------------------------------ */
 /* out[a, c] = fold_b in[a, b, c] for a dense row-major tensor viewed as [A, B, C];
  * f16 is folded in float.  Stands in for

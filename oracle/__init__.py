@@ -83,6 +83,9 @@ def lib():
         L.oracle_flash_bwd.argtypes = [ctypes.POINTER(FaArgs), i32, i32] + [vp] * 10
         L.oracle_flash_fwd_rng.argtypes = [ctypes.POINTER(FaArgs), i32, i32] + [vp] * 7
         L.oracle_flash_bwd_rng.argtypes = [ctypes.POINTER(FaArgs), i32, i32] + [vp] * 11
+        L.oracle_splitmix64_at.argtypes = [u64, u64]
+        L.oracle_splitmix64_at.restype = u64
+        L.oracle_fill.argtypes = [i32, i32, u64, u64, u64, ctypes.c_float, ctypes.c_float, vp]
         L.oracle_philox4x32.argtypes = [u64, u64, u64, i32, vp]
         L.oracle_dropout_keep.argtypes = [vp, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_uint8]
         L.oracle_dropout_keep.restype = i32
@@ -166,6 +169,17 @@ def reduce_canonicalize(in_shape, out_shape, dims):
 
 def use_reduce_column(A, B, C):
     return bool(lib().oracle_use_reduce_column(A, B, C))
+
+
+UNIFORM, NORMAL = 0, 1
+
+
+def fill(dtype_code, dist, seed, count, a=0.0, b=1.0, first=0):
+    """Elements first .. first + count - 1 of the counter-based sequence brt_rocm_fill writes:
+    float32 array for dtype_code 0, uint16 storage bits for 1 (f16) and 2 (bf16)."""
+    out = np.empty(int(count), dtype=np.float32 if dtype_code == 0 else np.uint16)
+    lib().oracle_fill(dtype_code, dist, int(seed), int(first), int(count), a, b, _p(out))
+    return out
 
 
 def reference_workspace_bytes(A, B, C, elem_size=4):

@@ -52,6 +52,46 @@ void oracle_set_threads(int n) { g_threads = n < 1 ? 1 : n; }
 int oracle_get_threads(void) { return g_threads; }
 
 /* ------------------------------------------------------------------------------------ */
+/* Counter-based synthetic data, the host side of brt_rocm_fill (include/brt_rocm_kernels.h): */
+/* element i = f(seed, i) through splitmix64 (Steele, Lea, Flood 2014; the mixer of           */
+/* java.util.SplittableRandom), integer sums and exact float operations.  Pinned by the        */
+/* published splitmix64 outputs for seed 1234567 and by moments of the two distributions.      */
+/* ------------------------------------------------------------------------------------ */
+uint64_t oracle_splitmix64_at(uint64_t seed, uint64_t i) {
+  uint64_t z = seed + (i + 1) * 0x9E3779B97F4A7C15ull;
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  return z ^ (z >> 31);
+}
+float oracle_h2f(uint16_t h);
+uint16_t oracle_f2h(float f);
+uint16_t oracle_f2bf(float f);
+/* dist 0: uniform [a, b); 1: normal, mean 0, sigma b.  dtype 0 f32, 1 f16, 2 bf16 (RNE).
+ * Fills out[0 .. count) with the elements first .. first + count - 1 of the sequence. */
+void oracle_fill(int dtype, int dist, uint64_t seed, uint64_t first, uint64_t count, float a, float b, void *out) {
+  for (uint64_t k = 0; k < count; ++k) {
+    const uint64_t i = first + k;
+    volatile float x;  /* every operation rounds to float, no contraction */
+    if (dist == 0) {
+      const float u = (float)(uint32_t)(oracle_splitmix64_at(seed, i) >> 40) * 0x1p-24f;
+      volatile float w = b - a;
+      x = fmaf(u, w, a);  /* one rounding, as the device's fused multiply-add */
+    } else {
+      uint32_t sum = 0;
+      for (int j = 0; j < 3; ++j) {
+        const uint64_t z = oracle_splitmix64_at(seed, 3 * i + j);
+        sum += (uint32_t)(z & 0xffff) + (uint32_t)((z >> 16) & 0xffff) + (uint32_t)((z >> 32) & 0xffff) + (uint32_t)(z >> 48);
+      }
+      volatile float t = (float)((int32_t)sum - 393210) * 0x1p-16f;
+      x = t * b;
+    }
+    if (dtype == 0) ((float *)out)[k] = x;
+    else if (dtype == 1) ((uint16_t *)out)[k] = oracle_f2h(x);
+    else ((uint16_t *)out)[k] = oracle_f2bf(x);
+  }
+}
+
+/* ------------------------------------------------------------------------------------ */
 /* 16-bit float storage types (round-to-nearest-even), bit-exact with IEEE binary16 and  */
 /* bfloat16.  dtype codes: 0 = f32, 1 = f16, 2 = bf16.                                   */
 /* ------------------------------------------------------------------------------------ */
