@@ -11,16 +11,20 @@
 //   OpKernel                             framework/op_kernel.h:69-178
 //   KernelRegistry + static registration framework/kernel_registry.h:28-94
 //   ExecutionProvider                    framework/execution_provider.h:41-115
-//   ExecutionContext / ExecutionFrame    context/execution_context.h:36-50, execution_frame.h
+//   ExecutionContext / ExecutionFrame    context/execution_context.h:36-50, execution_frame.h:97-160
+//   Events / EventListenerManager        framework/event.h:27-74
+//   OpKernelWithWorkspace                framework/op_kernel_impl_base.h:116-149 (the Workspace argument)
 //   Session / RequestContext             session/session.h:50-146, request_context.h:44-92
 // This host code includes no HIP header: devices are reached through the C ABI of
 // libbrt_rocm_kernels.so (include/brt_rocm_kernels.h).
 #pragma once
 
+#include <array>
 #include <cstdint>
 #include <functional>
 #include <map>
 #include <memory>
+#include <mutex>
 #include <stdexcept>
 #include <string>
 #include <unordered_map>
@@ -163,6 +167,33 @@ private:
 
 // ---- events ----------------------------------------------------------------------------------
 class OpKernelInfo;
+// Event kinds and their payloads, as the reference's Events (framework/event.h:27-50): a
+// listener is registered for one kind and receives that kind's struct.
+struct Events {
+  struct BeforeExecutionPlanRun { static constexpr uint8_t kIdx = 0; };
+  struct AfterExecutionPlanRun { static constexpr uint8_t kIdx = 1; };
+  struct BeforeOpKernelRun { static constexpr uint8_t kIdx = 2; const OpKernelInfo &info; };
+  struct AfterOpKernelRun { static constexpr uint8_t kIdx = 3; const OpKernelInfo &info; };
+  static constexpr uint8_t kSize = 4;
+  template <typename T> using Listener = std::function<void(const T &)>;
+};
+
+class EventListenerManager {
+public:
+  template <typename T> void AddEventListener(Events::Listener<T> &&listener) {
+    static_assert(T::kIdx < Events::kSize, "unknown event kind");
+    auto held = std::make_shared<Events::Listener<T>>(std::move(listener));
+    slots_[T::kIdx].push_back([held](const void *event) { (*held)(*static_cast<const T *>(event)); });
+  }
+  template <typename T> void SignalEvent(const T &event) {
+    for (auto &call : slots_[T::kIdx]) call(&event);
+  }
+
+private:
+  std::array<std::vector<std::function<void(const void *)>>, Events::kSize> slots_;
+};
+
+// the flat form the C ABI hands to foreign hosts: one callback for both op-kernel events
 struct OpRunEvent {
   const OpKernelInfo *info;
   bool after;  // false: BeforeOpKernelRun, true: AfterOpKernelRun
@@ -173,28 +204,50 @@ using OpRunListener = std::function<void(const OpRunEvent &)>;
 class Session;
 class ExecutionFrame {
 public:
+  // Names the per-frame state slots of a plan (workspaces, handles): a key gets one offset the
+  // first time any frame asks for it, every frame then fills its own slot at that offset
+  // (the reference's ExecutionFrame::StateInfo, context/execution_frame.h:97-160).
+  struct StateInfo {
+    bool HasState(const std::string &key);
+    size_t GetStateOffset(const std::string &key);  // throws for an unknown key
+    // creates the key's offset if needed, and this frame's state (by calling `make`) if the
+    // frame has none at that offset
+    common::Status CreateStateIfNotExist(const std::string &key, ExecutionFrame *frame, const std::function<void *()> &make);
+
+  private:
+    std::mutex mutex_;
+    std::unordered_map<std::string, size_t> name_to_offset_;
+  };
+
   // device pointer of a value id (entry argument, intermediate or alias)
   void *GetAsyncValue(int value_id) const;
-  // per-frame state owned by op kernels (workspaces), keyed by op index
-  void *GetState(int op_index) const;
-  void SetState(int op_index, void *p);
+  // per-frame state by StateInfo offset
+  void *GetState(size_t offset) const { return offset < state_.size() ? state_[offset] : nullptr; }
+  void SetState(size_t offset, void *p);
+  void *GetAndResetState(size_t offset);
 
 private:
   friend class Session;
   friend class RequestContext;
   std::vector<void *> base_;        // per value: bound/allocated pointer (aliases resolved lazily)
   std::vector<bool> owned_;         // allocated by the frame
-  std::vector<void *> state_;       // per op
+  std::vector<void *> state_;       // per StateInfo offset
   std::vector<std::pair<std::string, void *>> arenas_;  // one block per memory space for the intermediates
   const ir::ByREHandle *ir_ = nullptr;
   bool prologue_done_ = false;
   bool io_bound_ = false;
 };
 
+// A light bundle of what an op kernel may touch while it runs; owns nothing
+// (context/execution_context.h:36-50; the distributed backend of the reference is not part of
+// this build).
 struct ExecutionContext {
   ExecutionFrame *exec_frame;
   WorkQueue *work_queue;
-  std::vector<OpRunListener> *listeners;
+  ExecutionFrame::StateInfo &frame_state_info;
+  EventListenerManager *event_listener_manager;
+  ExecutionContext(ExecutionFrame *frame, WorkQueue *wq, ExecutionFrame::StateInfo &fs_info, EventListenerManager *event_mgr)
+      : exec_frame(frame), work_queue(wq), frame_state_info(fs_info), event_listener_manager(event_mgr) {}
 };
 
 // ---- op kernels --------------------------------------------------------------------------------
@@ -247,18 +300,50 @@ private:
 
 class OpKernel {
 public:
-  explicit OpKernel(const OpKernelInfo &info) : info_(info) {}
+  // The four flags say which hooks the kernel implements; the plan calls only those
+  // (framework/op_kernel.h:69-78, execution_plan.cc:313-352).
+  explicit OpKernel(const OpKernelInfo &info, bool prologue_per_session = false, bool epilogue_per_session = false,
+                    bool prologue_per_frame = false, bool epilogue_per_frame = false)
+      : info_(info), has_prologue_per_session_(prologue_per_session), has_epilogue_per_session_(epilogue_per_session),
+        has_prologue_per_frame_(prologue_per_frame), has_epilogue_per_frame_(epilogue_per_frame) {}
   virtual ~OpKernel() = default;
-  // enqueue on ctx.work_queue; never synchronises
-  virtual common::Status RunImpl(const ExecutionContext &ctx) = 0;
+  OpKernel(const OpKernel &) = delete;
+  OpKernel &operator=(const OpKernel &) = delete;
+  // once when the model has been loaded / when the session ends
+  virtual common::Status ProloguePerSession() { return common::Status::Fail("OpKernel no implemented."); }
+  virtual common::Status EpiloguePerSession() { return common::Status::Fail("OpKernel no implemented."); }
   // once per frame before its first run / when the frame is destroyed (workspace life cycle)
-  virtual common::Status ProloguePerFrame(const ExecutionContext &) { return common::Status::OK(); }
-  virtual common::Status EpiloguePerFrame(const ExecutionContext &) { return common::Status::OK(); }
-  common::Status Run(const ExecutionContext &ctx);  // listeners + RunImpl
+  virtual common::Status ProloguePerFrame(const ExecutionContext &) { return common::Status::Fail("OpKernel no implemented."); }
+  virtual common::Status EpiloguePerFrame(const ExecutionContext &) { return common::Status::Fail("OpKernel no implemented."); }
+  // enqueue on ctx.work_queue; never synchronises
+  virtual common::Status RunImpl(const ExecutionContext &) { return common::Status::Fail("OpKernel no implemented."); }
+  common::Status Run(const ExecutionContext &ctx);  // Before/AfterOpKernelRun events around RunImpl
   const OpKernelInfo &GetOpKernelInfo() const { return info_; }
+  bool HasProloguePerSession() const { return has_prologue_per_session_; }
+  bool HasEpiloguePerSession() const { return has_epilogue_per_session_; }
+  bool HasProloguePerFrame() const { return has_prologue_per_frame_; }
+  bool HasEpiloguePerFrame() const { return has_epilogue_per_frame_; }
 
 protected:
-  OpKernelInfo info_;
+  const OpKernelInfo info_;
+  bool has_prologue_per_session_, has_epilogue_per_session_, has_prologue_per_frame_, has_epilogue_per_frame_;
+};
+
+// An op kernel with a temporary workspace: the size is asked once per frame, the buffer comes
+// from the allocator of the kernel's last operand, lives in the frame's state under the op's
+// UID and is released with the frame -- what the reference's `Workspace` kernel argument does
+// (framework/op_kernel_impl_base.h:116-149).
+class OpKernelWithWorkspace : public OpKernel {
+public:
+  explicit OpKernelWithWorkspace(const OpKernelInfo &info) : OpKernel(info, false, false, true, true) {}
+  virtual size_t GetWorkspaceSize(const ExecutionContext &ctx) const = 0;
+  common::Status ProloguePerFrame(const ExecutionContext &ctx) override;
+  common::Status EpiloguePerFrame(const ExecutionContext &ctx) override;
+
+protected:
+  void *GetWorkspace(const ExecutionContext &ctx) const;  // nullptr when the size is 0
+  IAllocator *GetAllocator() const;
+  std::string GetOpUID() const;
 };
 
 using KernelCreateFn = std::function<std::shared_ptr<OpKernel>(const OpKernelInfo &)>;
@@ -327,7 +412,8 @@ public:
   void *GetArg(size_t offset);
   void FinishIOBinding();
   common::Status Sync();
-  void AddOpRunListener(OpRunListener l) { listeners_.push_back(std::move(l)); }
+  void AddOpRunListener(OpRunListener l);  // both op-kernel events through one callback
+  EventListenerManager &GetEventListenerManager() { return events_; }
   ExecutionFrame *GetExecutionFrame() { return frame_.get(); }
   WorkQueue *GetWorkQueue() { return wq_.get(); }
 
@@ -337,7 +423,7 @@ private:
   Session &session_;
   std::unique_ptr<ExecutionFrame> frame_;
   std::unique_ptr<WorkQueue> wq_;
-  std::vector<OpRunListener> listeners_;
+  EventListenerManager events_;
 };
 
 class Session {
@@ -392,16 +478,18 @@ private:
   std::vector<size_t> intermediate_offset_;
   std::unordered_map<std::string, size_t> arena_bytes_;
   std::function<WorkQueue *()> wq_factory_;
+  ExecutionFrame::StateInfo frame_state_info_;  // shared by every frame of this session
 };
 
 // ---- ROCm device layer (rocm_provider.cc) ------------------------------------------------------------
-// Allocators answering to the memory spaces "cuda" (so existing ByRE modules run unchanged) and
-// "cpu"; work queues on an owned or a caller-supplied HIP stream; the provider itself.
+// Allocators answering to the memory spaces "cuda" (so existing ByRE modules run unchanged),
+// "cudaPinned" (page-locked host memory) and "cpu"; work queues on an owned or a caller-supplied HIP stream; the provider itself.
 using ExternalAllocFn = void *(*)(size_t);
 using ExternalFreeFn = void (*)(void *);
 std::unique_ptr<IAllocator> MakeRocmAllocator(const std::string &key = "cuda");
 std::unique_ptr<IAllocator> MakeExternalAllocator(const std::string &key, ExternalAllocFn a, ExternalFreeFn f);
 std::unique_ptr<IAllocator> MakeHostAllocator(const std::string &key = "cpu");
+std::unique_ptr<IAllocator> MakeRocmPinnedAllocator(const std::string &key = "cudaPinned");
 WorkQueue *MakeRocmSingleStreamWorkQueue(int device_id);
 WorkQueue *MakeRocmExternalStreamWorkQueue(void *stream);
 common::Status DefaultROCMExecutionProviderFactory(Session *session, int device_id = 0);

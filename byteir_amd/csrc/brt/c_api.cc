@@ -39,7 +39,7 @@ brt_session *brt_session_create(int device_id, brt_alloc_fn alloc, brt_free_fn f
     std::unique_ptr<brt_session> s(new brt_session);
     if (device_id < 0) {  // plan-only: host memory stands in for every space, Run is refused
       s->plan_only = true;
-      for (const char *k : {"cuda", "rocm", "cpu"}) s->session.AddAllocator(MakeHostAllocator(k));
+      for (const char *k : {"cuda", "rocm", "cpu", "cudaPinned"}) s->session.AddAllocator(MakeHostAllocator(k));
       s->session.SetWorkQueueFactory([]() { return MakeRocmExternalStreamWorkQueue(nullptr); });
       s->session.AddExecutionProvider(std::unique_ptr<ExecutionProvider>(new ExecutionProvider(DeviceKind::ROCM, ProviderType::BRT)));
       return s.release();

@@ -50,6 +50,18 @@ private:
   ExternalFreeFn f_;
 };
 
+class RocmPinnedAllocator : public IAllocator {  // page-locked host memory (hipHostMalloc)
+public:
+  using IAllocator::IAllocator;
+  void *Alloc(size_t size) override {
+    void *p = nullptr;
+    const int e = brt_rocm_host_malloc(&p, size ? size : kAllocAlignment);
+    BRT_ENFORCE(e == 0, "pinned host allocation of " + std::to_string(size) + " bytes failed: " + HipErr(e));
+    return p;
+  }
+  void Free(void *p) override { if (p) brt_rocm_host_free(p); }
+};
+
 class HostAllocator : public IAllocator {
 public:
   using IAllocator::IAllocator;
@@ -84,9 +96,9 @@ void *StreamOf(const ExecutionContext &ctx) {
 // ---- ReduceSumOp / ReduceMaxOp ----------------------------------------------------------------------
 // Canonicalises the reduced dimensions to [A, B, C] exactly as ReduceImpl's constructor
 // (reduce_impl.h:30-59) and owns a per-frame workspace sized at plan time.
-class ReduceOpKernel : public OpKernel {
+class ReduceOpKernel : public OpKernelWithWorkspace {
 public:
-  ReduceOpKernel(const OpKernelInfo &info, int op, int dtype) : OpKernel(info), op_(op), dtype_(dtype) {
+  ReduceOpKernel(const OpKernelInfo &info, int op, int dtype) : OpKernelWithWorkspace(info), op_(op), dtype_(dtype) {
     OpAccessor acc(info_);
     BRT_ENFORCE(acc.GetNumArgs() == 2, "reduce takes an input and an output");
     Shape shape = acc.GetArgShape(0);
@@ -110,29 +122,13 @@ public:
     for (size_t i = (size_t)dims.back() + 1; i < shape.size(); ++i) C_ *= (size_t)shape[i];
   }
 
-  size_t GetWorkspaceSize() const { return brt_rocm_reduce_workspace_bytes(dtype_, A_, B_, C_); }
+  // asked once per frame, where the reference asks ReduceImpl::GetWorkspaceSize (reduce_impl.h:76-79)
+  size_t GetWorkspaceSize(const ExecutionContext &) const override { return brt_rocm_reduce_workspace_bytes(dtype_, A_, B_, C_); }
 
-  common::Status ProloguePerFrame(const ExecutionContext &ctx) override {
-    const size_t n = GetWorkspaceSize();
-    if (n == 0) return common::Status::OK();
-    OpAccessor acc(info_);
-    IAllocator *a = info_.GetAllocator(acc.GetArgSpace(acc.GetNumArgs() - 1));  // last operand's allocator
-    BRT_ENFORCE(a != nullptr, "no allocator for the reduce workspace");
-    ctx.exec_frame->SetState(info_.GetOpId(), a->Alloc(n));
-    return common::Status::OK();
-  }
-  common::Status EpiloguePerFrame(const ExecutionContext &ctx) override {
-    if (void *p = ctx.exec_frame->GetState(info_.GetOpId())) {
-      OpAccessor acc(info_);
-      if (IAllocator *a = info_.GetAllocator(acc.GetArgSpace(acc.GetNumArgs() - 1))) a->Free(p);
-      ctx.exec_frame->SetState(info_.GetOpId(), nullptr);
-    }
-    return common::Status::OK();
-  }
   common::Status RunImpl(const ExecutionContext &ctx) override {
     OpAccessor acc(info_, ctx.exec_frame);
     const int e = brt_rocm_reduce(op_, dtype_, acc.GetArgAsyncValueRef(0), acc.GetArgAsyncValueRef(1), A_, B_, C_,
-                                  ctx.exec_frame->GetState(info_.GetOpId()), GetWorkspaceSize(), StreamOf(ctx));
+                                  GetWorkspace(ctx), GetWorkspaceSize(ctx), StreamOf(ctx));
     return HipStatus(e, "reduce");
   }
 
@@ -200,19 +196,42 @@ public:
     const char *lib_version = *static_cast<const char **>(ver);
     if (lib_version && version != lib_version)
       std::fprintf(stderr, "brt: custom library %s reports version %s, the module asks for %s\n", lib_path.c_str(), lib_version, version.c_str());
+    // The (tensors, extra_args, stream) ABI has no error channel, and this library's entry
+    // points abort on arguments they cannot serve.  When the library also exports the
+    // error-returning forms (flash_attn_{fwd,bwd,kvcache}_checked + flash_attn_last_error), the
+    // op kernel calls those, so a bad module fails Session::Run instead of ending the process.
+    static const struct { const char *api, *checked; int dtype; } kChecked[] = {
+        {"run_flash_attn_fwd", "flash_attn_fwd_checked", 1},       {"run_flash_attn_fwd_bf16", "flash_attn_fwd_checked", 2},
+        {"run_flash_attn_bwd", "flash_attn_bwd_checked", 1},       {"run_flash_attn_bwd_bf16", "flash_attn_bwd_checked", 2},
+        {"run_flash_attn_kvcache", "flash_attn_kvcache_checked", 1}, {"run_flash_attn_kvcache_bf16", "flash_attn_kvcache_checked", 2}};
+    for (const auto &c : kChecked) {
+      if (api_name != c.api) continue;
+      checked_ = reinterpret_cast<CheckedFn>(dlsym(handle_, c.checked));
+      last_error_ = reinterpret_cast<LastErrorFn>(dlsym(handle_, "flash_attn_last_error"));
+      checked_dtype_ = c.dtype;
+    }
   }
   common::Status RunImpl(const ExecutionContext &ctx) override {
     OpAccessor acc(info_, ctx.exec_frame);
     std::vector<void *> tensors(acc.GetNumArgs());
     for (size_t i = 0; i < tensors.size(); ++i) tensors[i] = acc.GetArgAsyncValueRef(i);
     void *extra = acc.GetAttrAsVoidPtr("extra_args");
-    run_(tensors.data(), extra, StreamOf(ctx));
+    common::Status st = common::Status::OK();
+    if (checked_ && last_error_) {
+      const int e = checked_(tensors.data(), extra, checked_dtype_, StreamOf(ctx));
+      if (e < 0) st = common::Status::Fail(std::string("custom op: ") + last_error_());
+      else if (e > 0) st = HipStatus(e, "custom op launch");
+    } else {
+      run_(tensors.data(), extra, StreamOf(ctx));
+    }
     std::free(extra);
-    return common::Status::OK();
+    return st;
   }
 
 private:
   using RunFn = void (*)(void **, void *, void *);
+  using CheckedFn = int (*)(void **, const void *, int, void *);
+  using LastErrorFn = const char *(*)();
   static void *Open(const std::string &path) {
     if (void *h = dlopen(path.c_str(), RTLD_LAZY | RTLD_GLOBAL)) return h;
     const std::string base = path.substr(path.find_last_of('/') == std::string::npos ? 0 : path.find_last_of('/') + 1);
@@ -228,6 +247,9 @@ private:
   }
   void *handle_ = nullptr;
   RunFn run_ = nullptr;
+  CheckedFn checked_ = nullptr;
+  LastErrorFn last_error_ = nullptr;
+  int checked_dtype_ = 0;
 };
 
 // ---- copies: cpu2cuda, cuda2cpu, cuda2cuda (operands: src, dst) ---------------------------------------------
@@ -297,6 +319,7 @@ std::unique_ptr<IAllocator> MakeExternalAllocator(const std::string &key, Extern
   return std::unique_ptr<IAllocator>(new ExternalAllocator(key, a, f));
 }
 std::unique_ptr<IAllocator> MakeHostAllocator(const std::string &key) { return std::unique_ptr<IAllocator>(new HostAllocator(key)); }
+std::unique_ptr<IAllocator> MakeRocmPinnedAllocator(const std::string &key) { return std::unique_ptr<IAllocator>(new RocmPinnedAllocator(key)); }
 
 WorkQueue *MakeRocmSingleStreamWorkQueue(int device_id) {
   BRT_ENFORCE(brt_rocm_set_device(device_id) == 0, "cannot select device " + std::to_string(device_id));
@@ -320,6 +343,9 @@ common::Status ROCMAllocatorFactory(Session *session, int device_id) {
   session->AddAllocator(MakeRocmAllocator("cuda"));
   session->AddAllocator(MakeRocmAllocator("rocm"));
   session->AddAllocator(MakeHostAllocator("cpu"));
+  // page-locked host memory, the key the reference's CUDAAllocatorFactory registers beside
+  // "cuda" (runtime/lib/backends/cuda/device/cuda_allocator.cc:88-110)
+  session->AddAllocator(MakeRocmPinnedAllocator("cudaPinned"));
   return common::Status::OK();
 }
 

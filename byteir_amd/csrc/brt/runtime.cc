@@ -188,15 +188,41 @@ void *OpAccessor::GetArgAsyncValueRef(size_t i) const {
 }
 
 common::Status OpKernel::Run(const ExecutionContext &ctx) {
-  if (ctx.listeners) for (auto &l : *ctx.listeners) l(OpRunEvent{&info_, false});
+  if (ctx.event_listener_manager) ctx.event_listener_manager->SignalEvent<Events::BeforeOpKernelRun>({info_});
   common::Status s;
   try {
     s = RunImpl(ctx);
   } catch (const std::exception &e) {
     s = common::Status::Fail(e.what());
   }
-  if (ctx.listeners) for (auto &l : *ctx.listeners) l(OpRunEvent{&info_, true});
+  if (ctx.event_listener_manager) ctx.event_listener_manager->SignalEvent<Events::AfterOpKernelRun>({info_});
   return s;
+}
+
+// ---- op kernels with a workspace ---------------------------------------------------------------------
+std::string OpKernelWithWorkspace::GetOpUID() const { return OpAccessor(info_).GetUID(); }
+IAllocator *OpKernelWithWorkspace::GetAllocator() const {
+  OpAccessor acc(info_);
+  return info_.GetAllocator(acc.GetArgSpace(acc.GetNumArgs() - 1));  // the last operand's memory space
+}
+common::Status OpKernelWithWorkspace::ProloguePerFrame(const ExecutionContext &ctx) {
+  const size_t bytes = GetWorkspaceSize(ctx);
+  return ctx.frame_state_info.CreateStateIfNotExist(GetOpUID(), ctx.exec_frame, [&]() -> void * {
+    if (bytes == 0) return nullptr;
+    IAllocator *a = GetAllocator();
+    BRT_ENFORCE(a != nullptr, "no allocator for the workspace of " + GetOpUID());
+    return a->Alloc(bytes);
+  });
+}
+common::Status OpKernelWithWorkspace::EpiloguePerFrame(const ExecutionContext &ctx) {
+  if (!ctx.frame_state_info.HasState(GetOpUID())) return common::Status::OK();
+  if (void *p = ctx.exec_frame->GetAndResetState(ctx.frame_state_info.GetStateOffset(GetOpUID())))
+    if (IAllocator *a = GetAllocator()) a->Free(p);
+  return common::Status::OK();
+}
+void *OpKernelWithWorkspace::GetWorkspace(const ExecutionContext &ctx) const {
+  if (!ctx.frame_state_info.HasState(GetOpUID())) return nullptr;
+  return ctx.exec_frame->GetState(ctx.frame_state_info.GetStateOffset(GetOpUID()));
 }
 
 // ---- frame ------------------------------------------------------------------------------------------
@@ -208,12 +234,45 @@ void *ExecutionFrame::GetAsyncValue(int value_id) const {
   }
   return base_[value_id];
 }
-void *ExecutionFrame::GetState(int op_index) const { return state_[op_index]; }
-void ExecutionFrame::SetState(int op_index, void *p) { state_[op_index] = p; }
+void ExecutionFrame::SetState(size_t offset, void *p) {
+  if (offset >= state_.size()) state_.resize(offset + 1, nullptr);
+  state_[offset] = p;
+}
+void *ExecutionFrame::GetAndResetState(size_t offset) {
+  void *p = GetState(offset);
+  if (offset < state_.size()) state_[offset] = nullptr;
+  return p;
+}
+bool ExecutionFrame::StateInfo::HasState(const std::string &key) {
+  std::lock_guard<std::mutex> lock(mutex_);
+  return name_to_offset_.count(key) != 0;
+}
+size_t ExecutionFrame::StateInfo::GetStateOffset(const std::string &key) {
+  std::lock_guard<std::mutex> lock(mutex_);
+  auto it = name_to_offset_.find(key);
+  BRT_ENFORCE(it != name_to_offset_.end(), "no frame state named " + key);
+  return it->second;
+}
+common::Status ExecutionFrame::StateInfo::CreateStateIfNotExist(const std::string &key, ExecutionFrame *frame,
+                                                                const std::function<void *()> &make) {
+  size_t offset;
+  {
+    std::lock_guard<std::mutex> lock(mutex_);
+    auto it = name_to_offset_.find(key);
+    if (it == name_to_offset_.end()) it = name_to_offset_.emplace(key, name_to_offset_.size()).first;
+    offset = it->second;
+  }
+  // every frame fills its own slot, also when another frame created the offset
+  if (frame->GetState(offset) == nullptr) frame->SetState(offset, make());
+  return common::Status::OK();
+}
 
 // ---- session ------------------------------------------------------------------------------------------
 Session::Session() = default;
-Session::~Session() = default;
+Session::~Session() {
+  for (auto &k : kernels_)
+    if (k->HasEpiloguePerSession()) { try { k->EpiloguePerSession(); } catch (...) {} }
+}
 
 common::Status Session::AddExecutionProvider(std::unique_ptr<ExecutionProvider> provider) {
   providers_.push_back(std::move(provider));
@@ -248,6 +307,8 @@ common::Status Session::LoadFromMemory(const std::string &text, const std::strin
 // kernels (shape checks and dlopen happen here), as StaticBRTExecutionPlan::ProloguePerSession
 // does (execution_plan.cc:314-438).
 common::Status Session::BuildPlan() {
+  for (auto &k : kernels_)  // a model loaded earlier ends here
+    if (k->HasEpiloguePerSession()) { try { k->EpiloguePerSession(); } catch (...) {} }
   kernels_.clear();
   infos_.clear();
   in_offsets_.clear(); out_offsets_.clear(); weight_offsets_.clear();
@@ -293,6 +354,13 @@ common::Status Session::BuildPlan() {
       return common::Status::Fail("constructing " + key + " (line " + std::to_string(ir_->ops[i].line) + "): " + e.what());
     }
   }
+  // one-time preparation of the kernels that ask for it (the reference calls this from
+  // Session::Load through ExecutionPlan::ProloguePerSession, execution_plan.cc:313-330)
+  for (auto &k : kernels_) {
+    if (!k->HasProloguePerSession()) continue;
+    common::Status s = k->ProloguePerSession();
+    if (!s.IsOK()) return s;
+  }
   return common::Status::OK();
 }
 
@@ -310,9 +378,15 @@ common::Status Session::NewRequestContext(std::unique_ptr<RequestContext> *reque
   f.ir_ = ir_.get();
   f.base_.assign(ir_->values.size(), nullptr);
   f.owned_.assign(ir_->values.size(), false);
-  f.state_.assign(ir_->ops.size(), nullptr);
+  f.state_.clear();
   *request = std::move(r);
   return common::Status::OK();
+}
+
+void RequestContext::AddOpRunListener(OpRunListener l) {
+  auto shared = std::make_shared<OpRunListener>(std::move(l));
+  events_.AddEventListener<Events::BeforeOpKernelRun>([shared](const Events::BeforeOpKernelRun &e) { (*shared)(OpRunEvent{&e.info, false}); });
+  events_.AddEventListener<Events::AfterOpKernelRun>([shared](const Events::AfterOpKernelRun &e) { (*shared)(OpRunEvent{&e.info, true}); });
 }
 
 size_t Session::GetArgNum() const { return ir_ ? ir_->args.size() : 0; }
@@ -329,27 +403,31 @@ std::string Session::GetSpace(size_t offset) const { return ir_->values[ir_->arg
 common::Status Session::Run(RequestContext &request) {
   ExecutionFrame &f = *request.frame_;
   if (!f.io_bound_) return common::Status::Fail("FinishIOBinding has not been called");
-  ExecutionContext ctx{&f, request.wq_.get(), &request.listeners_};
+  ExecutionContext ctx(&f, request.wq_.get(), frame_state_info_, &request.events_);
   if (!f.prologue_done_) {  // first run of this frame: workspaces (op_kernel_impl_base.h:116-136)
     for (auto &k : kernels_) {
+      if (!k->HasProloguePerFrame()) continue;
       common::Status s = k->ProloguePerFrame(ctx);
       if (!s.IsOK()) return s;
     }
     f.prologue_done_ = true;
   }
+  request.events_.SignalEvent<Events::BeforeExecutionPlanRun>({});
   for (auto &k : kernels_) {
     common::Status s = k->Run(ctx);
     if (!s.IsOK()) return s;
   }
+  request.events_.SignalEvent<Events::AfterExecutionPlanRun>({});
   return common::Status::OK();
 }
 
 void Session::Cleanup(RequestContext &request) noexcept {
   ExecutionFrame &f = *request.frame_;
-  ExecutionContext ctx{&f, request.wq_.get(), nullptr};
+  ExecutionContext ctx(&f, request.wq_.get(), frame_state_info_, nullptr);
   if (request.wq_) request.wq_->Sync();
   if (f.prologue_done_) {
     for (auto &k : kernels_) {
+      if (!k->HasEpiloguePerFrame()) continue;
       try { k->EpiloguePerFrame(ctx); } catch (...) {}
     }
     f.prologue_done_ = false;

@@ -244,6 +244,39 @@ def test_external_kernel_library_registers_statically(tmp_path):
         s.close()
 
 
+def test_reference_style_external_kernel_compiles_and_prepares(tmp_path):
+    """An op kernel written against the reference's OpKernel surface -- five-argument
+    constructor, ProloguePerSession, per-frame hooks using ExecutionContext::frame_state_info,
+    registration from a lambda (runtime/test/external_kernels/cuda/kernels.cc:37-99) -- builds
+    against brt.h; loading a module that uses it runs ProloguePerSession once per load."""
+    import ctypes
+    from byteir_amd import _lib, brt
+    from external_kernel_src import build
+    B = _lib.brt()
+    lib = build(tmp_path, ROOT)
+    assert B.brt_register_kernels_from_dynlib(str(lib).encode()) == 0, B.brt_last_error().decode()
+    ext = ctypes.CDLL(str(lib))
+    s = brt.Session(device_id=-1)
+    try:
+        assert s.has_kernel("CustomCopyOp")
+        t, pinned = memref([64], "f32", "cuda"), memref([64], "f32", "cudaPinned")
+        mod = f"""func.func @t(%a : {t} {{byre.argname = "a", byre.argtype = 1: i32}},
+                     %b : {t} {{byre.argname = "b", byre.argtype = 2: i32}}) attributes {{byre.entry_point}} {{
+          byre.compute @CustomCopyOp(%a, %b) : {t}, {t}
+          return }}"""
+        before = ext.ext_prologue_per_session()
+        s.load_from_memory(mod)
+        assert ext.ext_prologue_per_session() == before + 1 and ext.ext_prologue_per_frame() == 0
+        # a memref in page-locked host memory: the "cudaPinned" allocator key of the reference
+        # (runtime/lib/backends/cuda/device/cuda_allocator.cc:104-108) is known to the session
+        s.load_from_memory(mod.replace(f"%a : {t}", f"%a : {pinned}").replace(f"(%a, %b) : {t}", f"(%a, %b) : {pinned}"))
+        assert s.get_space(0) == "cudaPinned"
+        with pytest.raises(RuntimeError, match="no allocator for memory space"):
+            s.load_from_memory(mod.replace('"cuda"', '"nowhere"'))
+    finally:
+        s.close()
+
+
 def test_reference_kvcache_module_loads_unchanged(session, golden_dir):
     """flash_attn_kvcache.mlir of the reference: eight operands (one of them memref<2xi32>), the
     library is found by file name, the 244-byte blob is what the oracle packs."""

@@ -488,3 +488,70 @@ def test_device_memset_any_alignment_and_inside_a_graph():
         torch.cuda.synchronize()
         h = buf.cpu().numpy()
         assert np.all(h[3:4004] == 0) and np.all(h[:3] == 0x77) and np.all(h[4004:] == 0x77)
+
+
+def test_reference_style_external_kernel_runs_with_its_hooks(tmp_path):
+    """The external kernel of tests/external_kernel_src.py on the GPU: ProloguePerFrame once per
+    frame (also when the frame runs twice), its state found through frame_state_info on every
+    run, events around each run, EpiloguePerFrame when the request is destroyed, and a custom
+    op whose arguments the library refuses fails Session::Run instead of ending the process."""
+    import ctypes
+    from byteir_amd import _lib, brt
+    from external_kernel_src import build
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    lib = build(tmp_path, root)
+    assert _lib.brt().brt_register_kernels_from_dynlib(str(lib).encode()) == 0
+    ext = ctypes.CDLL(str(lib))
+    s = brt.Session(device="ROCM")
+    try:
+        t = 'memref<1000xf32, "cuda">'
+        s.load_from_memory(f"""func.func @t(%a : {t} {{byre.argname = "a", byre.argtype = 1: i32}},
+                     %b : {t} {{byre.argname = "b", byre.argtype = 2: i32}}) attributes {{byre.entry_point}} {{
+          byre.compute @CustomCopyOp(%a, %b) : {t}, {t}
+          return }}""")
+        f0, e0, r0 = ext.ext_prologue_per_frame(), ext.ext_epilogue_per_frame(), ext.ext_runs()
+        a = torch.arange(1000, dtype=torch.float32, device="cuda")
+        b = torch.zeros(1000, device="cuda")
+        req = s.new_request_context()
+        seen = []
+        req.add_op_listener(lambda key, idx, after: seen.append((key, after)))
+        req.bind_arg(0, a.data_ptr()); req.bind_arg(1, b.data_ptr()); req.finish_io_binding()
+        req.run(); req.run(); req.sync()
+        assert torch.equal(a, b)
+        assert ext.ext_prologue_per_frame() == f0 + 1 and ext.ext_runs() == r0 + 2
+        assert seen == [("CustomCopyOp", False), ("CustomCopyOp", True)] * 2
+        req2 = s.new_request_context()  # a second frame of the same plan: its own state, same offset
+        req2.bind_arg(0, a.data_ptr()); req2.bind_arg(1, b.data_ptr()); req2.finish_io_binding()
+        req2.run(); req2.sync()
+        assert ext.ext_prologue_per_frame() == f0 + 2
+        req.close(); req2.close()
+        assert ext.ext_epilogue_per_frame() == e0 + 2
+    finally:
+        s.close()
+
+
+def test_custom_op_with_unsupported_arguments_fails_the_run(session, golden_dir):
+    """head_dim 20 is not a multiple of 8: through the plain ABI the library would abort the
+    process; the custom op kernel uses the library's error-returning entry point instead."""
+    text = open(os.path.join(golden_dir, "flash_attn_fwd.mlir")).read()
+    # the fixture is b1 s128 h3 d32; declare d = 20 in the blob (fields 16..18 head strides stay)
+    import re
+    m = re.search(r"extra_args = \[([^\]]*)\]", text)
+    fields = [f.strip() for f in m.group(1).split(",")]
+    # blob order (flash_api.cu:586-624): 4 batch strides, 4 row strides, 4 head strides, b, h, h_k, d, ...
+    assert fields[15].startswith("32")
+    fields[15] = "20 : i64"
+    text = text.replace(m.group(1), ", ".join(fields))
+    session.load_from_memory(text)
+    req = session.new_request_context()
+    q, k, v = (torch.zeros((1, 128, 3, 32), dtype=torch.float16, device="cuda") for _ in range(3))
+    o = torch.zeros_like(q)
+    lse = torch.zeros((1, 3, 128), device="cuda")
+    for name, t in (("Q", q), ("K", k), ("V", v), ("Out", o), ("SoftmaxLse", lse)):
+        off = session.get_graph_arg_offset(name)
+        if off >= 0:
+            req.bind_arg(off, t.data_ptr())
+    req.finish_io_binding()
+    with pytest.raises(RuntimeError, match="custom op"):
+        req.run()
+    req.sync()
