@@ -69,6 +69,9 @@ def kernels():
         L.brt_rocm_reduce_static.argtypes = [i32, i32, vp, vp, sz, sz, sz, vp]
         L.brt_rocm_softmax.argtypes = [i32, vp, vp, sz, sz, vp]
         L.brt_rocm_softmax_axis.argtypes = [i32, vp, vp, sz, sz, sz, vp]
+        L.brt_rocm_softmax_axis_ws.argtypes = [i32, vp, vp, sz, sz, sz, vp, sz, vp]
+        L.brt_rocm_softmax_workspace_bytes.argtypes = [i32, sz, sz, sz]
+        L.brt_rocm_softmax_workspace_bytes.restype = sz
         _kernels = L
     return _kernels
 
@@ -93,6 +96,15 @@ def flash_attn():
             f = getattr(L, n)
             f.argtypes = [ctypes.POINTER(vp), vp, vp]
             f.restype = None
+        sz, i32 = ctypes.c_size_t, ctypes.c_int
+        for n in ("fwd", "bwd", "kvcache"):
+            getattr(L, f"flash_attn_{n}_checked").argtypes = [ctypes.POINTER(vp), vp, i32, vp]
+            getattr(L, f"flash_attn_{n}_ws").argtypes = [ctypes.POINTER(vp), vp, i32, vp, sz, vp]
+            getattr(L, f"flash_attn_{n}_workspace_bytes").restype = sz
+        L.flash_attn_fwd_workspace_bytes.argtypes = [vp, i32]
+        L.flash_attn_kvcache_workspace_bytes.argtypes = [vp, i32]
+        L.flash_attn_bwd_workspace_bytes.argtypes = [vp, i32, sz]
+        L.flash_attn_last_error.restype = ctypes.c_char_p
         _flash = L
     return _flash
 

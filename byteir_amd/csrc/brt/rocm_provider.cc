@@ -140,9 +140,9 @@ private:
 // ---- byteir.softmax -----------------------------------------------------------------------------------
 // A new op kernel (the reference runtime has none): operands (input, output), attribute `axis`,
 // (any axis of the tensor, the last one by default); element type f32, f16 or bf16.
-class SoftmaxOpKernel : public OpKernel {
+class SoftmaxOpKernel : public OpKernelWithWorkspace {
 public:
-  explicit SoftmaxOpKernel(const OpKernelInfo &info) : OpKernel(info) {
+  explicit SoftmaxOpKernel(const OpKernelInfo &info) : OpKernelWithWorkspace(info) {
     OpAccessor acc(info_);
     BRT_ENFORCE(acc.GetNumArgs() == 2, "softmax takes an input and an output");
     const Shape s = acc.GetArgShape(0);
@@ -161,9 +161,12 @@ public:
     a_ = b_ = c_ = 1;
     for (int64_t i = 0; i < (int64_t)s.size(); ++i) (i < axis ? a_ : i == axis ? b_ : c_) *= (size_t)s[i];
   }
+  // segment partials of an inner-axis softmax with few columns and a long axis; 0 otherwise
+  size_t GetWorkspaceSize(const ExecutionContext &) const override { return brt_rocm_softmax_workspace_bytes(dtype_, a_, b_, c_); }
   common::Status RunImpl(const ExecutionContext &ctx) override {
     OpAccessor acc(info_, ctx.exec_frame);
-    return HipStatus(brt_rocm_softmax_axis(dtype_, acc.GetArgAsyncValueRef(0), acc.GetArgAsyncValueRef(1), a_, b_, c_, StreamOf(ctx)), "softmax");
+    return HipStatus(brt_rocm_softmax_axis_ws(dtype_, acc.GetArgAsyncValueRef(0), acc.GetArgAsyncValueRef(1), a_, b_, c_,
+                                              GetWorkspace(ctx), GetWorkspaceSize(ctx), StreamOf(ctx)), "softmax");
   }
 
 private:
@@ -180,9 +183,9 @@ private:
 // A relative lib_path that does not resolve from the working directory is looked up by file name
 // in $BRT_CUSTOM_LIB_DIR and next to this runtime library, so modules carrying the reference's
 // paths ("external_libs/libs/libflash_attn.so") run without a matching directory layout.
-class CustomOpKernel : public OpKernel {
+class CustomOpKernel : public OpKernelWithWorkspace {
 public:
-  explicit CustomOpKernel(const OpKernelInfo &info) : OpKernel(info) {
+  explicit CustomOpKernel(const OpKernelInfo &info) : OpKernelWithWorkspace(info) {
     OpAccessor acc(info_);
     const std::string lib_path = acc.GetAttrAsString("lib_path");
     const std::string api_name = acc.GetAttrAsString("api_name");
@@ -196,20 +199,41 @@ public:
     const char *lib_version = *static_cast<const char **>(ver);
     if (lib_version && version != lib_version)
       std::fprintf(stderr, "brt: custom library %s reports version %s, the module asks for %s\n", lib_path.c_str(), lib_version, version.c_str());
-    // The (tensors, extra_args, stream) ABI has no error channel, and this library's entry
-    // points abort on arguments they cannot serve.  When the library also exports the
-    // error-returning forms (flash_attn_{fwd,bwd,kvcache}_checked + flash_attn_last_error), the
-    // op kernel calls those, so a bad module fails Session::Run instead of ending the process.
-    static const struct { const char *api, *checked; int dtype; } kChecked[] = {
-        {"run_flash_attn_fwd", "flash_attn_fwd_checked", 1},       {"run_flash_attn_fwd_bf16", "flash_attn_fwd_checked", 2},
-        {"run_flash_attn_bwd", "flash_attn_bwd_checked", 1},       {"run_flash_attn_bwd_bf16", "flash_attn_bwd_checked", 2},
-        {"run_flash_attn_kvcache", "flash_attn_kvcache_checked", 1}, {"run_flash_attn_kvcache_bf16", "flash_attn_kvcache_checked", 2}};
-    for (const auto &c : kChecked) {
+    // The (tensors, extra_args, stream) ABI has no error channel and no way to hand over
+    // scratch: this library's plain entry points abort on arguments they cannot serve and
+    // allocate their scratch themselves.  When the library also exports the extended forms
+    // (flash_attn_{fwd,bwd,kvcache}_ws + _workspace_bytes + flash_attn_last_error), the op kernel
+    // uses those: a bad module fails Session::Run instead of ending the process, and the
+    // scratch is a per-frame workspace from the frame's allocator, sized when the frame is set up.
+    static const struct { const char *api, *stem; int dtype; } kExtended[] = {
+        {"run_flash_attn_fwd", "flash_attn_fwd", 1},         {"run_flash_attn_fwd_bf16", "flash_attn_fwd", 2},
+        {"run_flash_attn_bwd", "flash_attn_bwd", 1},         {"run_flash_attn_bwd_bf16", "flash_attn_bwd", 2},
+        {"run_flash_attn_kvcache", "flash_attn_kvcache", 1}, {"run_flash_attn_kvcache_bf16", "flash_attn_kvcache", 2}};
+    for (const auto &c : kExtended) {
       if (api_name != c.api) continue;
-      checked_ = reinterpret_cast<CheckedFn>(dlsym(handle_, c.checked));
+      const std::string stem(c.stem);
+      with_ws_ = reinterpret_cast<WsFn>(dlsym(handle_, (stem + "_ws").c_str()));
       last_error_ = reinterpret_cast<LastErrorFn>(dlsym(handle_, "flash_attn_last_error"));
-      checked_dtype_ = c.dtype;
+      is_bwd_ = stem == "flash_attn_bwd";
+      if (is_bwd_) bwd_bytes_ = reinterpret_cast<BwdBytesFn>(dlsym(handle_, (stem + "_workspace_bytes").c_str()));
+      else bytes_ = reinterpret_cast<BytesFn>(dlsym(handle_, (stem + "_workspace_bytes").c_str()));
+      ext_dtype_ = c.dtype;
     }
+    if (!with_ws_ || !last_error_ || (!bytes_ && !bwd_bytes_)) with_ws_ = nullptr;  // all or nothing
+  }
+  size_t GetWorkspaceSize(const ExecutionContext &) const override {
+    if (!with_ws_) return 0;
+    OpAccessor acc(info_);
+    void *extra = acc.GetAttrAsVoidPtr("extra_args");
+    size_t n = 0;
+    if (is_bwd_) {  // operand 11 is dq_accum (flash_api.cu:696-725): the library fills it first
+      const size_t accum = acc.GetNumArgs() > 11 ? (size_t)LinearizedShape(acc.GetArgShape(11)) * GetDTypeByte(acc.GetArgDTypeEnum(11)) : 0;
+      n = bwd_bytes_(extra, ext_dtype_, accum);
+    } else {
+      n = bytes_(extra, ext_dtype_);
+    }
+    std::free(extra);
+    return n;
   }
   common::Status RunImpl(const ExecutionContext &ctx) override {
     OpAccessor acc(info_, ctx.exec_frame);
@@ -217,8 +241,8 @@ public:
     for (size_t i = 0; i < tensors.size(); ++i) tensors[i] = acc.GetArgAsyncValueRef(i);
     void *extra = acc.GetAttrAsVoidPtr("extra_args");
     common::Status st = common::Status::OK();
-    if (checked_ && last_error_) {
-      const int e = checked_(tensors.data(), extra, checked_dtype_, StreamOf(ctx));
+    if (with_ws_) {
+      const int e = with_ws_(tensors.data(), extra, ext_dtype_, GetWorkspace(ctx), GetWorkspaceSize(ctx), StreamOf(ctx));
       if (e < 0) st = common::Status::Fail(std::string("custom op: ") + last_error_());
       else if (e > 0) st = HipStatus(e, "custom op launch");
     } else {
@@ -230,7 +254,9 @@ public:
 
 private:
   using RunFn = void (*)(void **, void *, void *);
-  using CheckedFn = int (*)(void **, const void *, int, void *);
+  using WsFn = int (*)(void **, const void *, int, void *, size_t, void *);
+  using BytesFn = size_t (*)(const void *, int);
+  using BwdBytesFn = size_t (*)(const void *, int, size_t);
   using LastErrorFn = const char *(*)();
   static void *Open(const std::string &path) {
     if (void *h = dlopen(path.c_str(), RTLD_LAZY | RTLD_GLOBAL)) return h;
@@ -247,9 +273,12 @@ private:
   }
   void *handle_ = nullptr;
   RunFn run_ = nullptr;
-  CheckedFn checked_ = nullptr;
+  WsFn with_ws_ = nullptr;
+  BytesFn bytes_ = nullptr;
+  BwdBytesFn bwd_bytes_ = nullptr;
   LastErrorFn last_error_ = nullptr;
-  int checked_dtype_ = 0;
+  bool is_bwd_ = false;
+  int ext_dtype_ = 0;
 };
 
 // ---- copies: cpu2cuda, cuda2cpu, cuda2cuda (operands: src, dst) ---------------------------------------------

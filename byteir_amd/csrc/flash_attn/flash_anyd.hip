@@ -683,6 +683,7 @@ hipError_t bwd_anyd_d(const Params &p, hipStream_t stream) {
     pk.dv_bs = p.v_bs; pk.dv_rs = p.v_rs; pk.dv_hs = p.v_hs;
     pk.gsplit = pk.qsplit = 1;
     const GroupSplit split = plan_group_split(p, (int64_t)p.n_nblocks * p.b * p.h_k, 256 * (DR <= 64 ? 2 : 1), p.d, kTile, stream);
+    if (p.ws_query) return hipSuccess;  // planning only
     apply_group_split(pk, p, split, p.d);
     pk.xcd_remap = ((p.b * pk.h_k) % 8 == 0) ? (p.wr >= 0 ? 2 : 1) : (p.wr >= 0 ? 3 : 0);
     const dim3 gks((unsigned)(p.n_nblocks * p.b * pk.h_k));
@@ -693,7 +694,7 @@ hipError_t bwd_anyd_d(const Params &p, hipStream_t stream) {
       if (e != hipSuccess) return e;
     }
   }
-  if (p.n_mblocks > 0) {
+  if (p.n_mblocks > 0 && !p.ws_query) {
     if (p.drop) dq_anyd_kernel<T, DR, true><<<gq, block, 0, stream>>>(p);
     else dq_anyd_kernel<T, DR, false><<<gq, block, 0, stream>>>(p);
   }
@@ -713,7 +714,7 @@ hipError_t fwd_anyd_t(const Params &p, hipStream_t stream) {
 template <typename T>
 hipError_t bwd_anyd_t(const Params &p, hipStream_t stream) {
   const int64_t rows = (int64_t)p.b * p.h * p.sq;
-  if (rows > 0) dot_do_o_anyd_kernel<T><<<dim3((unsigned)((rows + 7) / 8)), dim3(256), 0, stream>>>(p);
+  if (rows > 0 && !p.ws_query) dot_do_o_anyd_kernel<T><<<dim3((unsigned)((rows + 7) / 8)), dim3(256), 0, stream>>>(p);
   if (p.d <= 32) return bwd_anyd_d<T, 32>(p, stream);
   if (p.d <= 64) return bwd_anyd_d<T, 64>(p, stream);
   if (p.d <= 96) return bwd_anyd_d<T, 96>(p, stream);
@@ -727,7 +728,7 @@ hipError_t bwd_anyd_t(const Params &p, hipStream_t stream) {
 hipError_t launch_fwd_anyd(Params &p, int dtype, hipStream_t stream) {
   if (p.d <= 0 || p.d > 256 || p.d % 8 != 0) return hipErrorInvalidValue;
   p.n_mblocks = (p.sq + kRows - 1) / kRows;
-  if (p.n_mblocks == 0) return hipSuccess;
+  if (p.n_mblocks == 0 || p.ws_query) return hipSuccess;  // this path takes no scratch
   return dtype == 1 ? fwd_anyd_t<_Float16>(p, stream) : fwd_anyd_t<__bf16>(p, stream);
 }
 

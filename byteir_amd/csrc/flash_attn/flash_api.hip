@@ -134,12 +134,24 @@ const char *VERSION = "2.5.3";
 
 const char *flash_attn_last_error(void) { return g_err; }
 
-int flash_attn_fwd_checked(void **tensors, const void *extra_args, int dtype, void *stream) {
-  if (!tensors || !extra_args) return fail("null argument");
+}  // extern "C"
+
+namespace {
+// What every entry point funnels into.  query != nullptr: planning only (tensors may be null),
+// *query receives the scratch the same call would take.
+struct Scratch { void *ws; size_t ws_bytes; size_t *query; };
+
+int fwd_impl(void **tensors, const void *extra_args, int dtype, const Scratch &sc, void *stream) {
+  if ((!tensors && !sc.query) || !extra_args) return fail("null argument");
   if (dtype != 1 && dtype != 2) return fail("dtype %d is not supported (1 = fp16, 2 = bf16)", dtype);
   const Blob a = parse(extra_args);
   fa::Params p{};
   if (int r = fill(a, p)) return r;
+  p.ws = sc.ws; p.ws_bytes = sc.ws_bytes; p.ws_query = sc.query;
+  if (sc.query) {
+    *sc.query = 0;
+    return p.b == 0 || p.sq == 0 ? 0 : fa::launch_fwd(p, dtype, nullptr);
+  }
   // tensors: q, k, v, rng_state, o, softmax_lse, softmax_P
   p.q = tensors[0]; p.k = tensors[1]; p.v = tensors[2];
   p.rng_state = static_cast<const uint64_t *>(tensors[3]);
@@ -153,13 +165,21 @@ int flash_attn_fwd_checked(void **tensors, const void *extra_args, int dtype, vo
   return fa::launch_fwd(p, dtype, static_cast<hipStream_t>(stream));
 }
 
-int flash_attn_bwd_checked(void **tensors, const void *extra_args, int dtype, void *stream) {
-  if (!tensors || !extra_args) return fail("null argument");
+// dq_accum_bytes: only read when planning (the size of the dq_accum tensor the call will get)
+int bwd_impl(void **tensors, const void *extra_args, int dtype, const Scratch &sc, size_t dq_accum_bytes, void *stream) {
+  if ((!tensors && !sc.query) || !extra_args) return fail("null argument");
   if (dtype != 1 && dtype != 2) return fail("dtype %d is not supported (1 = fp16, 2 = bf16)", dtype);
   const Blob a = parse(extra_args);
   fa::Params p{};
   if (int r = fill(a, p)) return r;
   if (a.seqlen_q_rounded < a.seqlen_q) return fail("seqlen_q_rounded < seqlen_q");
+  p.ws = sc.ws; p.ws_bytes = sc.ws_bytes; p.ws_query = sc.query;
+  if (sc.query) {
+    *sc.query = 0;
+    p.dq_accum = dq_accum_bytes ? reinterpret_cast<void *>(uintptr_t(256)) : nullptr;  // never dereferenced when planning
+    p.dq_accum_bytes = dq_accum_bytes;
+    return p.b == 0 ? 0 : fa::launch_bwd(p, dtype, nullptr);
+  }
   // tensors: dout, q, k, v, out, softmax_lse, rng_state, dq, dk, dv, d_softmax, dq_accum
   p.dout = tensors[0]; p.q = tensors[1]; p.k = tensors[2]; p.v = tensors[3]; p.o = tensors[4];
   p.lse = static_cast<float *>(tensors[5]);
@@ -184,8 +204,8 @@ int flash_attn_bwd_checked(void **tensors, const void *extra_args, int dtype, vo
   return fa::launch_bwd(p, dtype, static_cast<hipStream_t>(stream));
 }
 
-int flash_attn_kvcache_checked(void **tensors, const void *extra_args, int dtype, void *stream_) {
-  if (!tensors || !extra_args) return fail("null argument");
+int kvcache_impl(void **tensors, const void *extra_args, int dtype, const Scratch &sc, void *stream_) {
+  if ((!tensors && !sc.query) || !extra_args) return fail("null argument");
   if (dtype != 1 && dtype != 2) return fail("dtype %d is not supported (1 = fp16, 2 = bf16)", dtype);
   hipStream_t stream = static_cast<hipStream_t>(stream_);
   const KvBlob k = parse_kv(extra_args);
@@ -201,6 +221,11 @@ int flash_attn_kvcache_checked(void **tensors, const void *extra_args, int dtype
   a.window_size_left = k.window_size_left; a.window_size_right = k.window_size_right;
   fa::Params p{};
   if (int r = fill(a, p)) return r;
+  p.ws = sc.ws; p.ws_bytes = sc.ws_bytes; p.ws_query = sc.query;
+  if (sc.query) {  // the split depends on the cache capacity, not on seqlens_k
+    *sc.query = 0;
+    return p.b == 0 || p.sq == 0 ? 0 : fa::launch_fwd(p, dtype, nullptr);
+  }
   // tensors: q, k cache, v cache, k new, v new, seqlens_k, o, softmax_lse (flash_api.cu:775-777)
   p.q = tensors[0]; p.k = tensors[1]; p.v = tensors[2];
   p.k_new = tensors[3]; p.v_new = tensors[4];
@@ -227,6 +252,41 @@ int flash_attn_kvcache_checked(void **tensors, const void *extra_args, int dtype
   }
   // without seqlens_k every batch attends to all seqlen_k cache rows (BlockInfo, block_info.h:27-37)
   return fa::launch_fwd(p, dtype, stream);
+}
+
+}  // namespace
+
+extern "C" {
+
+int flash_attn_fwd_checked(void **tensors, const void *extra_args, int dtype, void *stream) {
+  return fwd_impl(tensors, extra_args, dtype, Scratch{nullptr, 0, nullptr}, stream);
+}
+int flash_attn_bwd_checked(void **tensors, const void *extra_args, int dtype, void *stream) {
+  return bwd_impl(tensors, extra_args, dtype, Scratch{nullptr, 0, nullptr}, 0, stream);
+}
+int flash_attn_kvcache_checked(void **tensors, const void *extra_args, int dtype, void *stream) {
+  return kvcache_impl(tensors, extra_args, dtype, Scratch{nullptr, 0, nullptr}, stream);
+}
+int flash_attn_fwd_ws(void **tensors, const void *extra_args, int dtype, void *workspace, size_t workspace_bytes, void *stream) {
+  return fwd_impl(tensors, extra_args, dtype, Scratch{workspace, workspace_bytes, nullptr}, stream);
+}
+int flash_attn_bwd_ws(void **tensors, const void *extra_args, int dtype, void *workspace, size_t workspace_bytes, void *stream) {
+  return bwd_impl(tensors, extra_args, dtype, Scratch{workspace, workspace_bytes, nullptr}, 0, stream);
+}
+int flash_attn_kvcache_ws(void **tensors, const void *extra_args, int dtype, void *workspace, size_t workspace_bytes, void *stream) {
+  return kvcache_impl(tensors, extra_args, dtype, Scratch{workspace, workspace_bytes, nullptr}, stream);
+}
+size_t flash_attn_fwd_workspace_bytes(const void *extra_args, int dtype) {
+  size_t n = 0;
+  return fwd_impl(nullptr, extra_args, dtype, Scratch{nullptr, 0, &n}, nullptr) == 0 ? n : 0;
+}
+size_t flash_attn_bwd_workspace_bytes(const void *extra_args, int dtype, size_t dq_accum_bytes) {
+  size_t n = 0;
+  return bwd_impl(nullptr, extra_args, dtype, Scratch{nullptr, 0, &n}, dq_accum_bytes, nullptr) == 0 ? n : 0;
+}
+size_t flash_attn_kvcache_workspace_bytes(const void *extra_args, int dtype) {
+  size_t n = 0;
+  return kvcache_impl(nullptr, extra_args, dtype, Scratch{nullptr, 0, &n}, nullptr) == 0 ? n : 0;
 }
 
 static void die(const char *who, int r) {

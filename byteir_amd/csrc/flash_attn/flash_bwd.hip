@@ -788,7 +788,7 @@ __global__ void __launch_bounds__(256) group_sum_kernel(const Params p, const vo
 template <typename T, int D>
 hipError_t launch_bwd_td(const Params &p, hipStream_t stream) {
   const int64_t rows = (int64_t)p.b * p.h * p.sq;
-  if (rows > 0) {
+  if (rows > 0 && !p.ws_query) {
     constexpr int RPB = 256 / (D / 8);
     dot_do_o_kernel<T, D><<<dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(256), 0, stream>>>(p);
   }
@@ -804,6 +804,7 @@ hipError_t launch_bwd_td(const Params &p, hipStream_t stream) {
   pk.gsplit = pk.qsplit = 1;
   // chip slots for this kernel: 256 CUs, two workgroups each up to head_dim 64
   const GroupSplit split = plan_group_split(p, (int64_t)pk.n_nblocks * p.b * p.h_k, 256 * (D <= 64 ? 2 : 1), D, kQTile, stream);
+  if (p.ws_query) return hipSuccess;  // planning only
   apply_group_split(pk, p, split, D);
   pk.xcd_remap = ((p.b * pk.h_k) % 8 == 0) ? (p.wr >= 0 ? 2 : 1) : (p.wr >= 0 ? 3 : 0);
   if (pk.n_nblocks > 0)

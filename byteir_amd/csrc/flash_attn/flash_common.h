@@ -179,6 +179,14 @@ struct Params {
   float *o_part;                      // [n_splits][b][h][sq][d]
   float *ml_part;                     // [n_splits][b][h][sq][2]: reference maximum, row sum
   int n_splits, split_tiles;
+  // Scratch for the partial results above and for the backward's partial dK / dV: the caller's
+  // workspace when the call came through a flash_attn_*_ws entry point and it is large enough,
+  // else a stream-ordered allocation of the library's own.  ws_query != nullptr is the
+  // planning mode behind flash_attn_*_workspace_bytes: the launch code runs up to the point
+  // where it would take scratch, writes the size there and returns without launching anything.
+  void *ws;
+  size_t ws_bytes;
+  size_t *ws_query;
   // dropout (forward and backward calls): rng_state = {seed, offset} in device memory,
   // keep probability, its reciprocal and its 8-bit threshold floor(p_keep * 255)
   const uint64_t *rng_state;
@@ -209,7 +217,8 @@ hipError_t launch_dq_anyd128(const Params &p, int dtype, hipStream_t stream);
 // key/value head and key block leaves most CUs idle, so the query heads of a group are shared
 // out over `gs` workgroups that write float partials [b, sk, h_k * gs, row] of dK / dV, which
 // launch_group_sum adds (and rounds once).  The partials take the caller's dq_accum scratch as
-// far as it reaches, a stream-ordered allocation for the rest.
+// far as it reaches; the rest goes to the caller's workspace (flash_attn_bwd_ws) or, without
+// one, to a stream-ordered allocation.
 struct GroupSplit {
   int gs = 1;             // shares of a group's query heads; 1: no split
   int qs = 1;             // shares of a key block's query tiles on top of that
@@ -249,16 +258,19 @@ inline GroupSplit plan_group_split(const Params &p, int64_t base_wg, int slots, 
   if (gs * qs == 1) return r;
   const size_t one = (size_t)p.b * p.sk * p.h_k * gs * qs * row * sizeof(float);
   const bool usable = p.dq_accum && (reinterpret_cast<uintptr_t>(p.dq_accum) & 15) == 0;
-  if (usable && p.dq_accum_bytes >= 2 * one) {
-    r.dk = p.dq_accum;
-    r.dv = static_cast<char *>(p.dq_accum) + one;
-  } else if (usable && p.dq_accum_bytes >= one) {
-    if (hipMallocAsync(&r.owned, one, stream) == hipSuccess) { r.dk = p.dq_accum; r.dv = r.owned; }
-  } else if (hipMallocAsync(&r.owned, 2 * one, stream) == hipSuccess) {
-    r.dk = r.owned;
-    r.dv = static_cast<char *>(r.owned) + one;
+  const size_t in_accum = !usable ? 0 : p.dq_accum_bytes >= 2 * one ? 2 * one : p.dq_accum_bytes >= one ? one : 0;
+  const size_t need = 2 * one - in_accum;  // beyond what dq_accum holds
+  if (p.ws_query) { *p.ws_query = need; return r; }
+  char *extra = nullptr;
+  if (need) {
+    if (p.ws && (reinterpret_cast<uintptr_t>(p.ws) & 15) == 0 && p.ws_bytes >= need) extra = static_cast<char *>(p.ws);
+    else if (hipMallocAsync(&r.owned, need, stream) == hipSuccess) extra = static_cast<char *>(r.owned);
+    else { (void)hipGetLastError(); r.owned = nullptr; return r; }  // no scratch: no split
   }
-  if (!r.dk) { (void)hipGetLastError(); r.owned = nullptr; return r; }  // no scratch: no split
+  char *accum = static_cast<char *>(p.dq_accum);
+  if (in_accum == 2 * one) { r.dk = accum; r.dv = accum + one; }
+  else if (in_accum == one) { r.dk = accum; r.dv = extra; }
+  else { r.dk = extra; r.dv = extra + one; }
   r.gs = gs;
   r.qs = qs;
   return r;

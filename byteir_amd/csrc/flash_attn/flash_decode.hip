@@ -271,11 +271,15 @@ hipError_t decode_td(const Params &p, hipStream_t stream) {
   a.n_splits = n_splits;
   a.chunk = ((p.sk + n_splits - 1) / n_splits + kUnit * kDecWaves - 1) / (kUnit * kDecWaves) * (kUnit * kDecWaves);
   void *ws = nullptr;
+  bool owned = false;
   const size_t rows = (size_t)p.b * p.h * p.sq;
-  if (n_splits > 1) {
-    if (hipMallocAsync(&ws, (size_t)n_splits * rows * (D + 2) * sizeof(float), stream) != hipSuccess) {
-      (void)hipGetLastError();  // no workspace: one chunk per (batch, key/value head)
-      ws = nullptr;
+  const size_t need = n_splits > 1 ? (size_t)n_splits * rows * (D + 2) * sizeof(float) : 0;
+  if (p.ws_query) { *p.ws_query = need; return hipSuccess; }
+  if (need) {
+    if (p.ws && (reinterpret_cast<uintptr_t>(p.ws) & 15) == 0 && p.ws_bytes >= need) ws = p.ws;
+    else if (hipMallocAsync(&ws, need, stream) == hipSuccess) owned = true;
+    else { (void)hipGetLastError(); ws = nullptr; }
+    if (!ws) {  // no scratch: one chunk per (batch, key/value head)
       a.n_splits = 1;
       a.chunk = (p.sk + kUnit - 1) / kUnit * kUnit;
     } else {
@@ -290,8 +294,10 @@ hipError_t decode_td(const Params &p, hipStream_t stream) {
       decode_merge_kernel<T, D><<<dim3((unsigned)rows), dim3(D < 64 ? 64 : D), 0, stream>>>(p, a);
       e = hipGetLastError();
     }
-    const hipError_t f = hipFreeAsync(ws, stream);
-    if (e == hipSuccess) e = f;
+    if (owned) {
+      const hipError_t f = hipFreeAsync(ws, stream);
+      if (e == hipSuccess) e = f;
+    }
   }
   return e;
 }

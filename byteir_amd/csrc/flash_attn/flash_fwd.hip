@@ -445,20 +445,26 @@ hipError_t launch_fwd_d(Params &p, hipStream_t stream) {
   // Few query blocks and many keys (a long prompt chunk of one sequence): split the key axis over
   // workgroups until the chip is full, at least eight tiles per split (the reference's
   // num_splits_heuristic has the same aim, flash_api.cu:118-160, but its entry points never
-  // enable it).  The partials live in a stream-ordered allocation; without it: one split.
+  // enable it).  The partials live in the caller's workspace or, without one, in a
+  // stream-ordered allocation; with neither: one split.
   const int n_wg = p.n_mblocks * p.b * p.h, n_tiles = (p.sk + kBN - 1) / kBN;
   const int n_splits = pick_splits(n_wg, n_tiles);
   void *ws = nullptr;
+  bool owned = false;
   const size_t rows = (size_t)p.b * p.h * p.sq;
+  const size_t need = n_splits > 1 ? (size_t)n_splits * rows * (D + 2) * sizeof(float) : 0;
+  if (p.ws_query) { *p.ws_query = need; return hipSuccess; }
   p.n_splits = 1;
-  if (n_splits > 1 && hipMallocAsync(&ws, (size_t)n_splits * rows * (D + 2) * sizeof(float), stream) == hipSuccess) {
+  if (need) {
+    if (p.ws && (reinterpret_cast<uintptr_t>(p.ws) & 15) == 0 && p.ws_bytes >= need) ws = p.ws;
+    else if (hipMallocAsync(&ws, need, stream) == hipSuccess) owned = true;
+    else { (void)hipGetLastError(); ws = nullptr; }  // no scratch: one split
+  }
+  if (ws) {
     p.n_splits = n_splits;
     p.split_tiles = (n_tiles + n_splits - 1) / n_splits;
     p.o_part = static_cast<float *>(ws);
     p.ml_part = p.o_part + (size_t)n_splits * rows * D;
-  } else if (n_splits > 1) {
-    (void)hipGetLastError();
-    ws = nullptr;
   }
   const dim3 grid((unsigned)n_wg, (unsigned)p.n_splits), block(NW * 64);
   if (p.seqlens_k) flash_fwd_kernel<T, D, QB, NW, true><<<grid, block, 0, stream>>>(p);
@@ -466,8 +472,10 @@ hipError_t launch_fwd_d(Params &p, hipStream_t stream) {
   hipError_t e = hipGetLastError();
   if (ws) {
     if (e == hipSuccess) e = launch_split_merge(p, std::is_same<T, _Float16>::value ? 1 : 2, stream);
-    const hipError_t fr = hipFreeAsync(ws, stream);
-    if (e == hipSuccess) e = fr;
+    if (owned) {
+      const hipError_t fr = hipFreeAsync(ws, stream);
+      if (e == hipSuccess) e = fr;
+    }
   }
   return e;
 }

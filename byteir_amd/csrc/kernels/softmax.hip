@@ -533,8 +533,11 @@ softmax_inner_kernel(const T *__restrict__ in, T *__restrict__ out, uint64_t B, 
   }
 }
 
+// ws / ws_bytes: the caller's scratch for the segment partials (may be null); query: when not
+// null nothing is launched and the scratch size for 16-byte aligned tensors is written there.
 template <typename T>
-hipError_t run_inner(const T *in, T *out, uint64_t A, uint64_t B, uint64_t C, hipStream_t stream) {
+hipError_t run_inner(const T *in, T *out, uint64_t A, uint64_t B, uint64_t C, void *ws, size_t ws_bytes, size_t *query,
+                     hipStream_t stream) {
   constexpr int EPV = Elem<T>::EPV;
   const bool vec = C % EPV == 0 && ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15u) == 0;
   const uint64_t ncolv = vec ? C / EPV : C;
@@ -556,11 +559,18 @@ hipError_t run_inner(const T *in, T *out, uint64_t A, uint64_t B, uint64_t C, hi
   uint64_t seg_rows = ((B + S - 1) / S + ty - 1) / ty * ty;
   S = (B + seg_rows - 1) / seg_rows;
   float *part = nullptr;
-  if (S > 1 && hipMallocAsync(reinterpret_cast<void **>(&part), A * S * C * 2 * sizeof(float), stream) != hipSuccess) {
-    (void)hipGetLastError();  // no workspace: one workgroup per column tile
-    part = nullptr;
-    S = 1;
-    seg_rows = B;
+  bool owned = false;
+  const size_t need = S > 1 ? (size_t)(A * S * C * 2) * sizeof(float) : 0;
+  if (query) { *query = need; return hipSuccess; }
+  if (need) {
+    if (ws && (reinterpret_cast<uintptr_t>(ws) & 15u) == 0 && ws_bytes >= need) part = static_cast<float *>(ws);
+    else if (hipMallocAsync(reinterpret_cast<void **>(&part), need, stream) == hipSuccess) owned = true;
+    else {
+      (void)hipGetLastError();  // no scratch: one workgroup per column tile
+      part = nullptr;
+      S = 1;
+      seg_rows = B;
+    }
   }
   if (col_tiles > 0xffffffffull || A * col_tiles * S > 0x7fffffffull) return hipErrorInvalidValue;
   const dim3 grid((unsigned)(A * col_tiles * S)), block(kBlock);
@@ -577,8 +587,10 @@ hipError_t run_inner(const T *in, T *out, uint64_t A, uint64_t B, uint64_t C, hi
       if (vec) INNER_TX(EPV, 2); else INNER_TX(1, 2);
       e = hipGetLastError();
     }
-    const hipError_t f = hipFreeAsync(part, stream);
-    if (e == hipSuccess) e = f;
+    if (owned) {
+      const hipError_t f = hipFreeAsync(part, stream);
+      if (e == hipSuccess) e = f;
+    }
   }
 #undef INNER_TX
 #undef INNER
@@ -633,22 +645,38 @@ hipError_t run(const T *in, T *out, uint64_t rows, uint64_t cols, hipStream_t st
 
 }  // namespace
 
-extern "C" int brt_rocm_softmax_axis(int dtype, const void *input, void *output, size_t A, size_t B,
-                                     size_t C, void *stream_) {
-  if (C == 1) return brt_rocm_softmax(dtype, input, output, A, B, stream_);
+namespace {
+int softmax_axis_impl(int dtype, const void *input, void *output, size_t A, size_t B, size_t C, void *ws, size_t ws_bytes,
+                      size_t *query, void *stream_) {
   hipStream_t stream = static_cast<hipStream_t>(stream_);
+  if (query) *query = 0;
+  if (C == 1) return query ? hipSuccess : brt_rocm_softmax(dtype, input, output, A, B, stream_);
   if (A == 0 || B == 0 || C == 0) return hipSuccess;
-  if (!input || !output) return hipErrorInvalidValue;
+  if (!query && (!input || !output)) return hipErrorInvalidValue;
   switch (dtype) {
   case BRT_ROCM_F32:
-    return run_inner(static_cast<const float *>(input), static_cast<float *>(output), A, B, C, stream);
+    return run_inner(static_cast<const float *>(input), static_cast<float *>(output), A, B, C, ws, ws_bytes, query, stream);
   case BRT_ROCM_F16:
-    return run_inner(static_cast<const __half *>(input), static_cast<__half *>(output), A, B, C, stream);
+    return run_inner(static_cast<const __half *>(input), static_cast<__half *>(output), A, B, C, ws, ws_bytes, query, stream);
   case BRT_ROCM_BF16:
-    return run_inner(static_cast<const __bf16 *>(input), static_cast<__bf16 *>(output), A, B, C, stream);
+    return run_inner(static_cast<const __bf16 *>(input), static_cast<__bf16 *>(output), A, B, C, ws, ws_bytes, query, stream);
   default:
     return hipErrorInvalidValue;
   }
+}
+}  // namespace
+
+extern "C" int brt_rocm_softmax_axis(int dtype, const void *input, void *output, size_t A, size_t B,
+                                     size_t C, void *stream) {
+  return softmax_axis_impl(dtype, input, output, A, B, C, nullptr, 0, nullptr, stream);
+}
+extern "C" int brt_rocm_softmax_axis_ws(int dtype, const void *input, void *output, size_t A, size_t B, size_t C,
+                                        void *workspace, size_t workspace_bytes, void *stream) {
+  return softmax_axis_impl(dtype, input, output, A, B, C, workspace, workspace_bytes, nullptr, stream);
+}
+extern "C" size_t brt_rocm_softmax_workspace_bytes(int dtype, size_t A, size_t B, size_t C) {
+  size_t n = 0;
+  return softmax_axis_impl(dtype, nullptr, nullptr, A, B, C, nullptr, 0, &n, nullptr) == hipSuccess ? n : 0;
 }
 
 extern "C" int brt_rocm_softmax(int dtype, const void *input, void *output, size_t rows,

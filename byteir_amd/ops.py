@@ -101,8 +101,20 @@ def reduce(op, x, dims, stream=None):
     return reduce_abc(op, x, out, A, B, C, stream=stream)
 
 
-def softmax(x, out=None, stream=None, axis=-1):
-    """byteir.softmax over `axis` of a dense tensor (the last one by default)."""
+def softmax_workspace_bytes(x, axis=-1):
+    """brt_rocm_softmax_workspace_bytes for softmax(x, axis=axis)."""
+    axis = axis % x.dim()
+    a, b, c = 1, x.shape[axis], 1
+    for n in x.shape[:axis]:
+        a *= n
+    for n in x.shape[axis + 1:]:
+        c *= n
+    return _lib.kernels().brt_rocm_softmax_workspace_bytes(_DT[x.dtype], a, b, c)
+
+
+def softmax(x, out=None, stream=None, axis=-1, workspace=None):
+    """byteir.softmax over `axis` of a dense tensor (the last one by default).  workspace: the
+    caller's scratch (uint8 device tensor of softmax_workspace_bytes) for the inner-axis split."""
     if out is None:
         out = torch.empty_like(x)
     axis = axis % x.dim()
@@ -111,6 +123,11 @@ def softmax(x, out=None, stream=None, axis=-1):
         a *= n
     for n in x.shape[axis + 1:]:
         c *= n
+    if workspace is not None:
+        _lib.check(_lib.kernels().brt_rocm_softmax_axis_ws(_DT[x.dtype], _dev(x), _dev(out), a, b, c, _dev(workspace),
+                                                           workspace.numel() * workspace.element_size(), _stream(stream)),
+                   "brt_rocm_softmax_axis_ws")
+        return out
     _lib.check(_lib.kernels().brt_rocm_softmax_axis(_DT[x.dtype], _dev(x), _dev(out), a, b, c,
                                                     _stream(stream)), "brt_rocm_softmax_axis")
     return out
@@ -142,13 +159,37 @@ def _call_custom(fn, tensors, blob, stream):
     fn(arr, ctypes.cast(buf, ctypes.c_void_p), _stream(stream))
 
 
+def _call_custom_ws(kind, dtype, tensors, blob, workspace, stream):
+    """flash_attn_<kind>_ws: the error-returning entry point with the caller's scratch
+    (`workspace`: a uint8 device tensor, or None)."""
+    L = _lib.flash_attn()
+    arr = (ctypes.c_void_p * len(tensors))(*[t.data_ptr() if t is not None else None for t in tensors])
+    buf = ctypes.create_string_buffer(blob, len(blob))
+    ws = ctypes.c_void_p(workspace.data_ptr()) if workspace is not None else None
+    n = workspace.numel() * workspace.element_size() if workspace is not None else 0
+    rc = getattr(L, f"flash_attn_{kind}_ws")(arr, ctypes.cast(buf, ctypes.c_void_p), 1 if dtype == torch.float16 else 2, ws, n, _stream(stream))
+    if rc < 0:
+        raise ValueError(L.flash_attn_last_error().decode())
+    _lib.check(rc, f"flash_attn_{kind}_ws")
+
+
+def flash_attn_workspace_bytes(kind, dtype, blob, dq_accum_bytes=0):
+    """flash_attn_{fwd,bwd,kvcache}_workspace_bytes for an extra_args blob."""
+    L = _lib.flash_attn()
+    buf = ctypes.create_string_buffer(blob, len(blob))
+    code = 1 if dtype == torch.float16 else 2
+    if kind == "bwd":
+        return L.flash_attn_bwd_workspace_bytes(ctypes.cast(buf, ctypes.c_void_p), code, dq_accum_bytes)
+    return getattr(L, f"flash_attn_{kind}_workspace_bytes")(ctypes.cast(buf, ctypes.c_void_p), code)
+
+
 def rng_state_tensor(seed, offset, device):
     """The rng_state operand of the attention calls: {seed, offset} as two 64-bit words."""
     to_i64 = lambda x: int(x) - (1 << 64) if int(x) >= (1 << 63) else int(x)
     return torch.tensor([to_i64(seed), to_i64(offset)], dtype=torch.int64, device=device)
 
 
-def flash_attn_fwd(q, k, v, scale, window=(-1, -1), stream=None, out=None, p_dropout=0.0, rng_state=None):
+def flash_attn_fwd(q, k, v, scale, window=(-1, -1), stream=None, out=None, p_dropout=0.0, rng_state=None, workspace=None):
     """run_flash_attn_fwd: tensors {q, k, v, rng_state, o, softmax_lse, softmax_P}
     (external_libs/runtime/flash_attn/lib/flash_api.cu:586-654). -> (o, lse[b,h,sq] f32).
     out: optional (o, lse, rng_state) to write into instead of allocating.
@@ -162,8 +203,12 @@ def flash_attn_fwd(q, k, v, scale, window=(-1, -1), stream=None, out=None, p_dro
         o = torch.empty_like(q)
         lse = torch.empty((b, h, sq), dtype=torch.float32, device=q.device)
         rng = rng_state if rng_state is not None else torch.zeros(2, dtype=torch.int64, device=q.device)
+    blob = pack_flash_args(q, k, v, o, scale, window, p_dropout)
+    if workspace is not None:  # the caller's scratch for the key-axis split (flash_attn_fwd_ws)
+        _call_custom_ws("fwd", q.dtype, [q, k, v, rng, o, lse, None], blob, workspace, stream)
+        return o, lse
     fn = L.run_flash_attn_fwd if q.dtype == torch.float16 else L.run_flash_attn_fwd_bf16
-    _call_custom(fn, [q, k, v, rng, o, lse, None], pack_flash_args(q, k, v, o, scale, window, p_dropout), stream)
+    _call_custom(fn, [q, k, v, rng, o, lse, None], blob, stream)
     return o, lse
 
 
@@ -181,7 +226,7 @@ def flash_attn_bwd_buffers(q, k, v):
 
 
 def flash_attn_bwd(dout, q, k, v, o, lse, scale, window=(-1, -1), stream=None, out=None, p_dropout=0.0,
-                   rng_state=None):
+                   rng_state=None, workspace=None):
     """run_flash_attn_bwd: tensors {dout, q, k, v, out, softmax_lse, rng_state, dq, dk, dv,
     d_softmax, dq_accum} (flash_api.cu:656-725). -> (dq, dk, dv).
     out: optional result of flash_attn_bwd_buffers to write into instead of allocating.
@@ -190,9 +235,12 @@ def flash_attn_bwd(dout, q, k, v, o, lse, scale, window=(-1, -1), stream=None, o
     dq, dk, dv, dsm, dq_accum, rng = out if out is not None else flash_attn_bwd_buffers(q, k, v)
     if rng_state is not None:
         rng = rng_state
+    blob = pack_flash_args(q, k, v, o, scale, window, p_dropout)
+    if workspace is not None:  # the caller's scratch for partial dK / dV (flash_attn_bwd_ws)
+        _call_custom_ws("bwd", q.dtype, [dout, q, k, v, o, lse, rng, dq, dk, dv, dsm, dq_accum], blob, workspace, stream)
+        return dq, dk, dv
     fn = L.run_flash_attn_bwd if q.dtype == torch.float16 else L.run_flash_attn_bwd_bf16
-    _call_custom(fn, [dout, q, k, v, o, lse, rng, dq, dk, dv, dsm, dq_accum],
-                 pack_flash_args(q, k, v, o, scale, window, p_dropout), stream)
+    _call_custom(fn, [dout, q, k, v, o, lse, rng, dq, dk, dv, dsm, dq_accum], blob, stream)
     return dq, dk, dv
 
 
@@ -212,7 +260,7 @@ def pack_flash_kvcache_args(q, kcache, vcache, knew, vnew, o, scale, window):
     return struct.pack("<24q", *ints1) + struct.pack("<f", scale) + struct.pack("<6q", *ints2)
 
 
-def flash_attn_kvcache(q, kcache, vcache, knew, vnew, seqlens_k, scale, window=(-1, -1), stream=None):
+def flash_attn_kvcache(q, kcache, vcache, knew, vnew, seqlens_k, scale, window=(-1, -1), stream=None, workspace=None):
     """run_flash_attn_kvcache: tensors {q, k_cache, v_cache, k_new, v_new, seqlens_k, o,
     softmax_lse} (flash_api.cu:727-811).  Appends knew / vnew to the caches IN PLACE at row
     seqlens_k[b], then attends to the first seqlens_k[b] + seqlen_knew rows of each batch.
@@ -221,7 +269,10 @@ def flash_attn_kvcache(q, kcache, vcache, knew, vnew, seqlens_k, scale, window=(
     b, sq, h, d = q.shape
     o = torch.empty_like(q)
     lse = torch.empty((b, h, sq), dtype=torch.float32, device=q.device)
+    blob = pack_flash_kvcache_args(q, kcache, vcache, knew, vnew, o, scale, window)
+    if workspace is not None:
+        _call_custom_ws("kvcache", q.dtype, [q, kcache, vcache, knew, vnew, seqlens_k, o, lse], blob, workspace, stream)
+        return o, lse
     fn = L.run_flash_attn_kvcache if q.dtype == torch.float16 else L.run_flash_attn_kvcache_bf16
-    _call_custom(fn, [q, kcache, vcache, knew, vnew, seqlens_k, o, lse],
-                 pack_flash_kvcache_args(q, kcache, vcache, knew, vnew, o, scale, window), stream)
+    _call_custom(fn, [q, kcache, vcache, knew, vnew, seqlens_k, o, lse], blob, stream)
     return o, lse

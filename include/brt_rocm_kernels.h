@@ -157,6 +157,13 @@ int brt_rocm_softmax(int dtype, const void *input, void *output, size_t rows, si
  * back to one workgroup per column tile if that fails. */
 int brt_rocm_softmax_axis(int dtype, const void *input, void *output, size_t A, size_t B, size_t C,
                           void *stream);
+/* The same with the scratch supplied by the caller (the op kernel's per-frame workspace, asked
+ * and allocated where the reference's kernels ask for theirs, op_kernel_impl_base.h:116-149):
+ * brt_rocm_softmax_workspace_bytes is what the call takes for 16-byte aligned tensors (0: none);
+ * a NULL, misaligned or too small workspace falls back to the stream-ordered allocation. */
+size_t brt_rocm_softmax_workspace_bytes(int dtype, size_t A, size_t B, size_t C);
+int brt_rocm_softmax_axis_ws(int dtype, const void *input, void *output, size_t A, size_t B, size_t C,
+                             void *workspace, size_t workspace_bytes, void *stream);
 
 #ifdef __cplusplus
 }

@@ -37,6 +37,8 @@
 #ifndef BYTEIR_AMD_FLASH_API_H_
 #define BYTEIR_AMD_FLASH_API_H_
 
+#include <stddef.h>
+
 #ifdef __cplusplus
 extern "C" {
 #endif
@@ -90,6 +92,23 @@ int flash_attn_fwd_checked(void **tensors, const void *extra_args, int dtype, vo
 int flash_attn_bwd_checked(void **tensors, const void *extra_args, int dtype, void *stream);
 int flash_attn_kvcache_checked(void **tensors, const void *extra_args, int dtype, void *stream);
 const char *flash_attn_last_error(void);
+
+/* The same calls with their scratch supplied by the caller, for hosts that own all device
+ * memory (the runtime's per-frame workspace: the op kernel asks the size when a frame is set
+ * up and allocates through the frame's allocator, as the reference's kernels do for their
+ * workspaces, framework/op_kernel_impl_base.h:116-149; the reference library itself has no
+ * scratch because it never splits).  *_workspace_bytes returns what the call with this blob
+ * would take -- partial results of a key axis split over workgroups (forward, cache decode),
+ * partial dK / dV beyond what a dq_accum tensor of `dq_accum_bytes` holds (backward) -- and 0
+ * when it takes none or the blob is not supported; the size depends on the blob only.  The
+ * *_ws calls use `workspace` when it is 16-byte aligned and at least that large, and fall back
+ * to a stream-ordered allocation of their own otherwise (as the plain calls always do). */
+size_t flash_attn_fwd_workspace_bytes(const void *extra_args, int dtype);
+size_t flash_attn_bwd_workspace_bytes(const void *extra_args, int dtype, size_t dq_accum_bytes);
+size_t flash_attn_kvcache_workspace_bytes(const void *extra_args, int dtype);
+int flash_attn_fwd_ws(void **tensors, const void *extra_args, int dtype, void *workspace, size_t workspace_bytes, void *stream);
+int flash_attn_bwd_ws(void **tensors, const void *extra_args, int dtype, void *workspace, size_t workspace_bytes, void *stream);
+int flash_attn_kvcache_ws(void **tensors, const void *extra_args, int dtype, void *workspace, size_t workspace_bytes, void *stream);
 
 #ifdef __cplusplus
 }
