@@ -437,6 +437,38 @@ def _sampled_forward_check(q, k, v, o, lse, scale, window, code, n_rows, seed):
         assert abs(lf[bi, hi, i] - (m + np.log(e.sum()))) <= ATOL
 
 
+def _rows_forward_check_f64(q, k, v, o, lse, scale, causal, bi, heads, rows):
+    """O and LSE of the given query rows of batch bi, for every head in `heads`, against the
+    closed form in float64 (computed with torch on the GPU: plumbing for a 512 x seqlen_k matrix
+    per head).  -> (worst |O - ref|, worst |LSE - ref|)."""
+    sq, sk = q.shape[1], k.shape[1]
+    idx = torch.as_tensor(rows, device=q.device)
+    worst_o = worst_l = 0.0
+    for hi in heads:
+        hk = hi // (q.shape[2] // k.shape[2])
+        S = (q[bi, idx, hi].double() @ k[bi, :, hk].double().T) * scale
+        if causal:
+            S = S.masked_fill(torch.arange(sk, device=q.device)[None, :] > (idx + sk - sq)[:, None], float("-inf"))
+        L = torch.logsumexp(S, dim=-1)
+        O = torch.softmax(S, dim=-1) @ v[bi, :, hk].double()
+        worst_o = max(worst_o, float((o[bi, idx, hi].double() - O).abs().max()))
+        worst_l = max(worst_l, float((lse[bi, hi, idx].double() - L).abs().max()))
+    return worst_o, worst_l
+
+
+def _head_backward_check_f64(q, k, v, do, o, dq, dk, dv, scale, bi, hi):
+    """dQ, dK, dV of one (batch, head) against the analytic gradients in float64 (full
+    attention, h == h_k).  -> dict of worst absolute errors."""
+    Q, K, V, DO = (t[bi, :, hi].double() for t in (q, k, v, do))
+    P = torch.softmax((Q @ K.T) * scale, dim=-1)
+    O = P @ V
+    dP = DO @ V.T
+    dS = P * (dP - (DO * O).sum(-1, keepdim=True))
+    ref = {"dq": dS @ K * scale, "dk": dS.T @ Q * scale, "dv": P.T @ DO}
+    got = {"dq": dq, "dk": dk, "dv": dv}
+    return {n: float((got[n][bi, :, hi].double() - ref[n]).abs().max()) for n in ref}
+
+
 def test_baseline_config4_forward_full_size():
     """fp16 causal b4 h32 s2048 d128, scale 1/sqrt(128)."""
     from byteir_amd import ops
@@ -445,6 +477,11 @@ def test_baseline_config4_forward_full_size():
     scale = 1 / np.sqrt(128)
     o, lse = ops.flash_attn_fwd(q, k, v, scale, (-1, 0))
     _sampled_forward_check(q, k, v, o, lse, scale, (-1, 0), oracle.F16, 64, 1)
+    # 512 sampled query rows of every head of batch 0, float64 closed form
+    rows = np.sort(np.random.default_rng(0xC4).choice(2048, 512, replace=False))
+    wo, wl = _rows_forward_check_f64(q, k, v, o, lse, scale, True, 0, range(32), rows)
+    assert wo <= ATOL and wl <= ATOL, f"worst absolute error over 512 rows x 32 heads: O {wo:.5f}, LSE {wl:.5f} (bound {ATOL})"
+    print(f"c4 forward, 512 rows x 32 heads of batch 0: worst |O - f64| = {wo:.2e}, worst |LSE - f64| = {wl:.2e}")
     # one whole head against the oracle
     sl = (slice(1, 2), slice(None), slice(5, 6))
     _, lse_ref, o32 = oracle.flash_fwd(host(q[sl]), host(k[sl]), host(v[sl]), scale, (-1, 0), round_p=False)
@@ -463,22 +500,19 @@ def test_baseline_config5_forward_backward_full_size():
     scale = 0.125
     o, lse = ops.flash_attn_fwd(q, k, v, scale, (-1, -1))
     _sampled_forward_check(q, k, v, o, lse, scale, (-1, -1), oracle.BF16, 32, 2)
+    # 512 sampled query rows of all 16 heads of batch 0, float64 closed form
+    rows = np.sort(np.random.default_rng(0xC5).choice(8192, 512, replace=False))
+    wo, wl = _rows_forward_check_f64(q, k, v, o, lse, scale, False, 0, range(16), rows)
+    assert wo <= ATOL and wl <= ATOL, f"worst absolute error over 512 rows x 16 heads: O {wo:.5f}, LSE {wl:.5f} (bound {ATOL})"
+    print(f"c5 forward, 512 rows x 16 heads of batch 0: worst |O - f64| = {wo:.2e}, worst |LSE - f64| = {wl:.2e}")
     dq, dk, dv = ops.flash_attn_bwd(do, q, k, v, o, lse, scale, (-1, -1))
-    # closed form for one (batch, head) on the GPU in float64 via torch (plumbing only)
-    bi, hi = 1, 7
-    Q, K, V, DO = (t[bi, :, hi].double() for t in (q, k, v, do))
-    S = (Q @ K.T) * scale
-    P = torch.softmax(S, dim=-1)
-    O = P @ V
-    dV = P.T @ DO
-    dP = DO @ V.T
-    D = (DO * O).sum(-1, keepdim=True)
-    dS = P * (dP - D)
-    dQ = dS @ K * scale
-    dK = dS.T @ Q * scale
-    assert float((dq[bi, :, hi].double() - dQ).abs().max()) <= ATOL
-    assert float((dk[bi, :, hi].double() - dK).abs().max()) <= ATOL
-    assert float((dv[bi, :, hi].double() - dV).abs().max()) <= ATOL
+    # two whole (batch, head) pairs against the analytic gradients in float64 (torch on the GPU
+    # as plumbing).  Bound: north_star's 2e-2 absolute; the worst error is printed so that the
+    # margin is on record.
+    for bi, hi in ((1, 7), (0, 3)):
+        worst = _head_backward_check_f64(q, k, v, do, o, dq, dk, dv, scale, bi, hi)
+        assert all(e <= ATOL for e in worst.values()), f"batch {bi} head {hi}: worst absolute errors {worst} (bound {ATOL})"
+        print(f"c5 backward, batch {bi} head {hi}: worst absolute errors {worst}")
     # sum rule over all heads: sum_j dV_j = sum_i dO_i (softmax rows sum to one)
     lhs = dv.float().sum(dim=1)
     rhs = do.float().sum(dim=1)
