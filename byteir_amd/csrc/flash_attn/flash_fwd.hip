@@ -238,7 +238,11 @@ __global__ void __launch_bounds__(NW * 64, NW * QB >= 16 ? 2 : (QB == 2 ? 1 : 2)
     }
   };
 
-  // exponentials, row sums and P^T of one unit (branch free)
+  // exponentials, row sums and P^T of one unit (branch free).  At head_dim 128 the row sum is
+  // taken over the rounded P that the P V product uses, two elements per v_dot2c (fp32
+  // accumulation), which halves the additions; at head_dim 64 that measured no faster and the
+  // sum stays on the unrounded exponentials.
+  constexpr bool kDotSum = D >= 128;
   auto sm_exp = [&](Unit &u, vec8 (&pb)[QB][2]) {
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb) {
@@ -249,16 +253,17 @@ __global__ void __launch_bounds__(NW * 64, NW * QB >= 16 ? 2 : (QB == 2 ? 1 : 2)
       for (int i = 0; i < 16; ++i) {
         const float e = exp2_fast(fmaf(sc[i], c, -m_scaled));
         sc[i] = e;
-        rs += e;
+        if constexpr (!kDotSum) rs += e;
       }
-      l_run[qb] += rs;
 #pragma unroll
       for (int w = 0; w < 2; ++w) {
         float pf[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) pf[j] = sc[w * 8 + j];
         pb[qb][w] = pack8<T>(pf);
+        if constexpr (kDotSum) rs = sum8_acc<T>(pb[qb][w], rs);
       }
+      l_run[qb] += rs;
     }
   };
 

@@ -34,7 +34,7 @@ namespace {
 // HBM efficiency (79 us against 82 us with eight for the [16384, 8192] column fold).
 constexpr int kRowU = 4;
 constexpr int kColU = 4;
-constexpr int kColWideW = 2, kColWideU = 2;  // column groups per lane and rows in flight, wide kernel
+constexpr int kColWideU = 2;  // rows in flight per lane and column group, wide kernel
 constexpr int kBlock = 256;            // threads per workgroup (4 waves)
 constexpr uint64_t kFillThreads = 256ull * 1024;  // threads wanted in flight chip-wide
 
@@ -248,9 +248,9 @@ reduce_col_kernel(const T *__restrict__ in, TO *__restrict__ out, uint64_t B, ui
 
 // Wide tensors: a block of 256 lanes spans W * 4 KiB of a row, every lane owns W groups of
 // VEC adjacent columns 256 * VEC apart and keeps U rows in flight (W * U 128-bit loads per
-// lane).  No LDS: every lane stores its own columns.  Two groups with two rows in flight
-// measured fastest for the [16384, 8192] fold (77 us against 79.6 us with one group and
-// four rows), at the price of twice as many segments for the same 512 workgroups.
+// lane).  No LDS: every lane stores its own columns.  Several groups with two rows in flight
+// measured fastest for the [16384, 8192] fold: 77.3 us with two groups on 512 workgroups and
+// 76.8 us with four groups on 256, against 79.6 us with one group and four rows.
 template <typename T, typename TO, int OP, int VEC, int W, int U>
 __global__ void __launch_bounds__(kBlock)
 reduce_colwide_kernel(const T *__restrict__ in, TO *__restrict__ out, uint64_t B, uint64_t C,
@@ -360,8 +360,8 @@ Plan make_plan(int dtype, uint64_t A, uint64_t B, uint64_t C, bool allow_split) 
   p.vec = (C % vec_full == 0) ? vec_full : 1;
   const uint64_t ncolv = ceil_div(C, p.vec);
   if (allow_split && p.vec > 1 && ncolv >= 2 * kBlock) {
-    p.kind = 3;  // 8 KiB of a row per block
-    p.g = kColWideW * kBlock;
+    p.kind = 3;  // 8 or 16 KiB of a row per block (two or four column groups per lane)
+    p.g = (ncolv >= 4 * kBlock ? 4 : 2) * kBlock;
   } else if (allow_split) {
     // first (or only) pass: a block spans up to 256 lanes x 128 bits = 4 KiB of one row
     p.g = ncolv >= 256 ? 256 : ncolv > 32 ? 64 : ncolv > 8 ? 32 : 8;
@@ -376,8 +376,10 @@ Plan make_plan(int dtype, uint64_t A, uint64_t B, uint64_t C, bool allow_split) 
   const uint64_t blocks0 = A * p.col_tiles;
   uint64_t S = 1;
   // Long sequential streams from about two resident workgroups per CU measured fastest on
-  // MI355X (more, shorter segments lose HBM efficiency), so the split aims at 512 workgroups.
-  constexpr uint64_t kWantBlocks = 512;
+  // MI355X (more, shorter segments lose HBM efficiency), so the split aims at 512 workgroups;
+  // with four column groups per lane a workgroup keeps as many loads in flight as two of the
+  // others, and one per CU is enough.
+  const uint64_t kWantBlocks = (p.kind == 3 && p.g == 4 * kBlock) ? 256 : 512;
   if (allow_split && blocks0 < kWantBlocks && B > (uint64_t)ty * 8) {
     const uint64_t want = ceil_div(kWantBlocks, blocks0);
     const uint64_t room = ceil_div(B, (uint64_t)ty * 8);
@@ -422,7 +424,8 @@ hipError_t launch(const Plan &p, const T *in, TO *out, uint64_t A, uint64_t B, u
   if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
   const dim3 grid((unsigned)blocks), block(kBlock);
   if (p.kind == 3 && vec) {
-    reduce_colwide_kernel<T, TO, OP, VF, kColWideW, kColWideU><<<grid, block, 0, stream>>>(in, out, B, C, p.S, p.seg, col_tiles, len);
+    if (p.g == 4 * kBlock) reduce_colwide_kernel<T, TO, OP, VF, 4, kColWideU><<<grid, block, 0, stream>>>(in, out, B, C, p.S, p.seg, col_tiles, len);
+    else reduce_colwide_kernel<T, TO, OP, VF, 2, kColWideU><<<grid, block, 0, stream>>>(in, out, B, C, p.S, p.seg, col_tiles, len);
     return hipGetLastError();
   }
 #define COL(TX)                                                                                  \
