@@ -234,7 +234,7 @@ def main():
     ap.add_argument("--no-extras", action="store_true", help="skip the other benchmark configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--pmc-probe", action="store_true",
-                    help="counter-collection mode: one copy kernel of known size, then two steps")
+                    help="counter-collection mode: one copy kernel of known size, then two C2 steps, two cache-decode calls and two softmax calls")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build is single-GPU (one process, one MI355X); run with --gpus 1")
@@ -295,8 +295,15 @@ def main():
         for _ in range(2):
             ops.flash_attn_kvcache(qd, kc, vc, kn, vn, lens, 1.0 / np.sqrt(d_), (-1, -1))
         torch.cuda.synchronize()
+        # two calls of the fused softmax configuration ([32768, 4096] bf16: 256 MiB in, 256 MiB out)
+        del qd, kc, vc, kn, vn
+        x3 = ops.fill(torch.empty((32768, 4096), dtype=torch.bfloat16, device="cuda"), _lib.FILL_NORMAL, SEED["c3"], 0.0, 2.0)
+        y3 = torch.empty_like(x3)
+        for _ in range(2):
+            ops.softmax(x3, out=y3)
+        torch.cuda.synchronize()
         print(json.dumps({"pmc_probe": True, "copy_bytes_read": in_bytes, "copy_bytes_written": in_bytes,
-                          "decode_cache_bytes": 2 * b_ * sk_ * hk_ * d_ * 2}))
+                          "decode_cache_bytes": 2 * b_ * sk_ * hk_ * d_ * 2, "softmax_bytes_each_way": 32768 * 4096 * 2}))
         return
 
     # parity gate (and the CPU baseline's input): the host regenerates buffer 0 from its seed
