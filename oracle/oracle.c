@@ -308,15 +308,16 @@ void oracle_reduce(int op, int dtype, const void *in, void *out, uint64_t A, uin
       float *o = y + a * C;
       const float init = op == 0 ? 0.f : -INFINITY;
       for (uint64_t c = 0; c < C; ++c) o[c] = init;
-      /* for b, for c: keeps each output's chain in b order and walks memory linearly */
-      for (uint64_t b = 0; b < B; ++b) {
-        const float *row = x + (a * B + b) * C;
-        if (op == 0) {
-#pragma omp parallel for num_threads(g_threads) schedule(static) if (C >= 4096)
-          for (int64_t c = 0; c < (int64_t)C; ++c) o[c] = o[c] + row[c];
-        } else {
-#pragma omp parallel for num_threads(g_threads) schedule(static) if (C >= 4096)
-          for (int64_t c = 0; c < (int64_t)C; ++c) o[c] = op_max(o[c], row[c]);
+      /* for b, for c: keeps each output's chain in b order and walks memory linearly; with
+       * several threads every thread owns a contiguous stripe of columns and does the same */
+      const int nt = (C >= 4096 && g_threads > 1) ? g_threads : 1;
+#pragma omp parallel for num_threads(nt) schedule(static)
+      for (int t = 0; t < nt; ++t) {
+        const uint64_t c0 = C * (uint64_t)t / (uint64_t)nt, c1 = C * (uint64_t)(t + 1) / (uint64_t)nt;
+        for (uint64_t b = 0; b < B; ++b) {
+          const float *row = x + (a * B + b) * C;
+          if (op == 0) { for (uint64_t c = c0; c < c1; ++c) o[c] = o[c] + row[c]; }
+          else { for (uint64_t c = c0; c < c1; ++c) o[c] = op_max(o[c], row[c]); }
         }
       }
     }
