@@ -374,6 +374,34 @@ def test_strided_tensors(case, code):
         assert err <= ATOL, (name, float(err))
 
 
+@pytest.mark.parametrize("d", [64, 128])
+def test_head_slices_of_two_gib_take_the_generic_kernels(d):
+    """The tuned kernels address K / V (and Q / dO in the backward) with 32-bit byte offsets
+    inside a (batch, head) slice; a slice that spans 2 GiB or more (here: key rows 4 MiB apart)
+    must be routed to the kernels with 64-bit addressing and give the same answer."""
+    from byteir_amd import ops
+    b, sq, sk, h = 1, 192, 512, 2
+    window = (-1, 0)
+    q, k, v, do = make_inputs((b, sq, sk, h, h, d, window), oracle.F16, seed=77 + d)
+    scale = 1.0 / np.sqrt(d)
+    dq_, dk_, dv_, do_ = (dev(t) for t in (q, k, v, do))
+    row = 1 << 21  # elements between consecutive key rows: 512 rows span 2 GiB
+    wide = lambda x: torch.empty((sk - 1) * row + h * d, dtype=x.dtype, device="cuda").as_strided((b, sk, h, d), (0, row, d, 1))
+    kw, vw = wide(dk_), wide(dv_)
+    kw.copy_(dk_)
+    vw.copy_(dv_)
+    o_w, lse_w = ops.flash_attn_fwd(dq_, kw, vw, scale, window)
+    o_d, lse_d = ops.flash_attn_fwd(dq_, dk_, dv_, scale, window)
+    assert float((o_w.float() - o_d.float()).abs().max()) <= 4e-3
+    assert float((lse_w - lse_d).abs().max()) <= 1e-4
+    gq, gk, gv = ops.flash_attn_bwd(do_, dq_, dk_, dv_, o_d, lse_d, scale, window)
+    wq, wk, wv = ops.flash_attn_bwd(do_, dq_, kw, vw, o_d, lse_d, scale, window)
+    assert wk.stride() == kw.stride()
+    for name, got, want in (("dq", wq, gq), ("dk", wk, gk), ("dv", wv, gv)):
+        err = float((got.float() - want.float()).abs().max())
+        assert err <= 8e-3, (name, err)
+
+
 @pytest.mark.parametrize("case,p_drop", [
     ((2, 700, 700, 8, 2, 64, (-1, 0)), 0.0),     # tuned kernels, grouped heads
     ((1, 300, 2500, 4, 4, 128, (-1, -1)), 0.0),  # forward split over workgroups and merged
