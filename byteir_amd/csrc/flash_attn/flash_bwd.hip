@@ -466,8 +466,11 @@ __global__ void __launch_bounds__(256, (D <= 64 && KB == 1) ? 2 : 1) dkdv_kernel
   if constexpr (kLean) {
     // the wave's dK and dV rows -> its own [32][D] tiles in the idle Q and dO rings -> whole rows
     static_assert(KB == 1, "one key block per wave");
-    constexpr int OS = D + 8, CPRO = D / 8, RPI = 64 / CPRO;
-    static_assert(!kLean || 4 * 32 * OS <= kRing * kQTile * QS, "staging must fit the ring");
+    // unpadded tiles; the 16-byte chunks of row r are permuted by r >> 1 and odd rows swap the
+    // two 8-byte halves of a chunk: no bank conflicts for the 8-byte writes (a lane per row)
+    // nor for the 16-byte reads (16 lanes per row)
+    constexpr int OS = D, CPRO = D / 8, RPI = 64 / CPRO;
+    static_assert(!kLean || (D == 128 && 4 * 32 * OS <= kRing * kQTile * QS), "staging must fit the ring; 16 chunks per row");
     __syncthreads();  // every wave has left the last Q / dO tile
     T *Kt = &Qs[0][0] + wave * 32 * OS, *Vt = &dOs[0][0] + wave * 32 * OS;
     typedef T vec4 __attribute__((ext_vector_type(4)));
@@ -481,15 +484,17 @@ __global__ void __launch_bounds__(256, (D <= 64 && KB == 1) ? 2 : 1) dkdv_kernel
           a[j] = (T)(dk_acc[0][db][i4 * 4 + j] * p.scale);
           b[j] = (T)(dv_acc[0][db][i4 * 4 + j]);
         }
-        *reinterpret_cast<vec4 *>(&Kt[r32 * OS + db * 32 + i4 * 8 + g * 4]) = a;
-        *reinterpret_cast<vec4 *>(&Vt[r32 * OS + db * 32 + i4 * 8 + g * 4]) = b;
+        const int so = r32 * OS + (((db * 4 + i4) ^ (r32 >> 1)) * 8) + ((g ^ (r32 & 1)) * 4);
+        *reinterpret_cast<vec4 *>(&Kt[so]) = a;
+        *reinterpret_cast<vec4 *>(&Vt[so]) = b;
       }
     const int oc = lane % CPRO, orow = lane / CPRO;
 #pragma unroll
     for (int it = 0; it < 32 / RPI; ++it) {
       const int r = it * RPI + orow, kv = wkv0 + r;
-      const uint4 a = *reinterpret_cast<const uint4 *>(&Kt[r * OS + oc * 8]);
-      const uint4 b = *reinterpret_cast<const uint4 *>(&Vt[r * OS + oc * 8]);
+      uint4 a = *reinterpret_cast<const uint4 *>(&Kt[r * OS + ((oc ^ (r >> 1)) * 8)]);
+      uint4 b = *reinterpret_cast<const uint4 *>(&Vt[r * OS + ((oc ^ (r >> 1)) * 8)]);
+      if (r & 1) { a = uint4{a.z, a.w, a.x, a.y}; b = uint4{b.z, b.w, b.x, b.y}; }
       if (kv < p.sk) {
         *reinterpret_cast<uint4 *>(static_cast<T *>(p.dk) + bi * p.dk_bs + (int64_t)kv * p.dk_rs + hk * p.dk_hs + oc * 8) = a;
         *reinterpret_cast<uint4 *>(static_cast<T *>(p.dv) + bi * p.dv_bs + (int64_t)kv * p.dv_rs + hk * p.dv_hs + oc * 8) = b;

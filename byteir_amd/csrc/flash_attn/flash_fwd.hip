@@ -369,9 +369,11 @@ __global__ void __launch_bounds__(NW * 64, NW * QB >= 16 ? 2 : (QB == 2 ? 1 : 2)
     if constexpr (kStageO) {
       // O^T in the accumulators -> the wave's own [32][D] tile in the (now idle) K/V ring ->
       // whole 2*D-byte rows to global memory, 16 bytes per lane
-      // The tile is unpadded; the 16-byte chunks of row r are permuted by r & 15 and rows
-      // 16..31 swap the two 8-byte halves of a chunk, which keeps both the 8-byte writes (a
-      // lane per row) and the 16-byte reads (16 lanes per row) free of bank conflicts.
+      // The tile is unpadded; the 16-byte chunks of row r are permuted by r >> 1 and odd rows
+      // swap the two 8-byte halves of a chunk, which keeps both the 8-byte writes (a lane per
+      // row) and the 16-byte reads (16 lanes per row) free of bank conflicts (counter-checked
+      // in isolation: a padded tile costs 96 conflict cycles per wave, permuting by r & 15
+      // with the halves of rows 16..31 swapped 64, this layout none).
       constexpr int OS = D;
       static_assert(D == 128, "the chunk permutation assumes 16 chunks per row");
       static_assert(!kStageO || (NW / 2 * 32 * OS <= kStages * kBN * KS && NW / 2 * 32 * OS <= kStages * kBN * VS), "O staging must fit the ring");
@@ -385,16 +387,15 @@ __global__ void __launch_bounds__(NW * 64, NW * QB >= 16 ? 2 : (QB == 2 ? 1 : 2)
           vec4 v;
 #pragma unroll
           for (int j = 0; j < 4; ++j) v[j] = (T)(o_acc[qb][db][i4 * 4 + j] * inv);
-          *reinterpret_cast<vec4 *>(&Ot[r32 * OS + (((db * 4 + i4) ^ (r32 & 15)) * 8) + ((g ^ (r32 >> 4)) * 4)]) = v;
+          *reinterpret_cast<vec4 *>(&Ot[r32 * OS + (((db * 4 + i4) ^ (r32 >> 1)) * 8) + ((g ^ (r32 & 1)) * 4)]) = v;
         }
       constexpr int CPRO = D / 8, RPI = 64 / CPRO;  // 16-byte chunks per row, rows per store instruction
       const int oc = lane % CPRO, orow = lane / CPRO;
 #pragma unroll
       for (int it = 0; it < 32 / RPI; ++it) {
         const int r = it * RPI + orow, q = wq0 + qb * 32 + r;
-        uint4 v = *reinterpret_cast<const uint4 *>(&Ot[r * OS + ((oc ^ (r & 15)) * 8)]);
-        if ((it * RPI) & 16) v = uint4{v.z, v.w, v.x, v.y};
-        static_assert(RPI <= 16 && 16 % RPI == 0, "a store instruction stays inside one 16-row half");
+        uint4 v = *reinterpret_cast<const uint4 *>(&Ot[r * OS + ((oc ^ (r >> 1)) * 8)]);
+        if (r & 1) v = uint4{v.z, v.w, v.x, v.y};
         if (q < p.sq)
           *reinterpret_cast<uint4 *>(static_cast<T *>(p.o_w) + bi * p.o_bs + (int64_t)q * p.o_rs + hi * p.o_hs + oc * 8) = v;
       }
