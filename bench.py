@@ -486,18 +486,43 @@ def extras(all_cfg, ev, ops, _lib, oracle, args, np, torch, n_thr):
                 ops.reduce_abc(_lib.REDUCE_SUM, b, o1, 4096, 1024, 1, stream=torch.cuda.current_stream())
     torch.cuda.synchronize()
     ms_graph = time_ops(ev, [graph.replay], steps, warm)["ms"]
+    # and through the runtime itself: one ByRE module with 40 ReduceSumOp_f32_f32 ops, one per
+    # buffer, run by the C++ session (one `run` = 40 op-kernel launches on the request's stream)
+    from byteir_amd import brt
+    tin, tout = 'memref<4096x1024xf32, "cuda">', 'memref<4096xf32, "cuda">'
+    margs = ",\n".join(f'    %arg{j} : {tin} {{byre.argname = "A{j}", byre.argtype = 1: i32}}' for j in range(len(bufs)))
+    mops = "\n".join(f'    byre.compute @ReduceSumOp_f32_f32(%arg{j}, %out) {{dimensions = dense<[1]> : tensor<1xi64>, '
+                      f'memory_effects = [1 : i32, 2 : i32]}} : {tin}, {tout}' for j in range(len(bufs)))
+    module = ("module attributes {byre.container_module} {\n  func.func @c1(\n" + margs +
+              f',\n    %out : {tout} {{byre.argname = "B", byre.argtype = 2: i32}}) attributes {{byre.entry_point}} {{\n' +
+              mops + "\n    return\n  }\n}\n")
+    sess = brt.Session(device="ROCM", device_id=0)
+    sess.load_from_memory(module)
+    req = sess.new_request_context(torch.cuda.current_stream().cuda_stream)
+    for j, b in enumerate(bufs):
+        req.bind_arg(j, b.data_ptr())
+    o_sess = torch.zeros(4096, device="cuda")
+    req.bind_arg(len(bufs), o_sess.data_ptr())
+    req.finish_io_binding()
+    req.run()
+    req.sync()
+    gate(torch.equal(o_sess, ops.reduce_abc(_lib.REDUCE_SUM, bufs[-1], torch.empty_like(o_sess), 4096, 1024, 1)),
+         "c1 through the session differs from the direct call")
+    rs = time_ops(ev, [req.run], steps, warm)
     ms_direct = rd["ms"] / len(bufs)
     c1 = {"value": round(b1 / (ms_direct * 1e-3) / 1e9, 1), "unit": "GB/s", "us_per_op": round(ms_direct * 1e3, 2),
           "frac_of_hbm_peak": round(b1 / (ms_direct * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
           "median_us_per_op": round(rd["median_ms"] / len(bufs) * 1e3, 2),
           "python_mirror_GBs": round(b1 / (ms_cold / 10 * 1e-3) / 1e9, 1), "python_mirror_us_per_op": round(ms_cold / 10 * 1e3, 2),
           "python_mirror_warm_cache_us_per_op": round(ms_warm / 10 * 1e3, 2),
+          "brt_session_us_per_op": round(rs["ms"] / len(bufs) * 1e3, 2),
           "graph_replay_GBs": round(b1 / (ms_graph / len(bufs) * 1e-3) / 1e9, 1),
           "graph_replay_us_per_op": round(ms_graph / len(bufs) * 1e3, 2),
           "note": "16 MiB per launch: bound by launch latency, not by HBM (an empty kernel costs 2.4 us back to back); "
                   "value = back-to-back launches through the C ABI over 40 rotating buffers (beyond the last-level cache) "
                   "with the arguments marshalled once, python_mirror = the same through the Python mirror of the op "
-                  "interface (host-bound), graph_replay = the same 40 launches replayed from one HIP graph"}
+                  "interface (host-bound), brt_session = a ByRE module of 40 ReduceSumOp_f32_f32 ops run by the C++ session, "
+                  "graph_replay = the same 40 launches replayed from one HIP graph"}
     if do_cpu:
         t1, tn = cpu_both(oracle, lambda: oracle.reduce_abc(oracle.SUM, xh, 4096, 1024, 1), n_thr, 3)
         c1.update(cpu_1core_GBs=round(b1 / t1 / 1e9, 3), cpu_allcore_GBs=round(b1 / tn / 1e9, 3), cpu_cores=n_thr)
