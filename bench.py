@@ -324,6 +324,44 @@ def main():
     r2 = time_ops(ev, c2_fns, args.steps, args.warmup)
     ms_step, per, host_ms = r2["ms"], r2["per"], r2["host_ms"]
     value = step_bytes / (ms_step * 1e-3) / 1e9
+    # The same step as the runtime runs it: a ByRE module with the four Reduce{Max,Sum}Op_f32_f32
+    # ops, loaded by the C++ session (workspace from the frame's allocator), one `run` per step
+    # over the same three rotating inputs (one request context per input buffer).
+    from byteir_amd import brt
+    t_in, t_c, t_r = f'memref<{R}x{Cc}xf32, "cuda">', f'memref<{Cc}xf32, "cuda">', f'memref<{R}xf32, "cuda">'
+    mod = ("module attributes {byre.container_module} {\n  func.func @c2(\n"
+           f'    %x : {t_in} {{byre.argname = "X", byre.argtype = 1: i32}},\n'
+           f'    %cmax : {t_c} {{byre.argname = "CMAX", byre.argtype = 2: i32}},\n'
+           f'    %csum : {t_c} {{byre.argname = "CSUM", byre.argtype = 2: i32}},\n'
+           f'    %rmax : {t_r} {{byre.argname = "RMAX", byre.argtype = 2: i32}},\n'
+           f'    %rsum : {t_r} {{byre.argname = "RSUM", byre.argtype = 2: i32}}) attributes {{byre.entry_point}} {{\n'
+           + "".join(f'    byre.compute @Reduce{op}Op_f32_f32(%x, %{o}) {{dimensions = dense<[{d}]> : tensor<1xi64>, '
+                     f'memory_effects = [1 : i32, 2 : i32]}} : {t_in}, {t}\n'
+                     for op, o, d, t in (("Max", "cmax", 0, t_c), ("Sum", "csum", 0, t_c), ("Max", "rmax", 1, t_r), ("Sum", "rsum", 1, t_r)))
+           + "    return\n  }\n}\n")
+    sess = brt.Session(device="ROCM", device_id=0)
+    sess.load_from_memory(mod)
+    s_outs = [torch.empty(n, device="cuda") for n in (Cc, Cc, R, R)]
+    reqs = []
+    for x in xs:
+        rq = sess.new_request_context(torch.cuda.current_stream().cuda_stream)
+        rq.bind_arg(0, x.data_ptr())
+        for j, o in enumerate(s_outs):
+            rq.bind_arg(1 + j, o.data_ptr())
+        rq.finish_io_binding()
+        reqs.append(rq)
+    reqs[0].run()
+    reqs[0].sync()
+    ops.reduce_abc(_lib.REDUCE_SUM, xs[0], out_col, 1, R, Cc, workspace=ws_col)
+    ops.reduce_abc(_lib.REDUCE_MAX, xs[0], out_row, R, Cc, 1, workspace=ws_row)
+    gate(torch.equal(s_outs[1], out_col) and torch.equal(s_outs[2], out_row), "c2 through the session differs from the direct calls")
+    rq_i = [0]
+
+    def session_step():
+        rq_i[0] = (rq_i[0] + 1) % len(reqs)
+        reqs[rq_i[0]].run()
+
+    r_sess = time_ops(ev, [session_step], args.steps, args.warmup)
     # per-op figures: each pair of launches timed back to back on its own, one event pair around
     # all repeats (an event after every launch, as in `per`, leaves the GPU idle for a few
     # microseconds per launch and is kept only as a secondary figure)
@@ -380,6 +418,8 @@ def main():
                    "generator": "brt_rocm_fill / oracle_fill: splitmix64 counter stream per tensor (uniform: 24 bits; "
                                 "normal: sum of twelve 16-bit fields), seeds " + json.dumps({k: hex(v) for k, v in SEED.items()})},
         "roofline": roofline,
+        "through_brt_session": {"ms_per_step": round(r_sess["ms"], 4), "value": round(step_bytes / (r_sess["ms"] * 1e-3) / 1e9, 1),
+                                "unit": "GB/s", "what": "the same four ops as one ByRE module run by the C++ session"},
         "device": {"name": props.name, "compute_units": props.multi_processor_count,
                    "max_shader_clock_mhz": max_sclk, "hbm_bytes": props.total_memory,
                    "memory_clock_mhz": (getattr(props, "memory_clock_rate", 0) or 0) / 1e3 or None,
