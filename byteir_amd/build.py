@@ -7,6 +7,7 @@ Targets:
   kernels -> lib/libbrt_rocm_kernels.so   reductions, softmax, device plumbing (C ABI)
   flash   -> lib/libflash_attn.so         flash-attention custom library (C ABI)
   brt     -> lib/libbrt.so                BRT-shaped C++ host runtime (g++, no HIP headers)
+  index_check -> lib/libfa_index_check.so host-only bounds check of the flash-attention index arithmetic
 """
 import os
 import subprocess
@@ -64,11 +65,18 @@ def build_brt(verbose=False):
          + [f"-L{LIB}", "-lbrt_rocm_kernels", "-ldl", "-Wl,-rpath,$ORIGIN"], verbose)
 
 
-TARGETS = {"kernels": build_kernels, "flash": build_flash, "brt": build_brt}
+def build_index_check(verbose=False):
+    """Host-only bounds check of the flash-attention kernels' index arithmetic (g++, no GPU)."""
+    os.makedirs(LIB, exist_ok=True)
+    _run(["g++"] + CXX_FLAGS + ["-o", os.path.join(LIB, "libfa_index_check.so"),
+                                os.path.join(CSRC, "flash_attn", "index_check.cc")], verbose)
+
+
+TARGETS = {"kernels": build_kernels, "flash": build_flash, "brt": build_brt, "index_check": build_index_check}
 
 
 def build_all(verbose=False, targets=None):
-    for name in targets or ("kernels", "flash", "brt"):
+    for name in targets or ("kernels", "flash", "brt", "index_check"):
         TARGETS[name](verbose)
 
 

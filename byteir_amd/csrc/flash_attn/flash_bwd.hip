@@ -73,11 +73,10 @@ struct TileLoader {
   // 2 GiB so they cannot wrap.
   __device__ __forceinline__ void start(const T *base, int64_t row_stride, int row0, int n_rows) {
     const int c = threadIdx.x % CPR, r = threadIdx.x / CPR;
-    const unsigned bytes = n_rows > 0 ? (unsigned)((((int64_t)n_rows - 1) * row_stride + D) * 2) : 0u;
-    rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(base), 0, bytes, 0x00020000);
+    rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(base), 0, idx::rsrc_bytes(n_rows, row_stride, D), 0x00020000);
 #pragma unroll
-    for (int s = 0; s < NP; ++s) vo[s] = (unsigned)(((int64_t)(row0 + r + s * RPP) * row_stride + c * 8) * 2);
-    tile_b = (unsigned)(ROWS * row_stride * 2);
+    for (int s = 0; s < NP; ++s) vo[s] = idx::chunk_offset(row0 + r + s * RPP, c, row_stride);
+    tile_b = idx::tile_bytes(ROWS, row_stride);
   }
   // the next tile into a register set of the caller's (two tiles in flight at a workgroup's start)
   __device__ __forceinline__ void gload_into(uint4 (&r)[NP]) {
@@ -144,25 +143,9 @@ __global__ void __launch_bounds__(256, (D <= 64 && KB == 1) ? 2 : 1) dkdv_kernel
   // decisions) then stays scalar and branches on it are real branches
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r32 = lane & 31, g = lane >> 5;
-  int n_block, bh;
-  {
-    const int L = blockIdx.x;
-    if (p.xcd_remap == 2) {  // unequal blocks: the longest (first) key block of every head first
-      const int xcd = L & 7, slot = L >> 3, per_xcd = (p.b * p.h_k) >> 3;
-      bh = (slot % per_xcd) * 8 + xcd;
-      n_block = slot / per_xcd;
-    } else if (p.xcd_remap == 3) {
-      bh = L % (p.b * p.h_k);
-      n_block = L / (p.b * p.h_k);
-    } else if (p.xcd_remap) {
-      const int xcd = L & 7, slot = L >> 3;
-      bh = (slot / p.n_nblocks) * 8 + xcd;
-      n_block = slot % p.n_nblocks;
-    } else {
-      bh = L / p.n_nblocks;
-      n_block = L % p.n_nblocks;
-    }
-  }
+  // unequal blocks (a window): the longest (first) key block of every head first
+  const idx::BlockId blk = idx::decode_block((int)blockIdx.x, p.xcd_remap, p.b * p.h_k, p.n_nblocks);
+  const int bh = blk.bh, n_block = blk.blk;
   // a workgroup belongs to a key/value head; its dK, dV sum over the query heads of the group
   // (with shares: bh runs over virtual heads; hk = key/value head * gsplit + group share)
   const int bi = bh / p.h_k, vh = bh % p.h_k, hk = vh / p.qsplit, q_share = vh % p.qsplit;
@@ -214,17 +197,9 @@ __global__ void __launch_bounds__(256, (D <= 64 && KB == 1) ? 2 : 1) dkdv_kernel
 #pragma unroll
     for (int i = 0; i < D / 32; ++i) { dk_acc[kb][i] = float16v{0}; dv_acc[kb][i] = float16v{0}; }
 
-  // query tiles that can see keys [kvb0, kvb0 + kKeys)
-  int q_lo = 0, q_hi = p.sq;
-  if (p.wr >= 0) q_lo = max(0, kvb0 - off - p.wr);                 // hi(q) = q+1+off+wr > kvb0
-  if (p.wl >= 0) q_hi = min(p.sq, kvb0 + kKeys - off + p.wl);      // lo(q) = q+off-wl < kvb0+kKeys
-  int m_min = q_lo / kQTile;
-  int m_max = q_hi > 0 ? (q_hi + kQTile - 1) / kQTile : 0;
-  if (p.qsplit > 1) {  // this workgroup's share of the visible query tiles
-    const int per = (max(m_max - m_min, 0) + p.qsplit - 1) / p.qsplit;
-    m_min += q_share * per;
-    m_max = min(m_max, m_min + per);
-  }
+  // query tiles that can see keys [kvb0, kvb0 + kKeys); with shares, this workgroup's part of them
+  int m_min, m_max;
+  idx::query_tile_range(p.sq, p.sk, p.wl, p.wr, kvb0, kKeys, kQTile, p.qsplit, q_share, m_min, m_max);
   // the same for the wave's own keys [wkv0, wkv0 + 32*KB)
   int qw_lo = 0, qw_hi = p.sq;
   if (p.wr >= 0) qw_lo = max(0, wkv0 - off - p.wr);
@@ -484,7 +459,7 @@ __global__ void __launch_bounds__(256, (D <= 64 && KB == 1) ? 2 : 1) dkdv_kernel
           a[j] = (T)(dk_acc[0][db][i4 * 4 + j] * p.scale);
           b[j] = (T)(dv_acc[0][db][i4 * 4 + j]);
         }
-        const int so = r32 * OS + (((db * 4 + i4) ^ (r32 >> 1)) * 8) + ((g ^ (r32 & 1)) * 4);
+        const int so = idx::ostage_write_offset(r32, g, db, i4);
         *reinterpret_cast<vec4 *>(&Kt[so]) = a;
         *reinterpret_cast<vec4 *>(&Vt[so]) = b;
       }
@@ -492,8 +467,8 @@ __global__ void __launch_bounds__(256, (D <= 64 && KB == 1) ? 2 : 1) dkdv_kernel
 #pragma unroll
     for (int it = 0; it < 32 / RPI; ++it) {
       const int r = it * RPI + orow, kv = wkv0 + r;
-      uint4 a = *reinterpret_cast<const uint4 *>(&Kt[r * OS + ((oc ^ (r >> 1)) * 8)]);
-      uint4 b = *reinterpret_cast<const uint4 *>(&Vt[r * OS + ((oc ^ (r >> 1)) * 8)]);
+      uint4 a = *reinterpret_cast<const uint4 *>(&Kt[idx::ostage_read_offset(r, oc)]);
+      uint4 b = *reinterpret_cast<const uint4 *>(&Vt[idx::ostage_read_offset(r, oc)]);
       if (r & 1) { a = uint4{a.z, a.w, a.x, a.y}; b = uint4{b.z, b.w, b.x, b.y}; }
       if (kv < p.sk) {
         *reinterpret_cast<uint4 *>(static_cast<T *>(p.dk) + bi * p.dk_bs + (int64_t)kv * p.dk_rs + hk * p.dk_hs + oc * 8) = a;
@@ -550,26 +525,9 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) dq_kernel(const Params p
   // scalar and every combination is its own straight-line instance of the step
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r32 = lane & 31, g = lane >> 5;
-  int m_block, bh;
-  {
-    const int L = blockIdx.x;
-    if (p.xcd_remap == 2) {  // unequal blocks: the longest (last) query block of every head first
-      const int xcd = L & 7, slot = L >> 3, per_xcd = (p.b * p.h) >> 3;
-      bh = (slot % per_xcd) * 8 + xcd;
-      m_block = slot / per_xcd;
-    } else if (p.xcd_remap == 3) {
-      bh = L % (p.b * p.h);
-      m_block = L / (p.b * p.h);
-    } else if (p.xcd_remap) {
-      const int xcd = L & 7, slot = L >> 3;
-      bh = (slot / p.n_mblocks) * 8 + xcd;
-      m_block = slot % p.n_mblocks;
-    } else {
-      bh = L / p.n_mblocks;
-      m_block = L % p.n_mblocks;
-    }
-    m_block = p.n_mblocks - 1 - m_block;
-  }
+  // unequal blocks (a window): the longest (last) query block of every head first
+  const idx::BlockId blk = idx::decode_block((int)blockIdx.x, p.xcd_remap, p.b * p.h, p.n_mblocks);
+  const int bh = blk.bh, m_block = p.n_mblocks - 1 - blk.blk;
   const int bi = bh / p.h, hi = bh % p.h;
   const int m0 = m_block * kQBlock;
   const int wq0 = m0 + wave * 32;
@@ -579,11 +537,8 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) dq_kernel(const Params p
   row_limits(p, qrow, lo_lim, hi_lim);
   row_limits(p, wq0, w_lo_first, w_hi_first);
   row_limits(p, wq0 + 31, w_lo_last, w_hi_last);
-  int b_lo, b_hi, t0, t1;
-  row_limits(p, m0, b_lo, t0);
-  row_limits(p, m0 + kQBlock - 1, t1, b_hi);
-  const int n_min = b_lo / kKvTile;
-  const int n_max = b_hi > 0 ? (b_hi + kKvTile - 1) / kKvTile : 0;
+  int n_min, n_max;
+  idx::key_tile_range(p.sq, p.sk, p.wl, p.wr, m0, kQBlock, kKvTile, n_min, n_max);
 
   const int hk = hi / (p.h / p.h_k);
   const T *kg = static_cast<const T *>(p.k) + bi * p.k_bs + hk * p.k_hs;
@@ -808,7 +763,7 @@ hipError_t launch_bwd_td(const Params &p, hipStream_t stream) {
   const GroupSplit split = plan_group_split(p, (int64_t)pk.n_nblocks * p.b * p.h_k, 256 * (D <= 64 ? 2 : 1), D, kQTile, stream);
   if (p.ws_query) return hipSuccess;  // planning only
   apply_group_split(pk, p, split, D);
-  pk.xcd_remap = ((p.b * pk.h_k) % 8 == 0) ? (p.wr >= 0 ? 2 : 1) : (p.wr >= 0 ? 3 : 0);
+  pk.xcd_remap = idx::block_order_mode(p.b * pk.h_k, p.wr);
   if (pk.n_nblocks > 0)
     dkdv_kernel<T, D, KB><<<dim3((unsigned)(pk.n_nblocks * p.b * pk.h_k)), dim3(256), 0, stream>>>(pk);
   if (split.gs * split.qs > 1) {
@@ -861,13 +816,13 @@ hipError_t launch_group_sum(const Params &p, const GroupSplit &s, int row, int d
 hipError_t launch_bwd(Params &p, int dtype, hipStream_t stream) {
   p.n_mblocks = (p.sq + kQBlock - 1) / kQBlock;
   p.n_nblocks = (p.sk + kKvBlock - 1) / kKvBlock;
-  p.xcd_remap = ((p.b * p.h) % 8 == 0) ? (p.wr >= 0 ? 2 : 1) : (p.wr >= 0 ? 3 : 0);
+  p.xcd_remap = idx::block_order_mode(p.b * p.h, p.wr);
   if (p.b * p.h == 0) return hipSuccess;
   // The tuned kernels address Q / dO / K / V tiles with 32-bit offsets inside a (batch, head)
   // slice (buffer loads), including a few tiles of look-ahead past the end: larger slices
   // take the generic kernels.
   const int64_t max_rs = std::max(std::max(p.q_rs, p.o_rs), std::max(p.k_rs, p.v_rs));
-  const int64_t span = 2 * (((int64_t)std::max(p.sq, p.sk) + 256) * max_rs + 256);
+  const int64_t span = idx::bwd_stream_span_bytes(std::max(p.sq, p.sk), max_rs);
   if (p.drop || (p.d != 32 && p.d != 64 && p.d != 128) || span >= (int64_t(1) << 31)) return launch_bwd_anyd(p, dtype, stream);
   return dtype == 1 ? launch_bwd_t<_Float16>(p, stream) : launch_bwd_t<__bf16>(p, stream);
 }

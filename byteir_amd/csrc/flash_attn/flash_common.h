@@ -16,6 +16,8 @@
 #include <cstdint>
 #include <type_traits>
 
+#include "flash_index.h"
+
 namespace fa {
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
@@ -100,10 +102,7 @@ template <typename T> __device__ __forceinline__ short4v lds_read_tr4(const T *p
 template <typename T>
 __device__ __forceinline__ typename Traits<T>::vec8 lds_read_operand_tr(const T *tile, int stride,
                                                                          int row0, int col0) {
-  const int lane = threadIdx.x & 63;
-  const int i16 = lane & 15, b16 = lane >> 4;
-  const int gg = b16 >> 1;
-  const T *p = tile + (row0 + gg * 4 + (i16 >> 2)) * stride + col0 + (b16 & 1) * 16 + (i16 & 3) * 4;
+  const T *p = tile + idx::tr_operand_offset(threadIdx.x & 63, stride, row0, col0);
   const short4v lo = lds_read_tr4(p);
   const short4v hi = lds_read_tr4(p + 8 * stride);
   short8v v;
@@ -116,8 +115,8 @@ __device__ __forceinline__ typename Traits<T>::vec8 lds_read_operand_tr(const T 
 // want a stride of 4*odd banks; rows read with the transposing load (4 rows x 64 B per
 // half-wave) want a stride of 16 (mod 32) banks.
 template <int D> struct Pad {
-  static constexpr int kPlain = D + 8;
-  static constexpr int kTr = D % 64 == 32 ? D : D + 32;
+  static constexpr int kPlain = idx::pad_plain(D);
+  static constexpr int kTr = idx::pad_tr(D);
 };
 
 // Unpadded tiles that are read both ways (backward: Q, dO and K) cannot satisfy both stride
@@ -129,29 +128,17 @@ template <int D> struct Pad {
 // the 64 banks.  key(r) = key(r + 32), so a lane's offsets inside a 32-row unit do not depend
 // on the unit.
 template <int D> struct Swz {
-  static __device__ __forceinline__ int key(int row) {
-    if constexpr (D == 64) {
-      const int x = (row >> 1) & 7;  // rows 2x, 2x+1 share a key and differ in bank parity
-      return ((x & 1) << 2) | (x >> 1);
-    } else if constexpr (D == 128) {
-      return ((row & 3) << 2) | ((row >> 2) & 3);
-    } else {
-      return (row >> 2) & 3;  // D == 32: four rows span the banks
-    }
-  }
+  static __device__ __forceinline__ int key(int row) { return idx::swz_key<D>(row); }
   // element offset of logical chunk `chunk` of row `row`
-  static __device__ __forceinline__ int off(int row, int chunk) { return row * D + ((chunk ^ key(row)) << 3); }
+  static __device__ __forceinline__ int off(int row, int chunk) { return idx::swz_off<D>(row, chunk); }
 };
 
 // lds_read_operand_tr for a tile laid out with Swz<D>: rows row0.., columns db*32..
 template <typename T, int D>
 __device__ __forceinline__ typename Traits<T>::vec8 lds_read_operand_tr_swz(const T *tile, int row0, int db) {
   const int lane = threadIdx.x & 63;
-  const int i16 = lane & 15, b16 = lane >> 4;
-  const int row = row0 + (b16 >> 1) * 4 + (i16 >> 2);
-  const int chunk = db * 4 + (b16 & 1) * 2 + ((i16 & 3) >> 1), in_chunk = (i16 & 1) * 4;
-  const short4v lo = lds_read_tr4(tile + Swz<D>::off(row, chunk) + in_chunk);
-  const short4v hi = lds_read_tr4(tile + Swz<D>::off(row + 8, chunk) + in_chunk);
+  const short4v lo = lds_read_tr4(tile + idx::swz_tr_operand_offset<D>(lane, row0, db, false));
+  const short4v hi = lds_read_tr4(tile + idx::swz_tr_operand_offset<D>(lane, row0, db, true));
   short8v v;
   v.s0 = lo.s0; v.s1 = lo.s1; v.s2 = lo.s2; v.s3 = lo.s3;
   v.s4 = hi.s0; v.s5 = hi.s1; v.s6 = hi.s2; v.s7 = hi.s3;
@@ -216,10 +203,7 @@ struct Params {
 // Kept key range [lo, hi) for query row `q` when the sequence has `sk` keys
 // (reference: lib/mask.h:160-200).
 __device__ __forceinline__ void row_limits_sk(const Params &p, int sk, int q, int &lo, int &hi) {
-  lo = 0; hi = sk;
-  const int off = sk - p.sq;
-  if (p.wr >= 0) hi = min(sk, q + 1 + off + p.wr);
-  if (p.wl >= 0) lo = max(0, q + off - p.wl);
+  idx::row_limits(p.sq, sk, p.wl, p.wr, q, lo, hi);
 }
 __device__ __forceinline__ void row_limits(const Params &p, int q, int &lo, int &hi) {
   row_limits_sk(p, p.sk, q, lo, hi);
@@ -247,34 +231,19 @@ struct GroupSplit {
 // 32 query heads on 8; one / two / four rounds): D = 64 b1 s8192 1235 / 1083 / 1050 us,
 // b4 s4096 h16/4 637 / 571 / 570, b8 s2048 615 / 604 / 652; D = 128 b1 s4096 h32/4
 // 838 / 626 / 626, b4 s2048 626 / 628 / 681.
-constexpr int kGroupRounds = 2;
+using idx::kGroupRounds;
 inline GroupSplit plan_group_split(const Params &p, int64_t base_wg, int slots, int row, int q_tile, hipStream_t stream) {
   GroupSplit r;
-  const int group = p.h / p.h_k;
   // wanted: one round of workgroups over the chip's slots; more when a window makes them
-  // unequal, so that the longest-first order can even them out
-  const int64_t want_wg = (int64_t)slots * ((p.wr >= 0 || p.wl >= 0) ? kGroupRounds : 1);
-  if (base_wg <= 0 || base_wg >= want_wg) return r;
-  int gs = 1;
-  if (group > 1) {
-    gs = group;
-    for (int c = 2; c <= group; ++c)
-      if (group % c == 0 && base_wg * c >= want_wg) { gs = c; break; }
-  }
-  // still short: cut the query axis too, at least sixteen tiles per share, at most eight shares
-  // (bf16 backward, with / without: b1 h8 s4096 D=128 causal 242 / 270 us, b1 h4 s2048 D=64
-  // causal 71 / 88, b2 h8 on 2 s2048 D=128 causal 147 / 164; with eight tiles per share
-  // b1 h16 s1024 D=128 causal lost 6 %)
-  int qs = 1;
-  if (base_wg * gs < want_wg) {
-    const int64_t n_q_tiles = (p.sq + q_tile - 1) / q_tile;
-    qs = (int)((want_wg + base_wg * gs - 1) / (base_wg * gs));
-    if (qs > n_q_tiles / 16) qs = (int)(n_q_tiles / 16);
-    if (qs > 8) qs = 8;
-    if (qs < 1) qs = 1;
-  }
+  // unequal, so that the longest-first order can even them out.  First the query heads of a
+  // group are shared out; when that is still short, the query axis is cut too, at least sixteen
+  // tiles per share, at most eight shares (bf16 backward, with / without: b1 h8 s4096 D=128
+  // causal 242 / 270 us, b1 h4 s2048 D=64 causal 71 / 88, b2 h8 on 2 s2048 D=128 causal
+  // 147 / 164; with eight tiles per share b1 h16 s1024 D=128 causal lost 6 %)
+  int gs, qs;
+  idx::group_split_counts(p.h, p.h_k, p.sq, p.wl, p.wr, base_wg, slots, q_tile, gs, qs);
   if (gs * qs == 1) return r;
-  const size_t one = (size_t)p.b * p.sk * p.h_k * gs * qs * row * sizeof(float);
+  const size_t one = (size_t)idx::partial_bytes(p.b, p.sk, p.h_k, gs, qs, row);
   const bool usable = p.dq_accum && (reinterpret_cast<uintptr_t>(p.dq_accum) & 15) == 0;
   const size_t in_accum = !usable ? 0 : p.dq_accum_bytes >= 2 * one ? 2 * one : p.dq_accum_bytes >= one ? one : 0;
   const size_t need = 2 * one - in_accum;  // beyond what dq_accum holds

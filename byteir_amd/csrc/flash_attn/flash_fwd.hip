@@ -52,31 +52,14 @@ __global__ void __launch_bounds__(NW * 64, NW * QB >= 16 ? 2 : (QB == 2 ? 1 : 2)
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r32 = lane & 31, g = lane >> 5;
 
-  int m_block, bh;
-  {
-    const int L = blockIdx.x;
-    if (p.xcd_remap == 2) {
-      // Blocks of unequal length (a right window): within an XCD, the longest block of every
-      // (batch, head) first, then the second longest of every one, ...: longest-first list
-      // scheduling, which fills the CUs evenly over the causal triangle (measured 216 -> 178 us
-      // on fp16 causal b4 h32 s2048 d128) at the price of more (batch, head) pairs in flight
-      // per L2.
-      const int xcd = L & 7, slot = L >> 3, per_xcd = (p.b * p.h) >> 3;
-      bh = (slot % per_xcd) * 8 + xcd;
-      m_block = slot / per_xcd;
-    } else if (p.xcd_remap == 3) {  // the same order when b*h is not a multiple of the XCD count
-      bh = L % (p.b * p.h);
-      m_block = L / (p.b * p.h);
-    } else if (p.xcd_remap) {  // consecutive workgroup ids go round-robin over the 8 XCDs
-      const int xcd = L & 7, slot = L >> 3;
-      bh = (slot / p.n_mblocks) * 8 + xcd;
-      m_block = slot % p.n_mblocks;
-    } else {
-      bh = L / p.n_mblocks;
-      m_block = L % p.n_mblocks;
-    }
-    m_block = p.n_mblocks - 1 - m_block;  // longest (causal) blocks first
-  }
+  // Block order (idx::decode_block): consecutive workgroup ids go round-robin over the 8 XCDs and
+  // the blocks of a (batch, head) share one, so that its K/V are fetched into a single L2; with
+  // blocks of unequal length (a right window) the longest block of every (batch, head) comes
+  // first within an XCD, then the second longest of every one, ...: longest-first list
+  // scheduling, which fills the CUs evenly over the causal triangle (measured 216 -> 178 us on
+  // fp16 causal b4 h32 s2048 d128) at the price of more (batch, head) pairs in flight per L2.
+  const idx::BlockId blk = idx::decode_block((int)blockIdx.x, p.xcd_remap, p.b * p.h, p.n_mblocks);
+  const int bh = blk.bh, m_block = p.n_mblocks - 1 - blk.blk;  // longest (causal) blocks first
   const int bi = bh / p.h, hi = bh % p.h, hk = hi / (p.h / p.h_k);
   int sk = p.sk;
   if constexpr (VarK) sk = min(p.sk, p.seqlens_k[bi] + p.seqlen_knew);
@@ -95,11 +78,8 @@ __global__ void __launch_bounds__(NW * 64, NW * QB >= 16 ? 2 : (QB == 2 ? 1 : 2)
   }
   const int w_lo_first = h_lo_first[0], w_hi_last = h_hi_last[QB - 1];  // the wave's widest window
   // tile range of the workgroup
-  int b_lo, b_hi, t0, t1;
-  row_limits_sk(p, sk, m0, b_lo, t0);
-  row_limits_sk(p, sk, m0 + kBM - 1, t1, b_hi);
-  int n_min = b_lo / kBN;
-  int n_max = b_hi > 0 ? (b_hi + kBN - 1) / kBN : 0;
+  int n_min, n_max;
+  idx::key_tile_range(p.sq, sk, p.wl, p.wr, m0, kBM, kBN, n_min, n_max);
   const int split = blockIdx.y;  // key axis split over workgroups: this one's share of the tiles
   if (p.n_splits > 1) {
     n_min = max(n_min, split * p.split_tiles);
@@ -139,17 +119,16 @@ __global__ void __launch_bounds__(NW * 64, NW * QB >= 16 ? 2 : (QB == 2 ? 1 : 2)
   // the descriptor's size); launch_fwd keeps head slices below 2 GiB so the sum cannot wrap.
   typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
   constexpr unsigned kRsrcFlags = 0x00020000;  // raw buffer, 32-bit data format
-  const unsigned k_bytes = sk > 0 ? (unsigned)((((int64_t)sk - 1) * p.k_rs + D) * 2) : 0u;
-  const unsigned v_bytes = sk > 0 ? (unsigned)((((int64_t)sk - 1) * p.v_rs + D) * 2) : 0u;
+  const unsigned k_bytes = idx::rsrc_bytes(sk, p.k_rs, D), v_bytes = idx::rsrc_bytes(sk, p.v_rs, D);
   const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(kg), 0, k_bytes, kRsrcFlags);
   const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(vg), 0, v_bytes, kRsrcFlags);
   unsigned k_vo[NP], v_vo[NP];
 #pragma unroll
   for (int s = 0; s < NP; ++s) {  // surplus threads of a narrow head point beyond the buffer
-    k_vo[s] = ld_on ? (unsigned)(((int64_t)(ld_r + s * RPP) * p.k_rs + ld_c * 8) * 2) : 0xffffffffu;
-    v_vo[s] = ld_on ? (unsigned)(((int64_t)(ld_r + s * RPP) * p.v_rs + ld_c * 8) * 2) : 0xffffffffu;
+    k_vo[s] = ld_on ? idx::chunk_offset(ld_r + s * RPP, ld_c, p.k_rs) : 0xffffffffu;
+    v_vo[s] = ld_on ? idx::chunk_offset(ld_r + s * RPP, ld_c, p.v_rs) : 0xffffffffu;
   }
-  const unsigned k_tile_b = (unsigned)(kBN * p.k_rs * 2), v_tile_b = (unsigned)(kBN * p.v_rs * 2);
+  const unsigned k_tile_b = idx::tile_bytes(kBN, p.k_rs), v_tile_b = idx::tile_bytes(kBN, p.v_rs);
   unsigned k_so = (unsigned)n_min * k_tile_b, v_so = (unsigned)n_min * v_tile_b;  // byte offset of the next tile to fetch
   auto gload = [&]() {
 #pragma unroll
@@ -387,14 +366,14 @@ __global__ void __launch_bounds__(NW * 64, NW * QB >= 16 ? 2 : (QB == 2 ? 1 : 2)
           vec4 v;
 #pragma unroll
           for (int j = 0; j < 4; ++j) v[j] = (T)(o_acc[qb][db][i4 * 4 + j] * inv);
-          *reinterpret_cast<vec4 *>(&Ot[r32 * OS + (((db * 4 + i4) ^ (r32 >> 1)) * 8) + ((g ^ (r32 & 1)) * 4)]) = v;
+          *reinterpret_cast<vec4 *>(&Ot[idx::ostage_write_offset(r32, g, db, i4)]) = v;
         }
       constexpr int CPRO = D / 8, RPI = 64 / CPRO;  // 16-byte chunks per row, rows per store instruction
       const int oc = lane % CPRO, orow = lane / CPRO;
 #pragma unroll
       for (int it = 0; it < 32 / RPI; ++it) {
         const int r = it * RPI + orow, q = wq0 + qb * 32 + r;
-        uint4 v = *reinterpret_cast<const uint4 *>(&Ot[r * OS + ((oc ^ (r >> 1)) * 8)]);
+        uint4 v = *reinterpret_cast<const uint4 *>(&Ot[idx::ostage_read_offset(r, oc)]);
         if (r & 1) v = uint4{v.z, v.w, v.x, v.y};
         if (q < p.sq)
           *reinterpret_cast<uint4 *>(static_cast<T *>(p.o_w) + bi * p.o_bs + (int64_t)q * p.o_rs + hi * p.o_hs + oc * 8) = v;
@@ -536,11 +515,13 @@ hipError_t launch_append_kv(const Params &p, int dtype, hipStream_t stream) {
 }
 
 hipError_t launch_fwd(Params &p, int dtype, hipStream_t stream) {
-  p.xcd_remap = ((p.b * p.h) % 8 == 0) ? (p.wr >= 0 ? 2 : 1) : (p.wr >= 0 ? 3 : 0);
+  p.xcd_remap = idx::block_order_mode(p.b * p.h, p.wr);
   if (p.b * p.h == 0 || p.sq == 0) return hipSuccess;
   if (decode_eligible(p)) return launch_decode(p, dtype, stream);
   // the tuned kernel addresses a head's K and V rows through 32-bit buffer offsets
-  const int64_t kv_span = 2 * ((int64_t)p.sk * std::max(p.k_rs, p.v_rs) + 256);
+  // (the padded rows of the last tile and the tiles of look-ahead that the prologue always
+  // requests are part of the span: their offsets must not wrap either)
+  const int64_t kv_span = idx::fwd_stream_span_bytes(p.sk, std::max(p.k_rs, p.v_rs));
   if (p.drop || (p.d != 32 && p.d != 64 && p.d != 128) || kv_span >= (int64_t(1) << 31)) return launch_fwd_anyd(p, dtype, stream);
   return dtype == 1 ? launch_fwd_t<_Float16>(p, stream) : launch_fwd_t<__bf16>(p, stream);
 }

@@ -293,6 +293,15 @@ def test_random_cases_sweep():
     (1, 4096, 4096, 8, 8, 128, True),     # few heads: query-range shares
     (2, 3000, 3000, 8, 8, 64, False),
     (1, 2048, 6000, 4, 2, 96, True),      # generic kernels, sq != sk
+    # Two ragged shapes that were part of a run which ended in a GPU memory fault (together with
+    # a 64-rows-per-wave forward variant that is not in the tree).  The cause was not found;
+    # the host-side bounds check (tests/test_flash_index_bounds.py) walks every address the
+    # in-tree kernels form for exactly these shapes and finds them all in bounds, but until the
+    # fault is explained they are not run on the GPU: unverified there.
+    pytest.param((4, 1100, 1100, 64, 16, 64, True), marks=pytest.mark.skip(
+        reason="ran in a session that ended in an unexplained GPU memory fault; checked on the host only")),
+    pytest.param((2, 2100, 1500, 64, 64, 64, False), marks=pytest.mark.skip(
+        reason="ran in a session that ended in an unexplained GPU memory fault; checked on the host only")),
 ])
 def test_large_shapes_against_float32_matmul_attention_on_the_gpu(shape):
     """Sizes beyond what the CPU oracle finishes in seconds: the yardstick is plain float32
