@@ -159,6 +159,53 @@ def time_ops(ev, fns, steps, warmup, clocks=None):
     return {"ms": total, "per": per, "host_ms": host_ms, "median_ms": med, "clock": sampler.summary()}
 
 
+def time_regions(ev, fns, iters, warmup, regions=3, clocks=None):
+    """`regions` independent timed regions of `iters` steps each (a step = every closure of `fns`
+    once), one event pair per region on the launch stream, a synchronisation between regions.
+    -> dict(ms: the MEDIAN region's ms per step, min_ms, max_ms, region_ms, host_ms, clock: the
+    shader clock sampled over all regions).  A 2-3 % difference between two kernels is of the
+    size of the spread between regions; the three figures together say how much a number means."""
+    import torch
+    for _ in range(warmup):
+        for f in fns:
+            f()
+    torch.cuda.synchronize()
+    sampler = clocks if clocks is not None else ClockSampler()
+    region_ms, host = [], []
+    with sampler:
+        for _ in range(regions):
+            e0, e1 = ev.new(), ev.new()
+            t0 = time.perf_counter()
+            ev.record(e0)
+            for _ in range(iters):
+                for f in fns:
+                    f()
+            ev.record(e1)
+            torch.cuda.synchronize()
+            host.append((time.perf_counter() - t0) * 1e3 / iters)
+            region_ms.append(ev.elapsed_ms(e0, e1) / iters)
+            ev.free([e0, e1])
+    return {"ms": statistics.median(region_ms), "min_ms": min(region_ms), "max_ms": max(region_ms),
+            "region_ms": region_ms, "host_ms": statistics.median(host), "clock": sampler.summary(),
+            "iters": iters, "regions": regions}
+
+
+def spread(r, ops_per_step=1, digits=2):
+    """min / median / max microseconds per op over the timed regions of `r`."""
+    k = 1e3 / ops_per_step
+    return {"min_us_per_op": round(r["min_ms"] * k, digits), "median_us_per_op": round(r["ms"] * k, digits),
+            "max_us_per_op": round(r["max_ms"] * k, digits), "timed_regions": r["regions"], "iterations_per_region": r["iters"]}
+
+
+def roof(bound, kernel, work, unit_work, ms, peak, source):
+    """The roofline entry of one configuration: algorithmic bytes (or FLOP) per op over the
+    median time per op, against the published peak."""
+    rate = work / (ms * 1e-3) / (1e9 if bound == "hbm" else 1e12)
+    return {"bound": bound, "kernel": kernel, "achieved": round(rate, 1), "peak": peak,
+            "unit": "GB/s" if bound == "hbm" else "TFLOP/s", "frac": round(rate / peak, 4),
+            "algorithmic_" + unit_work: work, "us": round(ms * 1e3, 2), "duration_source": source}
+
+
 def prewarm(fn, seconds=0.5):
     """Run `fn` back to back for about `seconds` of wall time.  After idle time (the parity gate's
     CPU work) or after memory-bound kernels the matrix-heavy attention kernels run 10-20 % slower
@@ -216,13 +263,23 @@ def measured_traffic(K, _lib, R, Cc):
             vals[section].append(int(m.group(1)))
     if not vals["FETCH_SIZE"] or not vals["WRITE_SIZE"]:
         return None, "no reduce_colwide_kernel rows in the profile"
+    # the profile must name the very kernel instantiation the library plans today
+    buf = ctypes.create_string_buffer(256)
+    _lib.check(K.brt_rocm_reduce_plan_describe(_lib.F32, 1, R, Cc, buf, 256))
+    plan = buf.value.decode()
+    for op in "01":
+        name = plan.split(" S=")[0].replace("OP", op)
+        if name not in text:
+            sys.exit(f"bench.py: profiles/reduce_c2_hbm_traffic.txt was measured with another kernel than today's plan ({name}): re-measure it")
     ws_now = K.brt_rocm_reduce_workspace_bytes(_lib.F32, 1, R, Cc)
     ws_then = sum(vals["WRITE_SIZE"]) // len(vals["WRITE_SIZE"])  # the first pass writes exactly its partials
     if ws_now != ws_then:
         sys.exit(f"bench.py: the axis-0 split has changed (partials {ws_now} B now, {ws_then} B when "
                  "profiles/reduce_c2_hbm_traffic.txt was measured): re-measure the traffic profile")
     fetch = sum(vals["FETCH_SIZE"]) / len(vals["FETCH_SIZE"])
-    return int(round(fetch + ws_then)), "profiles/reduce_c2_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, copy-kernel scaled)"
+    return int(round(fetch + ws_then)), ("not measured in this run: read from the tracked profile profiles/reduce_c2_hbm_traffic.txt "
+                                         "(rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE per dispatch, copy-kernel scaled), which names the same "
+                                         "kernel instantiation and the same split as today's plan: " + plan)
 
 
 def main():
@@ -321,8 +378,11 @@ def main():
              f"c2 ReduceSum dims={dims} (1e-5 relative against the float64 fold)")
     oracle.set_threads(1)
 
-    r2 = time_ops(ev, c2_fns, args.steps, args.warmup)
-    ms_step, per, host_ms = r2["ms"], r2["per"], r2["host_ms"]
+    # `value`: three timed regions of exactly `steps` steps each (after `warmup` untimed steps),
+    # the median region counts; the per-launch breakdown comes from a marked pass of time_ops
+    r2 = time_regions(ev, c2_fns, args.steps, args.warmup)
+    r2m = time_ops(ev, c2_fns, args.steps, 0)
+    ms_step, per, host_ms = r2["ms"], r2m["per"], r2["host_ms"]
     value = step_bytes / (ms_step * 1e-3) / 1e9
     # The same step as the runtime runs it: a ByRE module with the four Reduce{Max,Sum}Op_f32_f32
     # ops, loaded by the C++ session (workspace from the frame's allocator), one `run` per step
@@ -361,12 +421,12 @@ def main():
         rq_i[0] = (rq_i[0] + 1) % len(reqs)
         reqs[rq_i[0]].run()
 
-    r_sess = time_ops(ev, [session_step], args.steps, args.warmup)
+    r_sess = time_regions(ev, [session_step], args.steps, args.warmup)
     # per-op figures: each pair of launches timed back to back on its own, one event pair around
     # all repeats (an event after every launch, as in `per`, leaves the GPU idle for a few
     # microseconds per launch and is kept only as a secondary figure)
-    r_col = time_ops(ev, c2_fns[:2], args.steps, max(2, args.warmup // 2))
-    r_row = time_ops(ev, c2_fns[2:], args.steps, max(2, args.warmup // 2))
+    r_col = time_regions(ev, c2_fns[:2], max(args.steps, 25), max(2, args.warmup // 2))
+    r_row = time_regions(ev, c2_fns[2:], max(args.steps, 25), max(2, args.warmup // 2))
     col_ms, row_ms = r_col["ms"] / 2, r_row["ms"] / 2
     col_ms_marked, row_ms_marked = (per[0] + per[1]) / 2, (per[2] + per[3]) / 2
     # The axis-0 op is two launches: the split first pass (the dominant kernel) and a small
@@ -407,7 +467,9 @@ def main():
     result = {
         "metric": METRIC, "value": round(value, 1), "unit": "GB/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_step, 4),
-        "median_ms_per_step": round(r2["median_ms"], 4),
+        "ms_per_step_regions": {"min": round(r2["min_ms"], 4), "median": round(r2["ms"], 4), "max": round(r2["max_ms"], 4),
+                                "timed_regions": r2["regions"], "steps_per_region": args.steps},
+        "ms_per_step_with_an_event_after_every_launch": round(r2m["median_ms"], 4),
         "host_ms_per_step": round(host_ms, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
         "data": "synthetic",
@@ -435,11 +497,17 @@ def main():
         "c2a_col_max_sum_axis0": {"value": round(col_op_gbs, 1), "unit": "GB/s", "us_per_op": round(col_ms * 1e3, 2),
                                   "frac_of_hbm_peak": round(col_op_gbs / HBM_PEAK_GBS, 4),
                                   "first_pass_kernel_GBs": round(col_gbs, 1),
-                                  "us_per_op_with_an_event_after_every_launch": round(col_ms_marked * 1e3, 2)},
+                                  "us_per_op_with_an_event_after_every_launch": round(col_ms_marked * 1e3, 2),
+                                  **spread(r_col, 2),
+                                  "roofline": roof("hbm", "reduce_colwide_kernel<float, float, OP, 4, 4, 2> + reduce_col_kernel<float, float, OP, 4, 8> (combine pass)",
+                                                   bytes_col, "bytes", col_ms, HBM_PEAK_GBS, "event pair around back-to-back ops (both launches of an op), median of three regions")},
         "c2b_row_max_sum_axis1": {"value": round(bytes_row / (row_ms * 1e-3) / 1e9, 1), "unit": "GB/s",
                                   "us_per_op": round(row_ms * 1e3, 2),
                                   "frac_of_hbm_peak": round(bytes_row / (row_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-                                  "us_per_op_with_an_event_after_every_launch": round(row_ms_marked * 1e3, 2)},
+                                  "us_per_op_with_an_event_after_every_launch": round(row_ms_marked * 1e3, 2),
+                                  **spread(r_row, 2),
+                                  "roofline": roof("hbm", "reduce_row_kernel<float, float, OP, 4, 256, false>", bytes_row, "bytes", row_ms, HBM_PEAK_GBS,
+                                                   "event pair around back-to-back launches, median of three regions")},
     }
 
     # ---- CPU baseline for the headline workload --------------------------------------------
@@ -470,9 +538,10 @@ def main():
 
 
 def with_clock(entry, r, peak, key):
-    """Adds the sampled shader clock and the fraction of the peak scaled to that clock."""
+    """Adds the spread over the timed regions, the sampled shader clock and the fraction of the
+    peak scaled to that clock."""
     c = r["clock"]
-    entry["median_us_per_op"] = round(r["median_ms"] * 1e3 / r.get("ops_per_step", 1), 2)
+    entry.update(spread(r, r.get("ops_per_step", 1), 1))
     if c:
         entry["shader_clock_mhz"] = c
         entry[key + "_at_sampled_clock"] = round(entry["value"] / (peak * c["mean_mhz"] / PEAK_CLOCK_MHZ), 4)
@@ -503,7 +572,7 @@ def extras(all_cfg, ev, ops, _lib, oracle, args, np, torch, n_thr):
         i[0] = (i[0] + 1) % len(bufs)
         ops.reduce_abc(_lib.REDUCE_SUM, bufs[i[0]], o1, 4096, 1024, 1)
 
-    rc = time_ops(ev, [c1_cold] * 10, steps, warm)
+    rc = time_regions(ev, [c1_cold] * 10, 50, warm)
     # the same launches through the C ABI itself with the arguments marshalled once (what a
     # compiled host pays per launch), instead of through the Python mirror of the op interface
     import functools
@@ -511,8 +580,8 @@ def extras(all_cfg, ev, ops, _lib, oracle, args, np, torch, n_thr):
     sp1 = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     direct = [functools.partial(K1.brt_rocm_reduce, _lib.REDUCE_SUM, _lib.F32, ctypes.c_void_p(b.data_ptr()),
                                 ctypes.c_void_p(o1.data_ptr()), 4096, 1024, 1, None, 0, sp1) for b in bufs]
-    rd = time_ops(ev, direct, steps, warm)
-    rw = time_ops(ev, [lambda: ops.reduce_abc(_lib.REDUCE_SUM, bufs[0], o1, 4096, 1024, 1)] * 10, steps, warm)
+    rd = time_regions(ev, direct, 50, warm)  # 50 x 40 launches per region
+    rw = time_regions(ev, [lambda: ops.reduce_abc(_lib.REDUCE_SUM, bufs[0], o1, 4096, 1024, 1)] * 10, 50, warm)
     ms_cold, ms_warm = rc["ms"], rw["ms"]
     # the same 40 cold launches captured once in a HIP graph: launch cost leaves the host
     side = torch.cuda.Stream()
@@ -525,7 +594,7 @@ def extras(all_cfg, ev, ops, _lib, oracle, args, np, torch, n_thr):
             for b in bufs:
                 ops.reduce_abc(_lib.REDUCE_SUM, b, o1, 4096, 1024, 1, stream=torch.cuda.current_stream())
     torch.cuda.synchronize()
-    ms_graph = time_ops(ev, [graph.replay], steps, warm)["ms"]
+    ms_graph = time_regions(ev, [graph.replay], 50, warm)["ms"]
     # and through the runtime itself: one ByRE module with 40 ReduceSumOp_f32_f32 ops, one per
     # buffer, run by the C++ session (one `run` = 40 op-kernel launches on the request's stream)
     from byteir_amd import brt
@@ -548,11 +617,13 @@ def extras(all_cfg, ev, ops, _lib, oracle, args, np, torch, n_thr):
     req.sync()
     gate(torch.equal(o_sess, ops.reduce_abc(_lib.REDUCE_SUM, bufs[-1], torch.empty_like(o_sess), 4096, 1024, 1)),
          "c1 through the session differs from the direct call")
-    rs = time_ops(ev, [req.run], steps, warm)
+    rs = time_regions(ev, [req.run], 50, warm)
     ms_direct = rd["ms"] / len(bufs)
     c1 = {"value": round(b1 / (ms_direct * 1e-3) / 1e9, 1), "unit": "GB/s", "us_per_op": round(ms_direct * 1e3, 2),
           "frac_of_hbm_peak": round(b1 / (ms_direct * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-          "median_us_per_op": round(rd["median_ms"] / len(bufs) * 1e3, 2),
+          **spread(rd, len(bufs)),
+          "roofline": roof("hbm", "reduce_row_kernel<float, float, 1, 4, 64, false>", b1, "bytes", ms_direct, HBM_PEAK_GBS,
+                           "event pair around 2000 back-to-back launches over 40 rotating buffers (launch gaps included), median of three regions"),
           "python_mirror_GBs": round(b1 / (ms_cold / 10 * 1e-3) / 1e9, 1), "python_mirror_us_per_op": round(ms_cold / 10 * 1e3, 2),
           "python_mirror_warm_cache_us_per_op": round(ms_warm / 10 * 1e3, 2),
           "brt_session_us_per_op": round(rs["ms"] / len(bufs) * 1e3, 2),
@@ -585,14 +656,35 @@ def extras(all_cfg, ev, ops, _lib, oracle, args, np, torch, n_thr):
         j[0] = (j[0] + 1) % 3
         ops.softmax(xs[j[0]], out=ys)
 
-    r3 = time_ops(ev, [c3], steps, warm)
-    ms3 = r3["ms"]
+    # The copy ceiling is measured here, interleaved with the softmax: a plain copy kernel (one
+    # 128-bit load and store per lane) of the same tensors, region by region in alternation, so
+    # that both see the same box, clock and memory state.
+    K3 = _lib.kernels()
+    sp3 = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def cp():
+        j[0] = (j[0] + 1) % 3
+        _lib.check(K3.brt_rocm_copy_kernel(ys.data_ptr(), xs[j[0]].data_ptr(), b3 // 2, sp3))
+
+    r3s, rcs = [], []
+    for _ in range(3):
+        r3s.append(time_regions(ev, [c3], 100, warm, regions=1))
+        rcs.append(time_regions(ev, [cp], 100, warm, regions=1))
+    ops.softmax(xs[0], out=ys)  # leave ys holding the softmax again
+    merge = lambda rs: {"ms": statistics.median(r["ms"] for r in rs), "min_ms": min(r["ms"] for r in rs), "max_ms": max(r["ms"] for r in rs),
+                        "regions": len(rs), "iters": rs[0]["iters"], "clock": rs[0]["clock"]}
+    r3, rcp = merge(r3s), merge(rcs)
+    ms3, msc = r3["ms"], rcp["ms"]
+    copy_gbs = b3 / (msc * 1e-3) / 1e9
     c3r = {"value": round(b3 / (ms3 * 1e-3) / 1e9, 1), "unit": "GB/s", "us_per_op": round(ms3 * 1e3, 2),
            "frac_of_hbm_peak": round(b3 / (ms3 * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-           "median_us_per_op": round(r3["median_ms"] * 1e3, 2),
-           "frac_of_copy_kernel_ceiling": round(b3 / (ms3 * 1e-3) / 1e9 / 6450.0, 4),
-           "note": "a plain copy of the same tensor (one 128-bit load and store per lane, non-temporal) tops out at "
-                   "6.43-6.50 TB/s on this part: equal parts of reads and writes do not reach the 7.0 TB/s of a pure read stream"}
+           **spread(r3),
+           "copy_kernel_same_tensors": {"value": round(copy_gbs, 1), "unit": "GB/s", **spread(rcp)},
+           "frac_of_copy_kernel_ceiling": round(msc / ms3, 4),
+           "roofline": roof("hbm", "softmax_split_kernel<__bf16, 4, true>", b3, "bytes", ms3, HBM_PEAK_GBS,
+                            "event pair around 100 back-to-back launches over 3 rotating inputs, median of three regions"),
+           "note": "copy_kernel_same_tensors is a plain 256 MiB -> 256 MiB copy (one 128-bit load and store per lane) timed in "
+                   "alternation with the softmax in this run: equal parts of reads and writes do not reach the 7.0 TB/s of a pure read stream"}
     if do_cpu:
         t1, tn = cpu_both(oracle, lambda: oracle.softmax(xh), n_thr)
         c3r.update(cpu_1core_GBs=round(2 * rows * 4096 * 2 / t1 / 1e9, 3), cpu_allcore_GBs=round(2 * rows * 4096 * 2 / tn / 1e9, 3),
@@ -621,10 +713,12 @@ def extras(all_cfg, ev, ops, _lib, oracle, args, np, torch, n_thr):
     gate(np.abs(fwd_out[0][0, -64:, 0].float().cpu().numpy() - o32[0, :, 0]).max() <= 2e-2 and
          np.abs(fwd_out[1][0, 0, -64:].cpu().numpy() - lse_ref[0, 0]).max() <= 2e-2, "c4 flash forward O / LSE (2e-2 absolute)")
     prewarm(c4_fwd)
-    r4 = time_ops(ev, [c4_fwd], steps, warm)
+    r4 = time_regions(ev, [c4_fwd], 100, warm)
     ms4 = r4["ms"]
     c4 = with_clock({"value": round(fl4 / (ms4 * 1e-3) / 1e12, 1), "unit": "TFLOP/s", "us_per_op": round(ms4 * 1e3, 1),
-                     "frac_of_mfma_peak": round(fl4 / (ms4 * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, 4), "flop": fl4},
+                     "frac_of_mfma_peak": round(fl4 / (ms4 * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, 4), "flop": fl4,
+                     "roofline": roof("mfma", "flash_fwd_kernel<_Float16, 128, 1, 8, false>", fl4, "flop", ms4, MFMA_PEAK_TFLOPS,
+                                      "event pair around 100 back-to-back calls, median of three regions")},
                     r4, MFMA_PEAK_TFLOPS, "frac_of_mfma_peak")
     if do_cpu:
         # the reference has no CPU attention; the naive oracle on one (batch, head) with 256
@@ -649,7 +743,7 @@ def extras(all_cfg, ev, ops, _lib, oracle, args, np, torch, n_thr):
     gate(np.abs(fwd_out[0][0, rows5, 0].float().cpu().numpy() - o32[0, :, 0]).max() <= 2e-2 and
          np.abs(fwd_out[1][0, 0, rows5].cpu().numpy() - lse_ref[0, 0]).max() <= 2e-2, "c5 flash forward O / LSE (2e-2 absolute)")
     prewarm(c5_fwd)
-    rf = time_ops(ev, [c5_fwd], steps, warm)
+    rf = time_regions(ev, [c5_fwd], 50, warm)
     msf = rf["ms"]
     o, lse = ops.flash_attn_fwd(q, k, v, 0.125, (-1, -1))
     bwd_out = ops.flash_attn_bwd_buffers(q, k, v)
@@ -670,16 +764,20 @@ def extras(all_cfg, ev, ops, _lib, oracle, args, np, torch, n_thr):
         ok = ok and worst[n] <= 2e-2 + 2.0 ** -8 * float(np.abs(ref).max())  # + 1 bf16 ulp of the largest value stored
     gate(ok, f"c5 flash backward dq/dk/dv (2e-2 absolute + 1 bf16 ulp of the largest value): {worst}")
     prewarm(c5_bwd)
-    rb = time_ops(ev, [c5_bwd], max(3, steps // 3), 2)
+    rb = time_regions(ev, [c5_bwd], 50, 2)
     msb = rb["ms"]
     all_cfg["c5_flash_fwd_bf16"] = with_clock({
         "value": round(fl5 / (msf * 1e-3) / 1e12, 1), "unit": "TFLOP/s", "us_per_op": round(msf * 1e3, 1),
-        "frac_of_mfma_peak": round(fl5 / (msf * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, 4), "flop": fl5}, rf, MFMA_PEAK_TFLOPS, "frac_of_mfma_peak")
+        "frac_of_mfma_peak": round(fl5 / (msf * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, 4), "flop": fl5,
+        "roofline": roof("mfma", "flash_fwd_kernel<__bf16, 64, 1, 8, false>", fl5, "flop", msf, MFMA_PEAK_TFLOPS,
+                         "event pair around 50 back-to-back calls, median of three regions")}, rf, MFMA_PEAK_TFLOPS, "frac_of_mfma_peak")
     flb = fl5 * 5 // 2
     all_cfg["c5_flash_bwd_bf16"] = with_clock({
         "value": round(flb / (msb * 1e-3) / 1e12, 1), "unit": "TFLOP/s", "us_per_op": round(msb * 1e3, 1),
         "frac_of_mfma_peak": round(flb / (msb * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, 4), "flop": flb,
         "gate_worst_abs_error": {n: round(e, 5) for n, e in worst.items()},
+        "roofline": roof("mfma", "dkdv_kernel<__bf16, 64, 1> + dq_kernel<__bf16, 64> + dot_do_o_kernel<__bf16, 64> (three launches per call)",
+                         fl5 * 5 // 2, "flop", msb, MFMA_PEAK_TFLOPS, "event pair around 50 back-to-back calls, median of three regions"),
         "note": "flop = 2.5 x forward (5 GEMMs); the kernels execute 7 (S and dP are recomputed by the dQ pass)"},
         rb, MFMA_PEAK_TFLOPS, "frac_of_mfma_peak")
     all_cfg["c5_flash_fwd_bwd_bf16"] = {
@@ -708,12 +806,15 @@ def extras(all_cfg, ev, ops, _lib, oracle, args, np, torch, n_thr):
     qd, kc, vc, kn, vn = mkd((b_, 1, h_, d_), 0), mkd((b_, sk_, hk_, d_), 1), mkd((b_, sk_, hk_, d_), 2), mkd((b_, 1, hk_, d_), 3), mkd((b_, 1, hk_, d_), 4)
     lens = torch.full((b_,), sk_ - 1, dtype=torch.int32, device="cuda")
     dec = lambda: ops.flash_attn_kvcache(qd, kc, vc, kn, vn, lens, 1.0 / np.sqrt(d_), (-1, -1))
-    rd = time_ops(ev, [dec], steps, warm)
+    rd = time_regions(ev, [dec], 50, warm)
     msd = rd["ms"]
     byt = 2 * b_ * sk_ * hk_ * d_ * 2
     all_cfg["kvcache_decode_fp16"] = {
         "value": round(byt / (msd * 1e-3) / 1e9, 1), "unit": "GB/s", "us_per_op": round(msd * 1e3, 1),
         "frac_of_hbm_peak": round(byt / (msd * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "algorithmic_bytes": byt,
+        **spread(rd, 1, 1),
+        "roofline": roof("hbm", "decode_kernel<_Float16, 128> (+ decode_merge_kernel)", byt, "bytes", msd, HBM_PEAK_GBS,
+                         "event pair around 50 back-to-back calls, median of three regions"),
         "note": "append kernel + decode kernel per call; bytes = K and V cache rows read once"}
 
 

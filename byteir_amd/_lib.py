@@ -66,6 +66,7 @@ def kernels():
         L.brt_rocm_reduce_workspace_bytes.restype = sz
         L.brt_rocm_reduce.argtypes = [i32, i32, vp, vp, sz, sz, sz, vp, sz, vp]
         L.brt_rocm_reduce_ex.argtypes = [i32, i32, vp, vp, sz, sz, sz, vp, sz, vp, vp]
+        L.brt_rocm_reduce_plan_describe.argtypes = [i32, sz, sz, sz, ctypes.c_char_p, sz]
         L.brt_rocm_reduce_static.argtypes = [i32, i32, vp, vp, sz, sz, sz, vp]
         L.brt_rocm_softmax.argtypes = [i32, vp, vp, sz, sz, vp]
         L.brt_rocm_softmax_axis.argtypes = [i32, vp, vp, sz, sz, sz, vp]

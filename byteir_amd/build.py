@@ -72,11 +72,24 @@ def build_index_check(verbose=False):
                                 os.path.join(CSRC, "flash_attn", "index_check.cc")], verbose)
 
 
-TARGETS = {"kernels": build_kernels, "flash": build_flash, "brt": build_brt, "index_check": build_index_check}
+def build_test_kernels(verbose=False):
+    """The external op-kernel library of the tests (tests/external_kernels/custom_add.hip, in the
+    style of the reference's runtime/test/external_kernels): built here, ahead of time, so that
+    the GPU tests only load it."""
+    src = os.path.join(ROOT, "tests", "external_kernels", "custom_add.hip")
+    if not os.path.exists(src):
+        return
+    _run([HIPCC] + HIP_FLAGS + [f"-I{os.path.join(CSRC, 'brt')}", "-o",
+                                os.path.join(ROOT, "tests", "external_kernels", "libcustom_add.so"), src,
+                                f"-L{LIB}", "-lbrt", "-lbrt_rocm_kernels", f"-Wl,-rpath,{LIB}"], verbose)
+
+
+TARGETS = {"kernels": build_kernels, "flash": build_flash, "brt": build_brt, "index_check": build_index_check,
+           "test_kernels": build_test_kernels}
 
 
 def build_all(verbose=False, targets=None):
-    for name in targets or ("kernels", "flash", "brt", "index_check"):
+    for name in targets or ("kernels", "flash", "brt", "index_check", "test_kernels"):
         TARGETS[name](verbose)
 
 

@@ -152,17 +152,60 @@ private:
 };
 
 // ---- work queues -----------------------------------------------------------------------------
+// A device pointer as op kernels see it (core/framework/value.h: AsyncValue is void *).
+using AsyncValue = void *;
+using AsyncValueRef = void *;
+namespace cuda {}  // sources written for the CUDA provider say `using namespace brt::cuda;`
+namespace rocm {}
+
+// Task kinds of a device work queue, with the reference's numbering
+// (include/brt/backends/cuda/device/cuda_work_queue.h:32-40); kernels written for the CUDA
+// provider pass them as plain integers.
+enum ROCMTaskType : int { kCompute = 0, kH2D = 1, kD2H = 2, kRecordEvent = 3, kWaitEvent = 4, kComputeDrv = 5, kD2D = 6 };
+using CUDATaskType = ROCMTaskType;
+
+// Launch extents as the args array of a kCompute task carries them: three 32-bit extents, the
+// layout of the CUDA / HIP dim3, so that a kernel source that includes <hip/hip_runtime.h> can
+// hand its own dim3 objects over.
+struct Dim3 {
+  unsigned x = 1, y = 1, z = 1;
+  Dim3() = default;
+  Dim3(unsigned x_, unsigned y_ = 1, unsigned z_ = 1) : x(x_), y(y_), z(z_) {}
+};
+// 1-D launch shape for `work_item` items, 256 per block (MakeCUDAGridAndBlock,
+// include/brt/backends/cuda/device/common/util.h:39-45)
+inline std::pair<Dim3, Dim3> MakeROCMGridAndBlock(int64_t work_item) {
+  return {Dim3((unsigned)((work_item + 255) / 256)), Dim3(256)};
+}
+inline std::pair<Dim3, Dim3> MakeCUDAGridAndBlock(int64_t work_item) { return MakeROCMGridAndBlock(work_item); }
+
 class WorkQueue {
 public:
   explicit WorkQueue(std::string name) : name_(std::move(name)) {}
   virtual ~WorkQueue() = default;
   const std::string &name() const { return name_; }
+  // Enqueue a call (core/context/work_queue.h:62-68).  kCompute: func is the host-side handle
+  // of a device function and args = {grid, block, dynamic LDS bytes (size_t), kernel
+  // argument 0, ...}, each a pointer to the value; kH2D / kD2H / kD2D: args = {dst, src, byte
+  // count}, each a pointer to the value.  op_id and dependency name the op and the ops it
+  // waits for; a single-stream queue orders by enqueueing and ignores them.
+  virtual common::Status AddTask(int task_type, const void *func, void **args, int op_id, const std::vector<int> &dependency) = 0;
+  // Enqueue a call on the host in queue order: `task` points to a std::function<void(void)>
+  // (what the DispatchHostTask macro below passes); the queue copies it.
+  virtual common::Status AddHostTask(const void *task, void **args, int op_id, const std::vector<int> &dependency) = 0;
+  // Enqueue through a functor, which is called immediately.
+  common::Status AddTask(std::function<common::Status()> enqueue_functor) { return enqueue_functor(); }
   virtual common::Status Sync() = 0;
   // device queues expose the stream kernels are enqueued on (void* == hipStream_t)
   virtual void *GetComputeStream() { return nullptr; }
 
+protected:
+  std::unordered_map<int, int> id_to_stream_map_;
+
 private:
   std::string name_;
+  WorkQueue(const WorkQueue &) = delete;
+  WorkQueue &operator=(const WorkQueue &) = delete;
 };
 
 // ---- events ----------------------------------------------------------------------------------
@@ -213,6 +256,7 @@ public:
     // creates the key's offset if needed, and this frame's state (by calling `make`) if the
     // frame has none at that offset
     common::Status CreateStateIfNotExist(const std::string &key, ExecutionFrame *frame, const std::function<void *()> &make);
+    void Clear();  // forgets every key (a session does this when it loads another model)
 
   private:
     std::mutex mutex_;
@@ -235,6 +279,7 @@ private:
   std::vector<std::pair<std::string, void *>> arenas_;  // one block per memory space for the intermediates
   const ir::ByREHandle *ir_ = nullptr;
   bool prologue_done_ = false;
+  size_t prologue_count_ = 0;       // kernels whose ProloguePerFrame has run on this frame (a prefix of the plan)
   bool io_bound_ = false;
 };
 
@@ -256,12 +301,16 @@ class ExecutionProvider;
 class OpKernelInfo {
 public:
   OpKernelInfo(const ExecutionProvider &provider, const ir::ByREHandle &ir, int op_index,
-               const std::unordered_map<std::string, std::unique_ptr<IAllocator>> &allocators)
-      : provider_(provider), ir_(ir), op_index_(op_index), allocators_(allocators) {}
+               const std::unordered_map<std::string, std::unique_ptr<IAllocator>> &allocators,
+               std::vector<int> dependency = {})
+      : provider_(provider), ir_(ir), op_index_(op_index), allocators_(allocators), dependency_(std::move(dependency)) {}
   const ExecutionProvider &GetExecutionProvider() const { return provider_; }
   const ir::ByREHandle &GetIR() const { return ir_; }
   const ir::Op &GetOp() const { return ir_.ops[op_index_]; }
   int GetOpId() const { return op_index_; }
+  // ids of the earlier ops whose results this op consumes, by the operands' memory effects
+  // (framework/op_kernel_info.h:95, computed as in execution_plan.cc:243-308)
+  const std::vector<int> &GetDependency() const { return dependency_; }
   IAllocator *GetAllocator(const std::string &space) const;
 
 private:
@@ -269,6 +318,7 @@ private:
   const ir::ByREHandle &ir_;
   int op_index_;
   const std::unordered_map<std::string, std::unique_ptr<IAllocator>> &allocators_;
+  std::vector<int> dependency_;
 };
 
 // Reads operands and attributes of one op; the only window op kernels have on the IR.
@@ -290,7 +340,7 @@ public:
   std::string GetUID() const;
   static int64_t GetNumElementsOfShape(const Shape &shape) { return LinearizedShape(shape); }
   // needs a frame
-  void *GetArgAsyncValueRef(size_t i) const;
+  AsyncValueRef GetArgAsyncValueRef(size_t i) const;
 
 private:
   const ir::Attr &Find(const std::string &name) const;
@@ -470,6 +520,8 @@ private:
   std::unordered_map<std::string, std::unique_ptr<IAllocator>> allocators_;
   std::unique_ptr<ir::ByREHandle> ir_;
   std::vector<std::shared_ptr<OpKernel>> kernels_;
+  std::vector<bool> session_prologue_done_;  // per kernel: ProloguePerSession has returned OK
+  void EndPlan() noexcept;                   // EpiloguePerSession of the kernels prepared so far, then drops the plan
   std::vector<std::unique_ptr<OpKernelInfo>> infos_;
   std::vector<size_t> in_offsets_, out_offsets_, weight_offsets_;
   // static memory plan of the memref.alloc intermediates: byte offset of each value inside the
@@ -496,3 +548,14 @@ common::Status DefaultROCMExecutionProviderFactory(Session *session, int device_
 common::Status ROCMAllocatorFactory(Session *session, int device_id = 0);
 
 }  // namespace brt
+
+// core/context/work_queue.h:91-101
+#define DispatchHostTask(wq, op_id, dependency, stmt)                                              \
+  if (wq) {                                                                                        \
+    std::function<void(void)> func = [=]() { stmt };                                               \
+    wq->AddHostTask(&func, nullptr, op_id, dependency);                                            \
+  } else {                                                                                         \
+    do {                                                                                           \
+      stmt                                                                                         \
+    } while (0);                                                                                   \
+  }

@@ -1,0 +1,7 @@
+// Forwarding header: the reference spreads its runtime interface over runtime/include/brt/backends/rocm/device/rocm_work_queue.h and
+// its neighbours; here one header (brt.h) holds it, and this path exists so that an op-kernel
+// source written against the reference's include lines compiles unchanged.
+#ifndef BRT_BACKENDS_ROCM_DEVICE_ROCM_WORK_QUEUE_H_
+#define BRT_BACKENDS_ROCM_DEVICE_ROCM_WORK_QUEUE_H_
+#include "../../../../brt.h"
+#endif

@@ -1,0 +1,7 @@
+// Forwarding header: the reference spreads its runtime interface over runtime/include/brt/core/framework/execution_provider.h and
+// its neighbours; here one header (brt.h) holds it, and this path exists so that an op-kernel
+// source written against the reference's include lines compiles unchanged.
+#ifndef BRT_CORE_FRAMEWORK_EXECUTION_PROVIDER_H_
+#define BRT_CORE_FRAMEWORK_EXECUTION_PROVIDER_H_
+#include "../../../brt.h"
+#endif

@@ -1,0 +1,7 @@
+// Forwarding header: the reference spreads its runtime interface over runtime/include/brt/core/framework/op_kernel_impl_base.h and
+// its neighbours; here one header (brt.h) holds it, and this path exists so that an op-kernel
+// source written against the reference's include lines compiles unchanged.
+#ifndef BRT_CORE_FRAMEWORK_OP_KERNEL_IMPL_BASE_H_
+#define BRT_CORE_FRAMEWORK_OP_KERNEL_IMPL_BASE_H_
+#include "../../../brt.h"
+#endif

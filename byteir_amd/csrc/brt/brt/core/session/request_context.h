@@ -1,0 +1,7 @@
+// Forwarding header: the reference spreads its runtime interface over runtime/include/brt/core/session/request_context.h and
+// its neighbours; here one header (brt.h) holds it, and this path exists so that an op-kernel
+// source written against the reference's include lines compiles unchanged.
+#ifndef BRT_CORE_SESSION_REQUEST_CONTEXT_H_
+#define BRT_CORE_SESSION_REQUEST_CONTEXT_H_
+#include "../../../brt.h"
+#endif

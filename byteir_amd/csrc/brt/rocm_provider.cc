@@ -82,8 +82,50 @@ public:
   }
   common::Status Sync() override { return HipStatus(brt_rocm_stream_synchronize(stream_), "stream synchronize"); }
   void *GetComputeStream() override { return stream_; }
+  // One stream: tasks run in the order they are enqueued, so op_id and dependency need no
+  // events here (CUDASingleStreamWorkQueue::AddTask, cuda_work_queue.cc:150-172).  There is no
+  // driver-API module loading in this provider, hence no kComputeDrv.
+  common::Status AddTask(int task_type, const void *func, void **args, int /*op_id*/, const std::vector<int> & /*dependency*/) override {
+    switch (task_type) {
+    case kCompute: {
+      BRT_ENFORCE(func != nullptr && args != nullptr, "kCompute needs a device function and {grid, block, shared bytes, arguments...}");
+      const Dim3 *grid = static_cast<const Dim3 *>(args[0]), *block = static_cast<const Dim3 *>(args[1]);
+      const size_t shared = *static_cast<const size_t *>(args[2]);
+      const unsigned g[3] = {grid->x, grid->y, grid->z}, b[3] = {block->x, block->y, block->z};
+      return HipStatus(brt_rocm_launch_kernel(func, g, b, args + 3, shared, stream_), "kernel launch");
+    }
+    case kH2D: case kD2H: case kD2D: {
+      BRT_ENFORCE(args != nullptr, "a copy task needs {dst, src, byte count}");
+      void *dst = *static_cast<void **>(args[0]), *src = *static_cast<void **>(args[1]);
+      const size_t count = *static_cast<const size_t *>(args[2]);
+      const int e = task_type == kH2D ? brt_rocm_memcpy_h2d(dst, src, count, stream_)
+                    : task_type == kD2H ? brt_rocm_memcpy_d2h(dst, src, count, stream_)
+                                        : brt_rocm_memcpy_d2d(dst, src, count, stream_);
+      return HipStatus(e, "copy task");
+    }
+    default:
+      return common::Status::Fail("unsupported task type " + std::to_string(task_type));
+    }
+  }
+  // The task is copied and runs on the host once everything enqueued before it has finished
+  // (hipLaunchHostFunc), so a task may read what earlier kernels wrote.  The reference's
+  // single-stream queue calls the function on the spot instead (cuda_work_queue.h:68-73) and
+  // its multi-stream queue enqueues it (cuda_work_queue.cc:258-264); the DispatchHostTask macro
+  // hands over a function object that dies with its scope, which is why it is copied here.
+  common::Status AddHostTask(const void *task, void ** /*args*/, int /*op_id*/, const std::vector<int> & /*dependency*/) override {
+    BRT_ENFORCE(task != nullptr, "AddHostTask needs a std::function<void(void)>");
+    auto *held = new std::function<void(void)>(*static_cast<const std::function<void(void)> *>(task));
+    const int e = brt_rocm_launch_host_func(stream_, &RocmWorkQueue::CallHostTask, held);
+    if (e != 0) delete held;
+    return HipStatus(e, "host task");
+  }
 
 private:
+  static void CallHostTask(void *task) {
+    auto *f = static_cast<std::function<void(void)> *>(task);
+    (*f)();
+    delete f;
+  }
   void *stream_;
   bool owned_;
 };
@@ -220,35 +262,33 @@ public:
       ext_dtype_ = c.dtype;
     }
     if (!with_ws_ || !last_error_ || (!bytes_ && !bwd_bytes_)) with_ws_ = nullptr;  // all or nothing
-  }
-  size_t GetWorkspaceSize(const ExecutionContext &) const override {
-    if (!with_ws_) return 0;
-    OpAccessor acc(info_);
-    void *extra = acc.GetAttrAsVoidPtr("extra_args");
-    size_t n = 0;
-    if (is_bwd_) {  // operand 11 is dq_accum (flash_api.cu:696-725): the library fills it first
-      const size_t accum = acc.GetNumArgs() > 11 ? (size_t)LinearizedShape(acc.GetArgShape(11)) * GetDTypeByte(acc.GetArgDTypeEnum(11)) : 0;
-      n = bwd_bytes_(extra, ext_dtype_, accum);
-    } else {
-      n = bytes_(extra, ext_dtype_);
+    // The packed extra_args blob and the scratch size depend on the op's attributes and static
+    // shapes only: both are made once here (the reference packs and frees the blob on every run,
+    // custom.cc:71-84; the libraries only read it) and live as long as the kernel.
+    extra_ = acc.GetAttrAsVoidPtr("extra_args");
+    if (with_ws_) {
+      if (is_bwd_) {  // operand 11 is dq_accum (flash_api.cu:696-725): the library fills it first
+        const size_t accum = acc.GetNumArgs() > 11 ? (size_t)LinearizedShape(acc.GetArgShape(11)) * GetDTypeByte(acc.GetArgDTypeEnum(11)) : 0;
+        ws_bytes_ = bwd_bytes_(extra_, ext_dtype_, accum);
+      } else {
+        ws_bytes_ = bytes_(extra_, ext_dtype_);
+      }
     }
-    std::free(extra);
-    return n;
   }
+  ~CustomOpKernel() override { std::free(extra_); }
+  size_t GetWorkspaceSize(const ExecutionContext &) const override { return ws_bytes_; }
   common::Status RunImpl(const ExecutionContext &ctx) override {
     OpAccessor acc(info_, ctx.exec_frame);
     std::vector<void *> tensors(acc.GetNumArgs());
     for (size_t i = 0; i < tensors.size(); ++i) tensors[i] = acc.GetArgAsyncValueRef(i);
-    void *extra = acc.GetAttrAsVoidPtr("extra_args");
     common::Status st = common::Status::OK();
     if (with_ws_) {
-      const int e = with_ws_(tensors.data(), extra, ext_dtype_, GetWorkspace(ctx), GetWorkspaceSize(ctx), StreamOf(ctx));
+      const int e = with_ws_(tensors.data(), extra_, ext_dtype_, GetWorkspace(ctx), ws_bytes_, StreamOf(ctx));
       if (e < 0) st = common::Status::Fail(std::string("custom op: ") + last_error_());
       else if (e > 0) st = HipStatus(e, "custom op launch");
     } else {
-      run_(tensors.data(), extra, StreamOf(ctx));
+      run_(tensors.data(), extra_, StreamOf(ctx));
     }
-    std::free(extra);
     return st;
   }
 
@@ -279,6 +319,8 @@ private:
   LastErrorFn last_error_ = nullptr;
   bool is_bwd_ = false;
   int ext_dtype_ = 0;
+  void *extra_ = nullptr;  // the packed extra_args blob (malloc'ed by the accessor)
+  size_t ws_bytes_ = 0;
 };
 
 // ---- copies: cpu2cuda, cuda2cpu, cuda2cuda (operands: src, dst) ---------------------------------------------

@@ -267,11 +267,24 @@ common::Status ExecutionFrame::StateInfo::CreateStateIfNotExist(const std::strin
   return common::Status::OK();
 }
 
+void ExecutionFrame::StateInfo::Clear() {
+  std::lock_guard<std::mutex> lock(mutex_);
+  name_to_offset_.clear();
+}
+
 // ---- session ------------------------------------------------------------------------------------------
 Session::Session() = default;
-Session::~Session() {
-  for (auto &k : kernels_)
-    if (k->HasEpiloguePerSession()) { try { k->EpiloguePerSession(); } catch (...) {} }
+Session::~Session() { EndPlan(); }
+
+// The per-session epilogue belongs to the kernels whose per-session prologue has run (a kernel
+// that was constructed but never prepared, because an earlier one failed, is only destroyed).
+void Session::EndPlan() noexcept {
+  for (size_t i = 0; i < kernels_.size(); ++i) {
+    const bool prepared = !kernels_[i]->HasProloguePerSession() || (i < session_prologue_done_.size() && session_prologue_done_[i]);
+    if (prepared && kernels_[i]->HasEpiloguePerSession()) { try { kernels_[i]->EpiloguePerSession(); } catch (...) {} }
+  }
+  kernels_.clear();
+  session_prologue_done_.clear();
 }
 
 common::Status Session::AddExecutionProvider(std::unique_ptr<ExecutionProvider> provider) {
@@ -307,9 +320,8 @@ common::Status Session::LoadFromMemory(const std::string &text, const std::strin
 // kernels (shape checks and dlopen happen here), as StaticBRTExecutionPlan::ProloguePerSession
 // does (execution_plan.cc:314-438).
 common::Status Session::BuildPlan() {
-  for (auto &k : kernels_)  // a model loaded earlier ends here
-    if (k->HasEpiloguePerSession()) { try { k->EpiloguePerSession(); } catch (...) {} }
-  kernels_.clear();
+  EndPlan();  // a model loaded earlier ends here
+  frame_state_info_.Clear();  // its per-frame state keys and offsets do not carry over
   infos_.clear();
   in_offsets_.clear(); out_offsets_.clear(); weight_offsets_.clear();
   for (size_t i = 0; i < ir_->args.size(); ++i) {
@@ -339,13 +351,36 @@ common::Status Session::BuildPlan() {
       total += (val.type.Bytes() + kAllocAlignment - 1) / kAllocAlignment * kAllocAlignment;
     }
   }
+  // Op dependencies (execution_plan.cc:243-308): an op depends on the last writer of every
+  // operand it reads.  memory_effects names read (1), write (2) or both per operand; without
+  // it every operand counts as read and written; a copy reads operand 0 and writes operand 1.
+  std::vector<std::vector<int>> dependency(ir_->ops.size());
+  {
+    std::unordered_map<int, int> last_writer;  // value id -> op id
+    for (size_t i = 0; i < ir_->ops.size(); ++i) {
+      const ir::Op &op = ir_->ops[i];
+      auto fx = op.attrs.find("memory_effects");
+      const bool is_copy = op.name == "byre.copy";
+      for (size_t k = 0; k < op.operands.size(); ++k) {
+        int effect = 3;
+        if (is_copy) effect = k == 0 ? 1 : 2;
+        else if (fx != op.attrs.end() && fx->second.elems.size() == op.operands.size()) effect = (int)fx->second.elems[k].i;
+        const int v = op.operands[k];
+        if (effect & 1) {
+          auto w = last_writer.find(v);
+          if (w != last_writer.end()) dependency[i].push_back(w->second);
+        }
+        if (effect & 2) last_writer[v] = (int)i;
+      }
+    }
+  }
   for (size_t i = 0; i < ir_->ops.size(); ++i) {
     const std::string &key = ir_->ops[i].key;
     ExecutionProvider *chosen = nullptr;
     for (auto &p : providers_)
       if (p->GetKernelRegistry()->HasKernel(key)) { chosen = p.get(); break; }
     if (!chosen) return common::Status::Fail("No providers support Op " + key);
-    infos_.emplace_back(new OpKernelInfo(*chosen, *ir_, (int)i, allocators_));
+    infos_.emplace_back(new OpKernelInfo(*chosen, *ir_, (int)i, allocators_, dependency[i]));
     try {
       std::shared_ptr<OpKernel> k = (*chosen->GetKernelRegistry())(key, *infos_.back());
       if (!k) return common::Status::Fail("kernel factory returned null for " + key);
@@ -356,10 +391,12 @@ common::Status Session::BuildPlan() {
   }
   // one-time preparation of the kernels that ask for it (the reference calls this from
   // Session::Load through ExecutionPlan::ProloguePerSession, execution_plan.cc:313-330)
-  for (auto &k : kernels_) {
-    if (!k->HasProloguePerSession()) continue;
-    common::Status s = k->ProloguePerSession();
+  session_prologue_done_.assign(kernels_.size(), false);
+  for (size_t i = 0; i < kernels_.size(); ++i) {
+    if (!kernels_[i]->HasProloguePerSession()) continue;
+    common::Status s = kernels_[i]->ProloguePerSession();
     if (!s.IsOK()) return s;
+    session_prologue_done_[i] = true;
   }
   return common::Status::OK();
 }
@@ -405,10 +442,26 @@ common::Status Session::Run(RequestContext &request) {
   if (!f.io_bound_) return common::Status::Fail("FinishIOBinding has not been called");
   ExecutionContext ctx(&f, request.wq_.get(), frame_state_info_, &request.events_);
   if (!f.prologue_done_) {  // first run of this frame: workspaces (op_kernel_impl_base.h:116-136)
-    for (auto &k : kernels_) {
-      if (!k->HasProloguePerFrame()) continue;
-      common::Status s = k->ProloguePerFrame(ctx);
-      if (!s.IsOK()) return s;
+    // A prologue that fails part-way (a status, or an exception from an allocator) leaves the
+    // kernels before it prepared: prologue_count_ records how far it got, so that Cleanup
+    // releases exactly their workspaces, and the next Run starts over from the first kernel
+    // after releasing them.
+    if (f.prologue_count_ > 0) {
+      for (size_t i = 0; i < f.prologue_count_ && i < kernels_.size(); ++i)
+        if (kernels_[i]->HasEpiloguePerFrame()) { try { kernels_[i]->EpiloguePerFrame(ctx); } catch (...) {} }
+      f.prologue_count_ = 0;
+    }
+    for (size_t i = 0; i < kernels_.size(); ++i) {
+      if (kernels_[i]->HasProloguePerFrame()) {
+        common::Status s;
+        try {
+          s = kernels_[i]->ProloguePerFrame(ctx);
+        } catch (const std::exception &e) {
+          s = common::Status::Fail(std::string("ProloguePerFrame: ") + e.what());
+        }
+        if (!s.IsOK()) return s;
+      }
+      f.prologue_count_ = i + 1;
     }
     f.prologue_done_ = true;
   }
@@ -425,13 +478,12 @@ void Session::Cleanup(RequestContext &request) noexcept {
   ExecutionFrame &f = *request.frame_;
   ExecutionContext ctx(&f, request.wq_.get(), frame_state_info_, nullptr);
   if (request.wq_) request.wq_->Sync();
-  if (f.prologue_done_) {
-    for (auto &k : kernels_) {
-      if (!k->HasEpiloguePerFrame()) continue;
-      try { k->EpiloguePerFrame(ctx); } catch (...) {}
-    }
-    f.prologue_done_ = false;
+  for (size_t i = 0; i < f.prologue_count_ && i < kernels_.size(); ++i) {  // also after a prologue that failed part-way
+    if (!kernels_[i]->HasEpiloguePerFrame()) continue;
+    try { kernels_[i]->EpiloguePerFrame(ctx); } catch (...) {}
   }
+  f.prologue_count_ = 0;
+  f.prologue_done_ = false;
   for (size_t i = 0; i < f.base_.size(); ++i) {
     if (f.owned_[i] && f.base_[i]) {
       if (IAllocator *a = GetAllocator(ir_->values[i].type.space)) a->Free(f.base_[i]);

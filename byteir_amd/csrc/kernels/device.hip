@@ -6,6 +6,7 @@
 #include <cstdint>
 
 #include "brt_rocm_kernels.h"
+#include "brt_rocm_bench.h"
 
 namespace {
 // grid-stride 128-bit copy; n16 = number of 16-byte words
@@ -78,6 +79,19 @@ int brt_rocm_memset(void *dst, int value, size_t bytes, void *stream) {
   fill_bytes_kernel<<<dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(
       static_cast<unsigned char *>(dst), (unsigned)value & 0xffu, bytes);
   return hipGetLastError();
+}
+
+int brt_rocm_launch_kernel(const void *func, const unsigned grid[3], const unsigned block[3],
+                           void **kernel_args, size_t shared_bytes, void *stream) {
+  if (!func || !grid || !block) return hipErrorInvalidValue;
+  if (grid[0] == 0 || grid[1] == 0 || grid[2] == 0) return hipSuccess;  // nothing to do
+  return hipLaunchKernel(func, dim3(grid[0], grid[1], grid[2]), dim3(block[0], block[1], block[2]), kernel_args,
+                         shared_bytes, static_cast<hipStream_t>(stream));
+}
+
+int brt_rocm_launch_host_func(void *stream, void (*fn)(void *), void *arg) {
+  if (!fn) return hipErrorInvalidValue;
+  return hipLaunchHostFunc(static_cast<hipStream_t>(stream), fn, arg);
 }
 
 int brt_rocm_stream_create(void **stream) {

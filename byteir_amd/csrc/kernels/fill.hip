@@ -17,6 +17,7 @@
 #include <cstdint>
 
 #include "brt_rocm_kernels.h"
+#include "brt_rocm_bench.h"
 
 namespace {
 

@@ -21,11 +21,13 @@
 #include <hip/hip_runtime.h>
 
 #include <atomic>
+#include <cstdio>
 
 #include <cstdint>
 #include <type_traits>
 
 #include "brt_rocm_kernels.h"
+#include "brt_rocm_bench.h"
 
 namespace {
 
@@ -462,6 +464,23 @@ hipError_t run(const T *in, T *out, uint64_t A, uint64_t B, uint64_t C, void *ws
 }
 
 }  // namespace
+
+// The first-pass kernel a fold of 16-byte aligned tensors is planned with, spelled the way a
+// profiler prints the instantiation (the operator as OP), and the split: what a stored counter
+// profile must name to be valid for today's library.
+extern "C" int brt_rocm_reduce_plan_describe(int dtype, size_t A, size_t B, size_t C, char *buf, size_t len) {
+  if (!buf || len == 0 || (dtype != BRT_ROCM_F32 && dtype != BRT_ROCM_F16)) return hipErrorInvalidValue;
+  const Plan p = make_plan(dtype, A, B, C, true);
+  const char *t = dtype == BRT_ROCM_F32 ? "float" : "__half";
+  const char *to = p.S > 1 ? "float" : t;
+  const int vf = dtype == BRT_ROCM_F32 ? 4 : 8;
+  int n = 0;
+  if (p.kind == 1) n = snprintf(buf, len, "reduce_row_kernel<%s, %s, OP, %d, %d, %s> S=%u", t, to, vf, p.g, p.vec > 1 ? "false" : "true", p.S);
+  else if (p.kind == 3) n = snprintf(buf, len, "reduce_colwide_kernel<%s, %s, OP, %d, %d, %d> S=%u col_tiles=%u", t, to, vf, p.g / kBlock, kColWideU, p.S, p.col_tiles);
+  else if (p.kind == 2) n = snprintf(buf, len, "reduce_col_kernel<%s, %s, OP, %d, %d> S=%u col_tiles=%u", t, to, p.vec > 1 ? vf : 1, p.g, p.S, p.col_tiles);
+  else n = snprintf(buf, len, "copy or fill");
+  return n > 0 && (size_t)n < len ? 0 : hipErrorInvalidValue;
+}
 
 extern "C" size_t brt_rocm_reduce_workspace_bytes(int dtype, size_t A, size_t B, size_t C) {
   if (dtype != BRT_ROCM_F32 && dtype != BRT_ROCM_F16) return 0;

@@ -62,34 +62,22 @@ int brt_rocm_memcpy_h2d(void *dst, const void *src, size_t bytes, void *stream);
 int brt_rocm_memcpy_d2h(void *dst, const void *src, size_t bytes, void *stream);
 int brt_rocm_memcpy_d2d(void *dst, const void *src, size_t bytes, void *stream);
 int brt_rocm_memset(void *dst, int value, size_t bytes, void *stream); /* a fill kernel, safe to capture in a HIP graph */
-/* device-to-device copy done by a plain compute kernel (128-bit loads and stores) rather than
- * a DMA engine: the cuda2cuda copy of runtime/lib/backends/cuda/providers/default/copy/copy.cc
- * for buffers that are multiples of 16 bytes and 16-byte aligned, and the known-traffic
- * reference launch against which hardware byte counters are scaled. */
-int brt_rocm_copy_kernel(void *dst, const void *src, size_t bytes, void *stream);
+/* Launches a device function by its host-side handle (what `&kernel<...>` yields in a HIP
+ * translation unit): grid and block are three extents each, kernel_args one pointer per kernel
+ * parameter.  What WorkQueue::AddTask(kCompute, ...) enqueues; stands in for the cudaLaunchKernel
+ * of CUDAWorkQueue's Compute (runtime/lib/backends/cuda/device/cuda_work_queue.cc:59-67). */
+int brt_rocm_launch_kernel(const void *func, const unsigned grid[3], const unsigned block[3],
+                           void **kernel_args, size_t shared_bytes, void *stream);
+/* Enqueues fn(arg) on the host in stream order (cudaLaunchHostFunc in ComputeHost,
+ * cuda_work_queue.cc:98-102); fn must not call into the HIP runtime. */
+int brt_rocm_launch_host_func(void *stream, void (*fn)(void *), void *arg);
 int brt_rocm_stream_create(void **stream);
 int brt_rocm_stream_destroy(void *stream);
 int brt_rocm_stream_synchronize(void *stream);
 int brt_rocm_device_synchronize(void);
-/* events, for timing a launch on the stream it runs on */
-int brt_rocm_event_create(void **event);
-int brt_rocm_event_destroy(void *event);
-int brt_rocm_event_record(void *event, void *stream);
-int brt_rocm_event_synchronize(void *event);
-int brt_rocm_event_elapsed_ms(float *ms, void *start, void *stop);
-
-/* ---- synthetic data -------------------------------------------------------------- */
-/* Fills `n` elements with a counter-based pseudo-random sequence: element i depends on
- * (seed, i) only -- splitmix64 output number i (uniform) or 3i .. 3i + 2 (normal) -- through
- * integer arithmetic and exact float operations, so a host restatement of the same lines gives
- * the same bits (the benchmark's and the tests' CPU side generates its own copy instead of
- * reading the buffer back).  BRT_ROCM_FILL_UNIFORM: x = fma(u, b - a, a), u = 24 random bits
- * * 2^-24 in [0, 1).  BRT_ROCM_FILL_NORMAL: x = b * (sum of twelve 16-bit fields - 393210) *
- * 2^-16, mean 0 and standard deviation b (twelve-term central limit, support +-6 b); a unused.
- * Stored as f32 / f16 / bf16 with round-to-nearest-even.  The reference has no counterpart: its
- * tests fill buffers on the host (runtime/test/include/brt/test/common/util.h). */
-enum { BRT_ROCM_FILL_UNIFORM = 0, BRT_ROCM_FILL_NORMAL = 1 };
-int brt_rocm_fill(int dtype, int dist, uint64_t seed, void *ptr, size_t n, float a, float b, void *stream);
+/* Measurement and test tooling that the same library exports (the benchmark's data generator,
+ * event timing, a copy kernel of known traffic, a reduce call with a timing hook) is declared in
+ * brt_rocm_bench.h: none of it stands in for a reference interface. */
 
 /* ---- reductions ------------------------------------------------------------------ */
 /* out[a, c] = fold_b in[a, b, c] for a dense row-major tensor viewed as [A, B, C];
@@ -112,14 +100,6 @@ int brt_rocm_fill(int dtype, int dist, uint64_t seed, void *ptr, size_t n, float
 size_t brt_rocm_reduce_workspace_bytes(int dtype, size_t A, size_t B, size_t C);
 int brt_rocm_reduce(int op, int dtype, const void *input, void *output, size_t A, size_t B,
                     size_t C, void *workspace, size_t workspace_bytes, void *stream);
-/* The same call with a timing hook: `first_pass_done`, when not NULL, is a hipEvent_t that is
- * recorded on `stream` right after the first (or only) pass has been enqueued, so that a caller
- * can time the split first pass apart from the combine pass.  No counterpart in the reference
- * (its hooks are host-side Before/AfterOpKernelRun events, framework/event.h:27-74). */
-int brt_rocm_reduce_ex(int op, int dtype, const void *input, void *output, size_t A, size_t B,
-                       size_t C, void *workspace, size_t workspace_bytes, void *stream,
-                       void *first_pass_done);
-
 /* The same fold for callers that must not allocate and have no workspace to hand over (code
  * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
  * counterpart in the reference, whose ReduceImpl always takes its workspace from the frame's

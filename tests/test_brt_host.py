@@ -28,7 +28,7 @@ def exported_functions(header):
     return sorted(set(n for n in names if not n.endswith("_fn") and n != "brt_op_listener"))
 
 
-@pytest.mark.parametrize("header,loader", [("brt_rocm_kernels.h", "kernels"), ("flash_api.h", "flash_attn"), ("brt_c_api.h", "brt")])
+@pytest.mark.parametrize("header,loader", [("brt_rocm_kernels.h", "kernels"), ("brt_rocm_bench.h", "kernels"), ("flash_api.h", "flash_attn"), ("brt_c_api.h", "brt")])
 def test_c_abi_exports_every_declared_symbol(header, loader):
     from byteir_amd import _lib
     L = getattr(_lib, loader)()
@@ -335,3 +335,66 @@ def test_missing_kernel_library_fails_loudly(tmp_path, monkeypatch):
             fresh.flash_attn()
     finally:
         importlib.reload(_lib)
+
+
+def test_op_dependencies_follow_the_memory_effects():
+    """OpKernelInfo::GetDependency (framework/op_kernel_info.h:95) as the reference computes it
+    (execution_plan.cc:243-308): an op depends on the last writer of each operand it reads;
+    without memory_effects every operand counts as read and written.  Seen through a kernel
+    compiled against brt.h with the reference's include paths (no GPU: plan-only session)."""
+    import subprocess, tempfile, ctypes
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    src = r'''
+#include "brt/core/framework/op_kernel.h"
+#include "brt/core/framework/op_kernel_info.h"
+#include "brt/core/framework/kernel_registry.h"
+#include "brt/core/context/work_queue.h"
+#include "brt/backends/common.h"
+using namespace brt;
+static int g_deps[16][4], g_ndeps[16], g_nops = 0;
+extern "C" int dep_nops() { return g_nops; }
+extern "C" int dep_count(int op) { return g_ndeps[op]; }
+extern "C" int dep_at(int op, int k) { return g_deps[op][k]; }
+namespace {
+class Probe final : public OpKernel {
+public:
+  explicit Probe(const OpKernelInfo &info) : OpKernel(info, false, false, false, false) {
+    const int id = info.GetOpId();
+    g_ndeps[id] = (int)info.GetDependency().size();
+    for (int k = 0; k < g_ndeps[id] && k < 4; ++k) g_deps[id][k] = info.GetDependency()[(size_t)k];
+    if (id + 1 > g_nops) g_nops = id + 1;
+  }
+  common::Status RunImpl(const ExecutionContext &) override { return common::Status::OK(); }
+};
+BRT_STATIC_KERNEL_REGISTRATION(DeviceKind::ROCM, ProviderType::BRT, [](KernelRegistry *registry) {
+  registry->Register("ProbeOp", [](const brt::OpKernelInfo &info) -> std::shared_ptr<OpKernel> { return std::make_shared<Probe>(info); });
+});
+}
+'''
+    from byteir_amd import _lib, brt
+    with tempfile.TemporaryDirectory() as tmp:
+        cc, so = os.path.join(tmp, "probe.cc"), os.path.join(tmp, "libprobe.so")
+        open(cc, "w").write(src)
+        libdir = os.path.join(root, "byteir_amd", "lib")
+        subprocess.run(["g++", "-std=c++17", "-O1", "-shared", "-fPIC", f"-I{os.path.join(root, 'byteir_amd', 'csrc', 'brt')}",
+                        f"-I{os.path.join(root, 'include')}", cc, "-o", so, f"-L{libdir}", "-lbrt", f"-Wl,-rpath,{libdir}"], check=True)
+        assert _lib.brt().brt_register_kernels_from_dynlib(so.encode()) == 0
+        ext = ctypes.CDLL(so)
+        s = brt.Session(device="ROCM", device_id=-1)  # plan only: no GPU needed
+        try:
+            t = 'memref<8xf32, "cuda">'
+            s.load_from_memory(f"""func.func @t(%a : {t} {{byre.argname = "a", byre.argtype = 1: i32}},
+                         %b : {t} {{byre.argname = "b", byre.argtype = 2: i32}},
+                         %c : {t} {{byre.argname = "c", byre.argtype = 2: i32}}) attributes {{byre.entry_point}} {{
+              byre.compute @ProbeOp(%a, %b) {{memory_effects = [1 : i32, 2 : i32]}} : {t}, {t}
+              byre.compute @ProbeOp(%a, %c) {{memory_effects = [1 : i32, 2 : i32]}} : {t}, {t}
+              byre.compute @ProbeOp(%b, %c) {{memory_effects = [1 : i32, 3 : i32]}} : {t}, {t}
+              byre.compute @ProbeOp(%a, %b) : {t}, {t}
+              return }}""")
+            assert ext.dep_nops() == 4
+            deps = [[ext.dep_at(i, k) for k in range(ext.dep_count(i))] for i in range(4)]
+            # op 0 and 1 read only %a (an input: no writer); op 2 reads %b (op 0) and reads+writes %c (op 1);
+            # op 3 has no memory_effects: %a never written -> none, %b last written by op 0
+            assert deps == [[], [], [0, 1], [0]], deps
+        finally:
+            s.close()

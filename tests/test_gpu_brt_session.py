@@ -530,6 +530,48 @@ def test_reference_style_external_kernel_runs_with_its_hooks(tmp_path):
         s.close()
 
 
+def test_external_kernel_in_the_reference_launch_idiom():
+    """tests/external_kernels/custom_add.hip (built ahead of time by byteir_amd.build): a
+    __global__ function handed to WorkQueue::AddTask with {grid, block, shared bytes, arguments},
+    the op id and GetDependency() -- the launch idiom of runtime/test/external_kernels/cuda/
+    kernels.cc:52-79 -- plus a host task through DispatchHostTask.  Two chained adds: the second
+    op reads what the first wrote, so its dependency list names the first."""
+    import ctypes
+    from byteir_amd import _lib, brt
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    lib = os.path.join(root, "tests", "external_kernels", "libcustom_add.so")
+    assert os.path.exists(lib), "run python -m byteir_amd.build test_kernels"
+    assert _lib.brt().brt_register_kernels_from_dynlib(lib.encode()) == 0
+    ext = ctypes.CDLL(lib)
+    s = brt.Session(device="ROCM")
+    try:
+        t = 'memref<5000xf32, "cuda">'
+        s.load_from_memory(f"""func.func @t(%a : {t} {{byre.argname = "a", byre.argtype = 1: i32}},
+                     %b : {t} {{byre.argname = "b", byre.argtype = 1: i32}},
+                     %c : {t} {{byre.argname = "c", byre.argtype = 2: i32}},
+                     %d : {t} {{byre.argname = "d", byre.argtype = 2: i32}}) attributes {{byre.entry_point}} {{
+          byre.compute @CustomAddOp(%a, %b, %c) {{memory_effects = [1 : i32, 1 : i32, 2 : i32]}} : {t}, {t}, {t}
+          byre.compute @CustomAddOp(%c, %b, %d) {{memory_effects = [1 : i32, 1 : i32, 2 : i32]}} : {t}, {t}, {t}
+          return }}""")
+        assert ext.ext_add_prologue_per_session() >= 2
+        f0, h0 = ext.ext_add_prologue_per_frame(), ext.ext_add_host_tasks()
+        gen = torch.Generator(device="cuda").manual_seed(7)
+        a, b = (torch.randn(5000, generator=gen, device="cuda") for _ in range(2))
+        c, d = torch.zeros(5000, device="cuda"), torch.zeros(5000, device="cuda")
+        req = s.new_request_context()
+        for i, x in enumerate((a, b, c, d)):
+            req.bind_arg(i, x.data_ptr())
+        req.finish_io_binding()
+        req.run(); req.sync()
+        assert torch.equal(c, a + b) and torch.equal(d, (a + b) + b)
+        assert ext.ext_add_prologue_per_frame() == f0 + 2          # once per op and frame
+        assert ext.ext_add_host_tasks() == h0 + 2                  # the host tasks ran, in queue order, before sync returned
+        assert ext.ext_add_last_op_id() == 1 and ext.ext_add_last_dependency_count() == 1  # op 1 waits for op 0 (%c)
+        req.close()
+    finally:
+        s.close()
+
+
 def test_custom_op_with_unsupported_arguments_fails_the_run(session, golden_dir):
     """head_dim 20 is not a multiple of 8: through the plain ABI the library would abort the
     process; the custom op kernel uses the library's error-returning entry point instead."""

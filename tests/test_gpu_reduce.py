@@ -8,6 +8,7 @@ import pytest
 import torch
 
 import oracle
+from reduce_exact import exact_fold, exact_input
 from gpu_util import dev, host
 
 pytestmark = pytest.mark.gpu
@@ -109,28 +110,18 @@ OTHER_SHAPES = REF_CASES + [
 ]
 
 
-def exact_input(op, shape, dims, rng):
-    """Values for which every partial result of the fold is exact in float whatever the order,
-    so that the sequential oracle is the expected value bit for bit: small integers for
-    min / mean / sum of squares; for the product, signs and a few factors of 2 and 1/2."""
-    if op != oracle.PROD:
-        return rng.integers(-2, 3, size=shape).astype(np.float32)
-    fold = int(np.prod([shape[d] for d in dims]))
-    e = rng.integers(-1, 2, size=shape) * (rng.random(shape) < min(1.0, 24.0 / fold))
-    return (np.exp2(e) * rng.choice(np.array([-1.0, 1.0]), size=shape)).astype(np.float32)
-
-
 @pytest.mark.parametrize("shape,dims", OTHER_SHAPES)
 @pytest.mark.parametrize("op", OTHER_OPS)
 @pytest.mark.parametrize("dtype", [np.float32, np.float16])
 def test_other_operators_bit_exact_on_exact_inputs(shape, dims, op, dtype):
     from byteir_amd import ops
-    if dtype == np.float16 and int(np.prod(shape)) > (1 << 22):
-        pytest.skip("the scalar f16 oracle is slow at this size; f32 covers the shape")
     rng = np.random.default_rng(abs(hash((shape, dims, op))) % (2 ** 32))
     x = exact_input(op, shape, dims, rng).astype(dtype)
     got = host(ops.reduce(op, dev(x), dims))
-    want = oracle.reduce_op(op, x, dims)
+    if dtype == np.float16 and int(np.prod(shape)) > (1 << 22):
+        want = exact_fold(op, x, dims)  # the scalar f16 oracle takes minutes at this size
+    else:
+        want = oracle.reduce_op(op, x, dims)
     assert got.dtype == dtype and got.shape == want.shape
     assert np.array_equal(got, want)
 

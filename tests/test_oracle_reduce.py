@@ -197,3 +197,16 @@ def test_tensors_without_elements():
     assert np.all(np.isnan(oracle.reduce_op(oracle.MEAN, x, (1,))))
     assert oracle.reduce_op(oracle.SUM, np.empty((0, 5), np.float32), (1,)).shape == (0,)
     assert oracle.reduce_op(oracle.SUM, np.empty((3, 5, 0), np.float32), (1,)).shape == (3, 0)
+
+
+@pytest.mark.parametrize("shape,dims", [((7, 13), (1,)), ((5, 333, 7), (1,)), ((4096, 64), (0,)), ((300, 2600), (0,)), ((16, 2049, 260), (1,))])
+@pytest.mark.parametrize("op", [oracle.MIN, oracle.PROD, oracle.MEAN, oracle.SUMSQR])
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_integer_arithmetic_fold_agrees_with_the_oracle(shape, dims, op, dtype):
+    """exact_fold (numpy integer arithmetic) is what the GPU tests compare the large f16 shapes
+    with, where the scalar oracle would take minutes: on the shapes the oracle does finish, the
+    two must agree bit for bit."""
+    from reduce_exact import exact_fold, exact_input
+    rng = np.random.default_rng(abs(hash((shape, dims, op))) % (2 ** 32))
+    x = exact_input(op, shape, dims, rng).astype(dtype)
+    assert np.array_equal(exact_fold(op, x, dims), oracle.reduce_op(op, x, dims))
