@@ -125,6 +125,19 @@ template <int OP> __device__ __forceinline__ float wave_fold(float r, int width)
   return r;
 }
 
+// Workgroup ids go round-robin over the 8 XCDs of the chip; this gives each XCD a contiguous
+// eighth of the launch instead of every eighth workgroup.
+#ifndef REDUCE_XCD_CONTIG
+#define REDUCE_XCD_CONTIG 1
+#endif
+__device__ __forceinline__ uint32_t xcd_contiguous(uint32_t b, uint32_t n) {
+#if REDUCE_XCD_CONTIG
+  return (n & 7u) == 0 ? (b & 7u) * (n >> 3) + (b >> 3) : b;
+#else
+  return b;
+#endif
+}
+
 // ---- rows: C == 1 -----------------------------------------------------------------------
 // unit = a * S + s; G lanes fold in[a, s*seg_len : min(B, (s+1)*seg_len)] into out[unit].
 // PEEL: the segment may start and end anywhere (a row length that is no multiple of the vector,
@@ -137,7 +150,7 @@ reduce_row_kernel(const T *__restrict__ in, TO *__restrict__ out, uint64_t units
   constexpr int GPB = kBlock / G;
   constexpr int U = kRowU;
   const int lane = threadIdx.x % G;
-  uint64_t unit = (uint64_t)blockIdx.x * GPB + threadIdx.x / G;
+  uint64_t unit = (uint64_t)xcd_contiguous(blockIdx.x, gridDim.x) * GPB + threadIdx.x / G;
   const bool valid = unit < units;
   if (!valid) unit = units - 1;  // surplus groups redo the last unit so shuffles stay whole
   const uint64_t a = unit / S, s = unit % S;
@@ -257,7 +270,7 @@ template <typename T, typename TO, int OP, int VEC, int W, int U>
 __global__ void __launch_bounds__(kBlock)
 reduce_colwide_kernel(const T *__restrict__ in, TO *__restrict__ out, uint64_t B, uint64_t C,
                       uint32_t S, uint64_t seg_rows, uint32_t col_tiles, float len) {
-  uint64_t bid = blockIdx.x;
+  uint64_t bid = xcd_contiguous(blockIdx.x, gridDim.x);
   const uint32_t tile = bid % col_tiles; bid /= col_tiles;
   const uint32_t s = bid % S;
   const uint64_t a = bid / S;
