@@ -698,6 +698,37 @@ def extras(all_cfg, ev, ops, _lib, oracle, args, np, torch, n_thr):
         t = t.view(np.float16) if code == 1 else t
         return np.ascontiguousarray(t if rows is None else t[:, rows])
 
+    # What a matrix-instruction stream reaches on this box: nothing but v_mfma_f32_32x32x16 on
+    # operands held in registers, once on zeros (the issue peak at the boost clock) and once on
+    # N(0,1) operands like the attention inputs (the chip lowers its clock under the toggling
+    # operand bits).  The second is the ceiling for any kernel that is fed such data.
+    mf_blocks, mf_iters = torch.cuda.get_device_properties(0).multi_processor_count, 8000
+    mf_ops = torch.empty(mf_blocks * 512 * 256, dtype=torch.uint8, device="cuda")
+    mf_sink = torch.empty(mf_blocks * 512, dtype=F, device="cuda")
+    mf_flop = mf_blocks * 8 * mf_iters * 16 * 32768
+    sp_m = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    mfma_rate = {}
+    for name, code, dt in (("f16", 1, H), ("bf16", 2, B16)):
+        view = mf_ops.view(dt)
+        probe = lambda: _lib.check(K3.brt_rocm_mfma_rate_probe(code, mf_ops.data_ptr(), mf_ops.numel(), mf_sink.data_ptr(),
+                                                                mf_sink.numel() * 4, mf_blocks, mf_iters, sp_m))
+        for what in ("zeros", "normal"):
+            if what == "zeros":
+                view.zero_()
+            else:
+                ops.fill(view, _lib.FILL_NORMAL, SEED["c4q"], 0.0, 1.0)
+            prewarm(probe, 0.3)
+            r = time_regions(ev, [probe], 5, 1)
+            mfma_rate[f"{name}_{what}"] = with_clock({"value": round(mf_flop / (r["ms"] * 1e-3) / 1e12, 1), "unit": "TFLOP/s"}, r, MFMA_PEAK_TFLOPS, "frac_of_mfma_peak")
+    mfma_rate["note"] = ("brt_rocm_mfma_rate_probe: 16 independent v_mfma_f32_32x32x16 per iteration and wave, 2 waves per SIMD, operands in registers, "
+                         f"{mf_blocks} workgroups x {mf_iters} iterations per launch; 'normal' = operands ~ N(0,1) as the attention inputs are")
+    all_cfg["mfma_rate_probe"] = mfma_rate
+    del mf_ops, mf_sink
+
+    def of_probe(entry, key):
+        entry["frac_of_mfma_rate_on_normal_operands"] = round(entry["value"] / mfma_rate[key]["value"], 4)
+        return entry
+
     # c4: flash-attention forward fp16 causal b4 h32 s2048 d128
     q, k, v = (mk((4, 2048, 32, 128), H, _lib.FILL_NORMAL, SEED[n], 0.0, 1.0) for n in ("c4q", "c4k", "c4v"))
     sc4 = 1.0 / np.sqrt(128.0)
@@ -727,7 +758,7 @@ def extras(all_cfg, ev, ops, _lib, oracle, args, np, torch, n_thr):
         t1, tn = cpu_both(oracle, lambda: oracle.flash_fwd(qs[:, -256:], ks_, vs_, sc4, (-1, 0)), n_thr, 1)
         c4.update(cpu_1core_TFLOPs=round(fl_s / t1 / 1e12, 6), cpu_allcore_TFLOPs=round(fl_s / tn / 1e12, 6), cpu_cores=n_thr,
                   cpu_sample="naive oracle, 1 batch x 1 head x last 256 query rows, by flop count")
-    all_cfg["c4_flash_fwd_fp16_causal"] = c4
+    all_cfg["c4_flash_fwd_fp16_causal"] = of_probe(c4, "f16_normal")
     del q, k, v, qs, ks_, vs_
 
     # c5: flash-attention forward + backward bf16 non-causal b2 h16 s8192 d64
@@ -780,6 +811,8 @@ def extras(all_cfg, ev, ops, _lib, oracle, args, np, torch, n_thr):
                          fl5 * 5 // 2, "flop", msb, MFMA_PEAK_TFLOPS, "event pair around 50 back-to-back calls, median of three regions"),
         "note": "flop = 2.5 x forward (5 GEMMs); the kernels execute 7 (S and dP are recomputed by the dQ pass)"},
         rb, MFMA_PEAK_TFLOPS, "frac_of_mfma_peak")
+    of_probe(all_cfg["c5_flash_fwd_bf16"], "bf16_normal")
+    of_probe(all_cfg["c5_flash_bwd_bf16"], "bf16_normal")
     all_cfg["c5_flash_fwd_bwd_bf16"] = {
         "value": round((fl5 + flb) / ((msf + msb) * 1e-3) / 1e12, 1), "unit": "TFLOP/s",
         "frac_of_mfma_peak": round((fl5 + flb) / ((msf + msb) * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, 4)}

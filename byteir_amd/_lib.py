@@ -53,6 +53,7 @@ def kernels():
             getattr(L, f"brt_rocm_memcpy_{n}").argtypes = [vp, vp, sz, vp]
         L.brt_rocm_memset.argtypes = [vp, i32, sz, vp]
         L.brt_rocm_copy_kernel.argtypes = [vp, vp, sz, vp]
+        L.brt_rocm_mfma_rate_probe.argtypes = [i32, vp, sz, vp, sz, i32, i32, vp]
         L.brt_rocm_stream_create.argtypes = [pvp]
         L.brt_rocm_stream_destroy.argtypes = [vp]
         L.brt_rocm_stream_synchronize.argtypes = [vp]

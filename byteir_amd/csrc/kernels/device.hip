@@ -20,9 +20,58 @@ __global__ void __launch_bounds__(256) copy16_kernel(uint4 *__restrict__ dst, co
   const u32x4 t = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src) + i);
   dst[i] = uint4{t.x, t.y, t.z, t.w};
 }
+
+// Nothing but matrix instructions: each wave keeps eight A and eight B operands (read once from
+// `operands`, 256 bytes per lane) and four accumulator tiles in registers and issues 16 independent
+// v_mfma_f32_32x32x16 per iteration.  What limits it is the clock the chip holds under that load,
+// which depends on how many operand bits toggle: the rate on zeros is the instruction-issue peak,
+// the rate on normally distributed operands is the ceiling that any kernel fed such data can reach.
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+template <bool Bf16>
+__global__ void __launch_bounds__(512, 2) mfma_rate_kernel(const u32x4 *__restrict__ operands, float *__restrict__ sink, int iters) {
+  const size_t t = (size_t)blockIdx.x * 512 + threadIdx.x;
+  u32x4 a[8], b[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) { a[i] = operands[t * 16 + i]; b[i] = operands[t * 16 + 8 + i]; }
+  f32x16 acc[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) acc[i] = f32x16{0};
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int m = 0; m < 16; ++m) {
+      const int ia = m & 7, ib = (m * 3 + (m >> 3)) & 7;
+      if (Bf16) acc[m & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a[ia]), __builtin_bit_cast(bf16x8, b[ib]), acc[m & 3], 0, 0, 0);
+      else acc[m & 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a[ia]), __builtin_bit_cast(f16x8, b[ib]), acc[m & 3], 0, 0, 0);
+    }
+    if ((it & 63) == 63) {  // keeps the sums finite; 64 multiplies per 1024 matrix instructions
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[i] *= 1e-3f;
+    }
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 16; ++j) s += acc[i][j];
+  sink[t] = s;
+}
 }  // namespace
 
 extern "C" {
+
+int brt_rocm_mfma_rate_probe(int dtype, const void *operands, size_t operand_bytes, float *sink, size_t sink_bytes,
+                             int blocks, int iters, void *stream) {
+  if (blocks <= 0 || iters < 0 || (dtype != BRT_ROCM_F16 && dtype != BRT_ROCM_BF16)) return hipErrorInvalidValue;
+  if (operand_bytes < (size_t)blocks * 512 * 256 || sink_bytes < (size_t)blocks * 512 * 4) return hipErrorInvalidValue;
+  if (reinterpret_cast<uintptr_t>(operands) & 15u) return hipErrorInvalidValue;
+  if (dtype == BRT_ROCM_BF16)
+    mfma_rate_kernel<true><<<dim3(blocks), dim3(512), 0, static_cast<hipStream_t>(stream)>>>(static_cast<const u32x4 *>(operands), sink, iters);
+  else
+    mfma_rate_kernel<false><<<dim3(blocks), dim3(512), 0, static_cast<hipStream_t>(stream)>>>(static_cast<const u32x4 *>(operands), sink, iters);
+  return hipGetLastError();
+}
 
 int brt_rocm_copy_kernel(void *dst, const void *src, size_t bytes, void *stream) {
   if (bytes % 16 != 0 || ((reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src)) & 15u))

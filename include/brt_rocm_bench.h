@@ -19,6 +19,16 @@ extern "C" {
  * copy ceiling the softmax figures are compared with. */
 int brt_rocm_copy_kernel(void *dst, const void *src, size_t bytes, void *stream);
 
+/* The rate of v_mfma_f32_32x32x16_{f16,bf16} on operands of the caller's choosing, with nothing
+ * else in the loop: `blocks` workgroups of eight waves each read 256 bytes of operands per lane
+ * (operand_bytes >= blocks * 512 * 256) once, then issue iters * 16 matrix instructions per wave
+ * on them; sink (blocks * 512 floats) receives the sums so that the work is not dead.  One launch
+ * does blocks * 8 * iters * 16 * 32768 flops.  The clock that the chip holds under this load
+ * depends on the operand bits, so the rate on zeros and the rate on normally distributed values
+ * differ: the second is the ceiling for a kernel that is fed such data. */
+int brt_rocm_mfma_rate_probe(int dtype, const void *operands, size_t operand_bytes, float *sink,
+                             size_t sink_bytes, int blocks, int iters, void *stream);
+
 /* events, for timing a launch on the stream it runs on */
 int brt_rocm_event_create(void **event);
 int brt_rocm_event_destroy(void *event);

@@ -52,6 +52,29 @@ def test_static_scratch_fold_equals_workspace_fold_on_two_calls_in_a_row(dtype):
     assert torch.equal(got, want)
 
 
+def test_static_scratch_fold_allocates_no_device_memory():
+    """Free device memory as the driver reports it (hipMemGetInfo) and the caching allocator's
+    counters are the same before and after the calls: a hipMalloc inside the entry point would
+    lower the first, an allocation through torch would raise the second."""
+    K = _lib.kernels()
+    A, B, C = 1, 16384, 2048
+    x = torch.ones(A * B * C, dtype=torch.float32, device="cuda")
+    out = torch.empty(A * C, dtype=torch.float32, device="cuda")
+    call = lambda op: K.brt_rocm_reduce_static(op, _lib.F32, ctypes.c_void_p(x.data_ptr()), ctypes.c_void_p(out.data_ptr()),
+                                               A, B, C, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert call(_lib.REDUCE_SUM) == 0  # first call on this device: the scratch address is looked up here
+    torch.cuda.synchronize()
+    free0, _ = torch.cuda.mem_get_info()
+    stats0 = {k: torch.cuda.memory_stats()[k] for k in ("allocation.all.allocated", "segment.all.allocated", "reserved_bytes.all.current")}
+    for op in (_lib.REDUCE_SUM, _lib.REDUCE_MAX, _lib.REDUCE_SUM):
+        assert call(op) == 0
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info()
+    stats1 = {k: torch.cuda.memory_stats()[k] for k in stats0}
+    assert free1 == free0 and stats1 == stats0
+    assert bool((out == float(B)).all())
+
+
 def test_static_scratch_refuses_a_fold_that_does_not_fit():
     K = _lib.kernels()
     limit = _lib.REDUCE_STATIC_SCRATCH_BYTES
