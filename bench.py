@@ -514,10 +514,10 @@ def main():
     if not args.no_cpu:
         step = lambda: (oracle.reduce_abc(oracle.MAX, xh, 1, R, Cc), oracle.reduce_abc(oracle.SUM, xh, 1, R, Cc),
                         oracle.reduce_abc(oracle.MAX, xh, R, Cc, 1), oracle.reduce_abc(oracle.SUM, xh, R, Cc, 1))
-        t_cpu, t_par = cpu_both(oracle, step, n_thr, 20)
+        t_cpu, t_par = cpu_both(oracle, step, n_thr, 60)
         result["cpu_baseline"] = {
             "value": round(step_bytes / t_cpu / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
-            "sample": "the full step (4 reductions of the [16384, 8192] tensor) run once per repeat, best of 20 (about 4 s of CPU work), "
+            "sample": "the full step (4 reductions of the [16384, 8192] tensor) run once per repeat, best of 60 (about 10 s of CPU work on one core), "
                       "by the scalar loop-nest oracle (the reference's CPU path is single-threaded LLVM-JIT'ed "
                       "loop nests, which cannot be built here)",
             "seconds": round(t_cpu, 3), "host_cores_available": os.cpu_count(),
