@@ -18,6 +18,7 @@
 #include <cctype>
 #include <cstdlib>
 #include <fstream>
+#include <functional>
 #include <sstream>
 
 #include "brt.h"
@@ -168,6 +169,9 @@ public:
 
   void Run() {
     if (lx_.Accept("module")) {
+      if (lx_.Accept("@")) {  // module @IrToMhlo.2452 attributes {...}: the symbol name is not used
+        if (lx_.Peek() == '"') lx_.String(); else lx_.Ident();
+      }
       if (lx_.Accept("attributes")) ParseAttrDict();
       lx_.Expect("{");
       ParseFunc();
@@ -276,12 +280,17 @@ private:
         elems.push_back(s);
       };
       bool splat = true;
+      // dense<[[0, 0], [1, 1]]> : tensor<2x2xi64>: nested lists are flattened in row-major order
+      std::function<void()> list = [&]() {
+        if (lx_.Accept("]")) return;
+        do {
+          if (lx_.Accept("[")) list(); else one();
+        } while (lx_.Accept(","));
+        lx_.Expect("]");
+      };
       if (lx_.Accept("[")) {
         splat = false;
-        if (!lx_.Accept("]")) {
-          do one(); while (lx_.Accept(","));
-          lx_.Expect("]");
-        }
+        list();
       } else {
         one();
       }
@@ -430,12 +439,36 @@ private:
       h_->ops.push_back(std::move(op));
       return;
     }
+    if (lx_.Accept("byre.copy")) {  // byre.copy(%src, %dst) {callee = "cuda2cuda"} : type, type (ByreOps.td:170-186)
+      Op op;
+      op.name = "byre.copy";
+      op.line = line;
+      op.operands = ParseOperands();
+      if (op.operands.size() != 2) lx_.Fail("byre.copy takes a source and a target");
+      if (lx_.Peek() == '{') op.attrs = ParseAttrDict();
+      lx_.Expect(":");
+      CheckType(op.operands[0], ParseMemRef());
+      lx_.Expect(",");
+      CheckType(op.operands[1], ParseMemRef());
+      // the registry key of a copy is its callee attribute (ByreInterface::getCalleeName, ByreBase.td:170-190)
+      if (!op.attrs.count("callee") || op.attrs["callee"].s.empty()) lx_.Fail("byre.copy without callee");
+      op.key = op.attrs["callee"].s;
+      h_->ops.push_back(std::move(op));
+      return;
+    }
     if (lx_.Peek() == '"') {  // generic form
       Op op;
       op.name = lx_.String();
       op.line = line;
       op.operands = ParseOperands();
-      if (lx_.Peek() == '{') op.attrs = ParseAttrDict();
+      if (lx_.Accept("<")) {  // inherent attributes printed as properties: "op"(...) <{offset = 0 : i64}> {device = "cuda"}
+        op.attrs = ParseAttrDict();
+        lx_.Expect(">");
+      }
+      if (lx_.Peek() == '{') {
+        auto more = ParseAttrDict();
+        for (auto &kv : more) op.attrs[kv.first] = std::move(kv.second);
+      }
       lx_.Expect(":");
       lx_.Expect("(");
       for (size_t i = 0; i < op.operands.size(); ++i) {

@@ -398,3 +398,99 @@ BRT_STATIC_KERNEL_REGISTRATION(DeviceKind::ROCM, ProviderType::BRT, [](KernelReg
             assert deps == [[], [], [0, 1], [0]], deps
         finally:
             s.close()
+
+
+RESNET_DIR = "/root/reference/runtime/test/test_files"
+RESNET_FILES = ["resnet18_fw_bw_host_cuda.mlir", "resnet18_fw_host_cuda.mlir", "resnet18_bw_host_cuda.mlir"]
+
+_RESNET_CHILD = r'''
+import ctypes, json, os, re, subprocess, sys, tempfile
+root, path = sys.argv[1], sys.argv[2]
+sys.path.insert(0, root)
+from byteir_amd import _lib, brt
+text = open(path).read()
+keys = sorted(set(re.findall(r"byre\.compute @([\w.]+)", text)) | set(re.findall(r'byre\.copy\(.*callee = "(\w+)"', text)))
+probe = brt.Session(device_id=-1)
+missing = [k for k in keys if not probe.has_kernel(k)]
+probe.close()
+# kernels that do nothing for the op keys this provider has no kernel for (cuDNN / cuBLAS / PTX ops)
+src = '#include "brt.h"\nnamespace { class Stub final : public brt::OpKernel { public: explicit Stub(const brt::OpKernelInfo &i) : brt::OpKernel(i) {}\n' \
+      '  brt::common::Status RunImpl(const brt::ExecutionContext &) override { return brt::common::Status::OK(); } };\n' \
+      'void Reg(brt::KernelRegistry *r) {\n' + "".join(
+          f'  r->Register("{k}", [](const brt::OpKernelInfo &i) -> std::shared_ptr<brt::OpKernel> {{ return std::make_shared<Stub>(i); }});\n' for k in missing) + \
+      '} }\nBRT_STATIC_KERNEL_REGISTRATION(brt::DeviceKind::ROCM, brt::ProviderType::BRT, Reg)\n'
+with tempfile.TemporaryDirectory() as tmp:
+    cc, so = os.path.join(tmp, "stubs.cc"), os.path.join(tmp, "libstubs.so")
+    open(cc, "w").write(src)
+    libdir = os.path.join(root, "byteir_amd", "lib")
+    subprocess.run(["g++", "-std=c++17", "-O0", "-shared", "-fPIC", "-I" + os.path.join(root, "byteir_amd", "csrc", "brt"),
+                    cc, "-o", so, "-L" + libdir, "-lbrt", "-Wl,-rpath," + libdir], check=True)
+    assert _lib.brt().brt_register_kernels_from_dynlib(so.encode()) == 0
+    s = brt.Session(device_id=-1)
+    s.load(path)
+    print(json.dumps({"missing": missing, "ops": s.get_op_keys(), "args": s.get_arg_num(),
+                      "cuda_bytes": s.get_intermediate_bytes("cuda")}))
+    s.close()
+'''
+
+
+@pytest.mark.skipif(not os.path.isdir(RESNET_DIR), reason="the reference checkout is not mounted")
+@pytest.mark.parametrize("name", RESNET_FILES)
+def test_reference_resnet_modules_parse_and_plan(name):
+    """The reference's ResNet-18 host modules, as its compiler wrote them (module symbol name,
+    nested dense attributes, byre.alias into one memref.alloc arena, byre.copy in custom assembly,
+    hundreds of arguments).  With the provider's own kernels alone the load ends where the
+    reference's would on a provider without cuDNN / PTX ops: `No providers support Op <key>`,
+    not a parse error.  With do-nothing kernels registered for those keys from an external
+    library (in a child process, so they do not stay registered) the whole module loads: every
+    op in file order, the reduce ops bound to this provider's kernels, the arena planned."""
+    import json
+    import subprocess
+    import sys
+    from byteir_amd import brt
+    path = os.path.join(RESNET_DIR, name)
+    text = open(path).read()
+    s = brt.Session(device_id=-1)
+    try:
+        with pytest.raises(RuntimeError, match=r"^No providers support Op \w+"):
+            s.load(path)
+    finally:
+        s.close()
+    out = subprocess.run([sys.executable, "-c", _RESNET_CHILD, ROOT, path], check=True, capture_output=True, text=True).stdout
+    got = json.loads(out.strip().splitlines()[-1])
+    want_ops = re.findall(r"^\s*(?:byre\.compute @([\w.]+)|byre\.copy\(.*callee = \"(\w+)\")", text, flags=re.M)
+    want_ops = [a or b for a, b in want_ops]
+    assert got["ops"] == want_ops and len(want_ops) > 100
+    assert not any(k.startswith("Reduce") for k in got["missing"])  # the reduce ops are this provider's
+    assert sum(k.startswith("Reduce") for k in got["ops"]) == len(re.findall(r"byre\.compute @Reduce", text))
+    assert got["args"] == len(re.findall(r"byre\.argname", text))
+    alloc = re.search(r"memref\.alloc\(\) : memref<(\d+)xi8", text)
+    assert alloc and got["cuda_bytes"] >= int(alloc.group(1))
+
+
+def test_reader_accepts_copy_in_custom_assembly_and_nested_dense(session):
+    """byre.copy(%src, %dst) {callee = ...} : type, type (ByreOps.td:170-186; the key is the callee,
+    ByreBase.td:170-190) and dense<[[..], [..]]> attributes, as in resnet18_fw_host_cuda.mlir:16,184."""
+    t = memref([64], "f32", "cuda")
+    session.load_from_memory(f"""module @IrToMhlo.77 attributes {{byre.container_module, gpu.container_module}} {{
+      func.func @main(%a : {t} {{byre.argname = "a", byre.argtype = 1 : i32}},
+                      %b : {t} {{byre.argname = "b", byre.argtype = 2 : i32}}) attributes {{byre.entry_point}} {{
+        byre.copy(%a, %b) {{callee = "cuda2cuda", device = "cuda", padding = dense<[[0, 0], [1, 1]]> : tensor<2x2xi64>}} : {t}, {t}
+        return
+      }}
+    }}""")
+    assert session.get_op_keys() == ["cuda2cuda"]
+    # inherent attributes printed as a property dictionary (Distributed/ccl.mlir:8): the alias offset
+    t2 = memref([8, 4], "f32", "cuda")
+    session.load_from_memory(f"""func.func @main(%a : {t} {{byre.argname = "a", byre.argtype = 1 : i32}},
+                      %b : {memref([8], "f32", "cuda")} {{byre.argname = "b", byre.argtype = 2 : i32}}) attributes {{byre.entry_point}} {{
+        %alloc = memref.alloc() : memref<512xi8, "cuda">
+        %0 = "byre.alias"(%alloc) <{{offset = 256 : i64}}> {{device = "cuda"}} : (memref<512xi8, "cuda">) -> {t2}
+        byre.compute @ReduceSumOp_f32_f32(%0, %b) {{dimensions = dense<1> : tensor<1xi64>}} : {t2}, {memref([8], "f32", "cuda")}
+        return }}""")
+    assert session.get_op_keys() == ["ReduceSumOp_f32_f32"] and session.get_intermediate_bytes("cuda") == 512
+    with pytest.raises(RuntimeError, match="byre.copy without callee"):
+        session.load_from_memory(f"""func.func @main(%a : {t} {{byre.argname = "a", byre.argtype = 1 : i32}},
+                      %b : {t} {{byre.argname = "b", byre.argtype = 2 : i32}}) attributes {{byre.entry_point}} {{
+        byre.copy(%a, %b) : {t}, {t}
+        return }}""")

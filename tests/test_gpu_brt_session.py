@@ -80,6 +80,72 @@ def test_unregistered_reference_operators_through_session(session, shape, dims, 
     req.close()
 
 
+def test_reduce_ops_of_the_reference_resnet_modules_run_as_written(session, golden_dir):
+    """Every `byre.compute @Reduce*` line of the reference's ResNet-18 host modules
+    (runtime/test/test_files/resnet18_{fw_bw,fw,bw}_host_cuda.mlir), character for character as the
+    reference's compiler wrote them (tests/golden/make_resnet_reduce_module.py gathers them into
+    one entry function): f16 and f32, `dense<[3, 2]>` dimensions in descending order, a fold of
+    all dimensions into a rank-0 memref, and a fold of a dimension of extent 1."""
+    session.load(os.path.join(golden_dir, "resnet18_reduce_ops.mlir"))
+    keys = session.get_op_keys()
+    assert len(keys) == 8 and set(keys) == {"ReduceSumOp_f16_f16", "ReduceMaxOp_f16_f16", "ReduceSumOp_f32_f32"}
+    dims_of = [(1,), (3, 2), (1,), (1,), (0, 1), (0,), (3, 2), (0,)]  # the `dimensions` attributes, in file order
+    req = session.new_request_context()
+    rng = np.random.default_rng(18)
+    bufs = []
+    for i in range(len(keys)):
+        shape, dt = session.get_static_shape(2 * i), session.get_data_type(2 * i)
+        assert session.get_data_type(2 * i + 1) == dt
+        tdt = getattr(torch, dt)  # "float16" / "float32"
+        x = torch.from_numpy(rng.standard_normal(shape).astype(np.float32)).to("cuda", tdt)
+        y = torch.full(tuple(session.get_static_shape(2 * i + 1)), -7.0, dtype=tdt, device="cuda")
+        req.bind_arg(2 * i, x.data_ptr())
+        req.bind_arg(2 * i + 1, y.data_ptr())
+        bufs.append((x, y))
+    req.finish_io_binding()
+    req.run()
+    req.sync()
+    for key, dims, (x, y) in zip(keys, dims_of, bufs):
+        x64 = x.double().cpu().numpy()
+        if "Max" in key:
+            assert np.array_equal(y.double().cpu().numpy(), x64.max(axis=dims))
+            continue
+        want, sabs = x64.sum(axis=dims), np.abs(x64).sum(axis=dims)
+        got = y.double().cpu().numpy()
+        assert got.shape == want.shape
+        tol = 1e-5 if x.dtype == torch.float32 else 2.0 ** -10  # f16: one rounding of the float fold
+        assert np.all(np.abs(got - want) <= tol * np.maximum(np.abs(want), 1e-2 * sabs) + (0 if x.dtype == torch.float32 else 2.0 ** -11 * np.abs(want))), key
+    req.close()
+
+
+def test_copy_in_custom_assembly_into_an_alias_with_a_property_offset(session):
+    """byre.copy(%src, %dst) {callee = "cuda2cuda"} (resnet18_fw_host_cuda.mlir:184) into an alias
+    whose offset is printed as a property dictionary (Distributed/ccl.mlir:8), then a fold of the
+    alias: the copy's key is its callee, the alias lands 256 bytes into the arena."""
+    t, to = 'memref<8x4xf32, "cuda">', 'memref<8xf32, "cuda">'
+    session.load_from_memory(f"""module @M.1 attributes {{byre.container_module}} {{
+      func.func @main(%a : {t} {{byre.argname = "a", byre.argtype = 1 : i32}},
+                      %b : {to} {{byre.argname = "b", byre.argtype = 2 : i32}}) attributes {{byre.entry_point}} {{
+        %alloc = memref.alloc() : memref<512xi8, "cuda">
+        %0 = "byre.alias"(%alloc) <{{offset = 256 : i64}}> {{device = "cuda"}} : (memref<512xi8, "cuda">) -> {t}
+        byre.copy(%a, %0) {{callee = "cuda2cuda", device = "cuda"}} : {t}, {t}
+        byre.compute @ReduceSumOp_f32_f32(%0, %b) {{device = "cuda", dimensions = dense<1> : tensor<1xi64>, memory_effects = [1 : i32, 2 : i32]}} : {t}, {to}
+        return
+      }}
+    }}""")
+    assert session.get_op_keys() == ["cuda2cuda", "ReduceSumOp_f32_f32"]
+    req = session.new_request_context()
+    x = torch.arange(32, dtype=torch.float32, device="cuda").reshape(8, 4)
+    y = torch.full((8,), -7.0, device="cuda")
+    req.bind_arg(0, x.data_ptr())
+    req.bind_arg(1, y.data_ptr())
+    req.finish_io_binding()
+    req.run()
+    req.sync()
+    assert torch.equal(y, x.sum(dim=1))
+    req.close()
+
+
 @pytest.mark.parametrize("op_name", ["ReduceSumOp_f32_f32", "ReduceMaxOp_f32_f32"])
 def test_nan_propagation_through_session(session, op_name):
     # reduction_test.cc:182-215: 1024 elements, NaN first; runtime-allocated arguments
