@@ -84,12 +84,33 @@ def build_test_kernels(verbose=False):
                                 f"-L{LIB}", "-lbrt", "-lbrt_rocm_kernels", f"-Wl,-rpath,{LIB}"], verbose)
 
 
+def build_emu(verbose=False):
+    """The flash-attention sources compiled for the host (tests/emu/wave_emu.h stands in for the
+    HIP runtime header and runs every lane as a fiber): tests/emu/libflash_attn_emu.so, the
+    library's C ABI on host memory, for the tests that need no GPU.  Needs a host clang (vector
+    extensions, _Float16, __bf16); skipped when there is none."""
+    clang = os.path.join(os.environ.get("ROCM_PATH", "/opt/rocm"), "llvm", "bin", "clang++")
+    emu = os.path.join(ROOT, "tests", "emu")
+    if not os.path.exists(clang) or not os.path.isdir(emu):
+        return
+    import concurrent.futures
+    obj = os.path.join(emu, "obj")
+    os.makedirs(obj, exist_ok=True)
+    flags = ["-std=c++17", "-O2", "-fPIC", "-DFA_EMULATE", f"-I{os.path.join(emu, 'include')}", f"-I{emu}",
+             f"-I{os.path.join(CSRC, 'flash_attn')}", f"-I{os.path.join(ROOT, 'include')}", "-Wno-unknown-attributes"]
+    jobs = [(src, os.path.join(obj, os.path.basename(src) + ".o"), ["-x", "c++"]) for src in _glob("flash_attn", (".hip",))]
+    jobs.append((os.path.join(emu, "wave_emu.cc"), os.path.join(obj, "wave_emu.o"), []))
+    with concurrent.futures.ThreadPoolExecutor(max_workers=6) as pool:
+        list(pool.map(lambda j: _run([clang] + j[2] + flags + ["-c", j[0], "-o", j[1]], False), jobs))
+    _run([clang, "-shared", "-fPIC", "-o", os.path.join(emu, "libflash_attn_emu.so")] + [j[1] for j in jobs], verbose)
+
+
 TARGETS = {"kernels": build_kernels, "flash": build_flash, "brt": build_brt, "index_check": build_index_check,
-           "test_kernels": build_test_kernels}
+           "test_kernels": build_test_kernels, "emu": build_emu}
 
 
 def build_all(verbose=False, targets=None):
-    for name in targets or ("kernels", "flash", "brt", "index_check", "test_kernels"):
+    for name in targets or ("kernels", "flash", "brt", "index_check", "test_kernels", "emu"):
         TARGETS[name](verbose)
 
 

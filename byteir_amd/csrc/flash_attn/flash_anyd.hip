@@ -669,8 +669,8 @@ __global__ void __launch_bounds__(256, (DR <= 96 || (DR == 128 && !Drop)) ? 2 : 
 template <typename T, int DR>
 hipError_t fwd_anyd_d(const Params &p, hipStream_t stream) {
   const dim3 grid((unsigned)(p.n_mblocks * p.b * p.h)), block(256);
-  if (p.drop) fwd_anyd_kernel<T, DR, true><<<grid, block, 0, stream>>>(p);
-  else fwd_anyd_kernel<T, DR, false><<<grid, block, 0, stream>>>(p);
+  if (p.drop) FA_LAUNCH((fwd_anyd_kernel<T, DR, true>), grid, block, stream, p);
+  else FA_LAUNCH((fwd_anyd_kernel<T, DR, false>), grid, block, stream, p);
   return hipGetLastError();
 }
 
@@ -687,16 +687,16 @@ hipError_t bwd_anyd_d(const Params &p, hipStream_t stream) {
     apply_group_split(pk, p, split, p.d);
     pk.xcd_remap = ((p.b * pk.h_k) % 8 == 0) ? (p.wr >= 0 ? 2 : 1) : (p.wr >= 0 ? 3 : 0);
     const dim3 gks((unsigned)(p.n_nblocks * p.b * pk.h_k));
-    if (p.drop) dkdv_anyd_kernel<T, DR, true><<<gks, block, 0, stream>>>(pk);
-    else dkdv_anyd_kernel<T, DR, false><<<gks, block, 0, stream>>>(pk);
+    if (p.drop) FA_LAUNCH((dkdv_anyd_kernel<T, DR, true>), gks, block, stream, pk);
+    else FA_LAUNCH((dkdv_anyd_kernel<T, DR, false>), gks, block, stream, pk);
     if (split.gs * split.qs > 1) {
       const hipError_t e = launch_group_sum(p, split, p.d, std::is_same<T, _Float16>::value ? 1 : 2, stream);
       if (e != hipSuccess) return e;
     }
   }
   if (p.n_mblocks > 0 && !p.ws_query) {
-    if (p.drop) dq_anyd_kernel<T, DR, true><<<gq, block, 0, stream>>>(p);
-    else dq_anyd_kernel<T, DR, false><<<gq, block, 0, stream>>>(p);
+    if (p.drop) FA_LAUNCH((dq_anyd_kernel<T, DR, true>), gq, block, stream, p);
+    else FA_LAUNCH((dq_anyd_kernel<T, DR, false>), gq, block, stream, p);
   }
   return hipGetLastError();
 }
@@ -714,7 +714,7 @@ hipError_t fwd_anyd_t(const Params &p, hipStream_t stream) {
 template <typename T>
 hipError_t bwd_anyd_t(const Params &p, hipStream_t stream) {
   const int64_t rows = (int64_t)p.b * p.h * p.sq;
-  if (rows > 0 && !p.ws_query) dot_do_o_anyd_kernel<T><<<dim3((unsigned)((rows + 7) / 8)), dim3(256), 0, stream>>>(p);
+  if (rows > 0 && !p.ws_query) FA_LAUNCH((dot_do_o_anyd_kernel<T>), dim3((unsigned)((rows + 7) / 8)), dim3(256), stream, p);
   if (p.d <= 32) return bwd_anyd_d<T, 32>(p, stream);
   if (p.d <= 64) return bwd_anyd_d<T, 64>(p, stream);
   if (p.d <= 96) return bwd_anyd_d<T, 96>(p, stream);
@@ -741,8 +741,8 @@ hipError_t launch_dq_anyd128(const Params &p, int dtype, hipStream_t stream) {
   pq.n_mblocks = (p.sq + kRows - 1) / kRows;
   if (pq.n_mblocks == 0) return hipSuccess;
   const dim3 grid((unsigned)(pq.n_mblocks * p.b * p.h)), block(256);
-  if (dtype == 1) dq_anyd_kernel<_Float16, 128, false><<<grid, block, 0, stream>>>(pq);
-  else dq_anyd_kernel<__bf16, 128, false><<<grid, block, 0, stream>>>(pq);
+  if (dtype == 1) FA_LAUNCH((dq_anyd_kernel<_Float16, 128, false>), grid, block, stream, pq);
+  else FA_LAUNCH((dq_anyd_kernel<__bf16, 128, false>), grid, block, stream, pq);
   return hipGetLastError();
 }
 

@@ -188,7 +188,7 @@ __global__ void __launch_bounds__(256, (D <= 64 && KB == 1) ? 2 : 1) dkdv_kernel
 #pragma unroll
     for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
-      for (int ks = 0; ks < D / 16; ++ks) asm volatile("" : "+v"(kf[kb][ks]), "+v"(vf[kb][ks]));
+      for (int ks = 0; ks < D / 16; ++ks) FA_PIN2(kf[kb][ks], vf[kb][ks]);
   };
   if constexpr (!kLean) consume_kv();
   float16v dk_acc[KB][D / 32], dv_acc[KB][D / 32];
@@ -562,8 +562,8 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) dq_kernel(const Params p
   }
   // consume the fragments once so that the wait for their loads sits here, not inside the loop
 #pragma unroll
-  for (int ks = 0; ks < D / 16; ++ks) asm volatile("" : "+v"(qf[ks]), "+v"(dof[ks]));
-  asm volatile("" : "+v"(lse_l), "+v"(dsm_l));
+  for (int ks = 0; ks < D / 16; ++ks) FA_PIN2(qf[ks], dof[ks]);
+  FA_PIN2(lse_l, dsm_l);
   // -D of the lane's row in all 16 accumulator slots: dP^T starts from it (the MFMA's C
   // operand), which takes the subtraction of dS = P (dP - D) off the vector ALU
   float16v neg_d;
@@ -747,7 +747,7 @@ hipError_t launch_bwd_td(const Params &p, hipStream_t stream) {
   const int64_t rows = (int64_t)p.b * p.h * p.sq;
   if (rows > 0 && !p.ws_query) {
     constexpr int RPB = 256 / (D / 8);
-    dot_do_o_kernel<T, D><<<dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(256), 0, stream>>>(p);
+    FA_LAUNCH((dot_do_o_kernel<T, D>), dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(256), stream, p);
   }
   // One 32-key block per wave.  Two blocks halve the LDS reads per MFMA (LDS bandwidth is
   // what bounds this kernel) but need about 450 registers: one wave per SIMD and accumulators
@@ -765,7 +765,7 @@ hipError_t launch_bwd_td(const Params &p, hipStream_t stream) {
   apply_group_split(pk, p, split, D);
   pk.xcd_remap = idx::block_order_mode(p.b * pk.h_k, p.wr);
   if (pk.n_nblocks > 0)
-    dkdv_kernel<T, D, KB><<<dim3((unsigned)(pk.n_nblocks * p.b * pk.h_k)), dim3(256), 0, stream>>>(pk);
+    FA_LAUNCH((dkdv_kernel<T, D, KB>), dim3((unsigned)(pk.n_nblocks * p.b * pk.h_k)), dim3(256), stream, pk);
   if (split.gs * split.qs > 1) {
     const hipError_t e = launch_group_sum(p, split, D, std::is_same<T, _Float16>::value ? 1 : 2, stream);
     if (e != hipSuccess) return e;
@@ -783,7 +783,7 @@ hipError_t launch_bwd_td(const Params &p, hipStream_t stream) {
     }
   }
   if (pq.n_mblocks > 0)
-    dq_kernel<T, D><<<dim3((unsigned)(pq.n_mblocks * p.b * p.h)), dim3(256), 0, stream>>>(pq);
+    FA_LAUNCH((dq_kernel<T, D>), dim3((unsigned)(pq.n_mblocks * p.b * p.h)), dim3(256), stream, pq);
   return hipGetLastError();
 }
 
@@ -802,8 +802,8 @@ hipError_t launch_group_sum(const Params &p, const GroupSplit &s, int row, int d
   hipError_t e = hipSuccess;
   if (chunks > 0) {
     const dim3 grid((unsigned)((chunks + 255) / 256)), block(256);
-    if (dtype == 1) group_sum_kernel<_Float16><<<grid, block, 0, stream>>>(p, s.dk, s.dv, s.gs * s.qs, row);
-    else group_sum_kernel<__bf16><<<grid, block, 0, stream>>>(p, s.dk, s.dv, s.gs * s.qs, row);
+    if (dtype == 1) FA_LAUNCH((group_sum_kernel<_Float16>), grid, block, stream, p, s.dk, s.dv, s.gs * s.qs, row);
+    else FA_LAUNCH((group_sum_kernel<__bf16>), grid, block, stream, p, s.dk, s.dv, s.gs * s.qs, row);
     e = hipGetLastError();
   }
   if (s.owned) {

@@ -18,6 +18,26 @@
 
 #include "flash_index.h"
 
+// A kernel launch on `stream` without dynamic LDS.  The kernel name goes in parentheses (its
+// template arguments hold commas).  A host build of these sources for tests defines its own
+// FA_LAUNCH (and FA_PIN) before this header and runs the workgroups on the CPU.
+#ifndef FA_LAUNCH
+#define FA_LAUNCH(kernel, grid, block, stream, ...) kernel<<<(grid), (block), 0, (stream)>>>(__VA_ARGS__)
+#endif
+// Consumes a value in a vector register at this point of the program: the wait for the loads
+// that produce it is placed here instead of in front of its first use.
+// Marks a point where the lanes of one wave exchange data through LDS without a workgroup
+// barrier: what all lanes wrote before it is read by other lanes of the same wave after it.
+// On the GPU a wave executes its LDS instructions in program order for all lanes at once, so
+// nothing is needed; a lane-by-lane host execution joins the wave's lanes here.
+#ifndef FA_WAVE_SYNC
+#define FA_WAVE_SYNC() ((void)0)
+#endif
+#ifndef FA_PIN
+#define FA_PIN(x) asm volatile("" : "+v"(x))
+#define FA_PIN2(x, y) asm volatile("" : "+v"(x), "+v"(y))
+#endif
+
 namespace fa {
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));

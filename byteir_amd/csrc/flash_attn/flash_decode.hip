@@ -120,6 +120,7 @@ __global__ void __launch_bounds__(kDecWaves * 64, D <= 128 ? 2 : 1) decode_kerne
       *reinterpret_cast<uint4 *>(&Kt[(s * RPP + v_r) * KS + v_c * 8]) = kn[s];
       *reinterpret_cast<uint4 *>(&Vt[(s * RPP + v_r) * VS + v_c * 8]) = vn[s];
     }
+    FA_WAVE_SYNC();  // the wave's own tile: written by all its lanes, read across lanes, no workgroup barrier
   };
 
   float16v o_acc[D / 32];
@@ -287,11 +288,11 @@ hipError_t decode_td(const Params &p, hipStream_t stream) {
       a.ml_part = a.o_part + (size_t)n_splits * rows * D;
     }
   }
-  decode_kernel<T, D><<<dim3((unsigned)(base * a.n_splits)), dim3(kDecWaves * 64), 0, stream>>>(p, a);
+  FA_LAUNCH((decode_kernel<T, D>), dim3((unsigned)(base * a.n_splits)), dim3(kDecWaves * 64), stream, p, a);
   hipError_t e = hipGetLastError();
   if (ws) {
     if (e == hipSuccess) {
-      decode_merge_kernel<T, D><<<dim3((unsigned)rows), dim3(D < 64 ? 64 : D), 0, stream>>>(p, a);
+      FA_LAUNCH((decode_merge_kernel<T, D>), dim3((unsigned)rows), dim3(D < 64 ? 64 : D), stream, p, a);
       e = hipGetLastError();
     }
     if (owned) {
@@ -308,9 +309,9 @@ hipError_t split_merge_t(const Params &p, hipStream_t stream) {
   a.o_part = p.o_part; a.ml_part = p.ml_part; a.n_splits = p.n_splits;
   const dim3 grid((unsigned)((size_t)p.b * p.h * p.sq));
   switch (p.d) {
-  case 32: decode_merge_kernel<T, 32><<<grid, dim3(64), 0, stream>>>(p, a); break;
-  case 64: decode_merge_kernel<T, 64><<<grid, dim3(64), 0, stream>>>(p, a); break;
-  case 128: decode_merge_kernel<T, 128><<<grid, dim3(128), 0, stream>>>(p, a); break;
+  case 32: FA_LAUNCH((decode_merge_kernel<T, 32>), grid, dim3(64), stream, p, a); break;
+  case 64: FA_LAUNCH((decode_merge_kernel<T, 64>), grid, dim3(64), stream, p, a); break;
+  case 128: FA_LAUNCH((decode_merge_kernel<T, 128>), grid, dim3(128), stream, p, a); break;
   default: return hipErrorInvalidValue;
   }
   return hipGetLastError();

@@ -105,7 +105,7 @@ __global__ void __launch_bounds__(NW * 64, NW * QB >= 16 ? 2 : (QB == 2 ? 1 : 2)
 #pragma unroll
   for (int qb = 0; qb < QB; ++qb)
 #pragma unroll
-    for (int ks = 0; ks < D / 16; ++ks) asm volatile("" : "+v"(qf[qb][ks]));
+    for (int ks = 0; ks < D / 16; ++ks) FA_PIN(qf[qb][ks]);
 
   constexpr int CPR = D / 8;                       // 16-byte chunks per tile row
   constexpr int RPP = kThreads / CPR;              // rows covered by one pass of the workgroup
@@ -357,6 +357,7 @@ __global__ void __launch_bounds__(NW * 64, NW * QB >= 16 ? 2 : (QB == 2 ? 1 : 2)
       static_assert(D == 128, "the chunk permutation assumes 16 chunks per row");
       static_assert(!kStageO || (NW / 2 * 32 * OS <= kStages * kBN * KS && NW / 2 * 32 * OS <= kStages * kBN * VS), "O staging must fit the ring");
       if (qb == 0) __syncthreads();  // every wave has left the last K/V tile
+      else FA_WAVE_SYNC();           // every lane has read the previous half back
       T *Ot = (wave < NW / 2 ? &Ks[0][0] : &Vs[0][0]) + (wave % (NW / 2)) * 32 * OS;
 #pragma unroll
       for (int db = 0; db < D / 32; ++db)
@@ -368,6 +369,7 @@ __global__ void __launch_bounds__(NW * 64, NW * QB >= 16 ? 2 : (QB == 2 ? 1 : 2)
           for (int j = 0; j < 4; ++j) v[j] = (T)(o_acc[qb][db][i4 * 4 + j] * inv);
           *reinterpret_cast<vec4 *>(&Ot[idx::ostage_write_offset(r32, g, db, i4)]) = v;
         }
+      FA_WAVE_SYNC();  // the wave's tile is complete; it is read back across lanes
       constexpr int CPRO = D / 8, RPI = 64 / CPRO;  // 16-byte chunks per row, rows per store instruction
       const int oc = lane % CPRO, orow = lane / CPRO;
 #pragma unroll
@@ -458,8 +460,8 @@ hipError_t launch_fwd_d(Params &p, hipStream_t stream) {
     p.ml_part = p.o_part + (size_t)n_splits * rows * D;
   }
   const dim3 grid((unsigned)n_wg, (unsigned)p.n_splits), block(NW * 64);
-  if (p.seqlens_k) flash_fwd_kernel<T, D, QB, NW, true><<<grid, block, 0, stream>>>(p);
-  else flash_fwd_kernel<T, D, QB, NW, false><<<grid, block, 0, stream>>>(p);
+  if (p.seqlens_k) FA_LAUNCH((flash_fwd_kernel<T, D, QB, NW, true>), grid, block, stream, p);
+  else FA_LAUNCH((flash_fwd_kernel<T, D, QB, NW, false>), grid, block, stream, p);
   hipError_t e = hipGetLastError();
   if (ws) {
     if (e == hipSuccess) e = launch_split_merge(p, std::is_same<T, _Float16>::value ? 1 : 2, stream);
@@ -509,8 +511,8 @@ hipError_t launch_append_kv(const Params &p, int dtype, hipStream_t stream) {
   const int64_t total = (int64_t)p.b * p.seqlen_knew * p.h_k * (p.d / 8);
   if (total == 0) return hipSuccess;
   const dim3 grid((unsigned)((total + 255) / 256)), block(256);
-  if (dtype == 1) append_kv_kernel<_Float16><<<grid, block, 0, stream>>>(p);
-  else append_kv_kernel<__bf16><<<grid, block, 0, stream>>>(p);
+  if (dtype == 1) FA_LAUNCH((append_kv_kernel<_Float16>), grid, block, stream, p);
+  else FA_LAUNCH((append_kv_kernel<__bf16>), grid, block, stream, p);
   return hipGetLastError();
 }
 

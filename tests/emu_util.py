@@ -1,0 +1,112 @@
+"""The flash-attention library executed on the host (tests/emu/libflash_attn_emu.so: the HIP
+sources compiled against tests/emu/wave_emu.h, every lane a fiber): the same C ABI as
+libflash_attn.so, on CPU tensors.  Tensors are registered with the emulator for the duration of
+a call, so that buffer loads that pass their descriptor's range check are also checked against
+the tensors' extents; `guarded` tensors end at (or start behind) a protected page, which turns
+any stray access of a plain load or store into a reported fault."""
+import ctypes
+import os
+import subprocess
+import sys
+
+import numpy as np
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LIB = os.path.join(ROOT, "tests", "emu", "libflash_attn_emu.so")
+_vp = ctypes.c_void_p
+_L = None
+
+
+class EmuFault(RuntimeError):
+    pass
+
+
+def lib():
+    global _L
+    if _L is None:
+        if not os.path.exists(LIB):
+            subprocess.check_call([sys.executable, "-m", "byteir_amd.build", "emu"], cwd=ROOT)
+        L = ctypes.CDLL(LIB)
+        for n in ("fwd", "bwd", "kvcache"):
+            f = getattr(L, f"flash_attn_{n}_checked")
+            f.argtypes = [ctypes.POINTER(_vp), _vp, ctypes.c_int, _vp]
+            f.restype = ctypes.c_int
+        L.fa_emu_last_error.restype = ctypes.c_char_p
+        L.flash_attn_last_error.restype = ctypes.c_char_p
+        L.fa_emu_alloc.restype = _vp
+        L.fa_emu_alloc.argtypes = [ctypes.c_size_t, ctypes.c_int]
+        L.fa_emu_free.argtypes = [_vp]
+        L.fa_emu_register.argtypes = [_vp, ctypes.c_size_t]
+        L.fa_emu_unregister.argtypes = [_vp]
+        L.fa_emu_select.argtypes = [ctypes.c_longlong, ctypes.c_longlong]
+        L.fa_emu_blocks_run.restype = ctypes.c_longlong
+        _L = L
+    return _L
+
+
+def select(stride=1, phase=0):
+    """Run only the workgroups of every launch whose linear id is `phase` modulo `stride`."""
+    lib().fa_emu_select(stride, phase)
+
+
+def guarded(shape, dtype, at_end=True):
+    """A tensor whose last byte is the last byte before a protected page (at_end) or whose first
+    byte is the first behind one.  Lives until the process ends."""
+    L = lib()
+    n = int(np.prod(shape))
+    nbytes = n * torch.empty(0, dtype=dtype).element_size()
+    p = L.fa_emu_alloc(max(nbytes, 16), 1 if at_end else 0)
+    if not p:
+        raise MemoryError("fa_emu_alloc")
+    buf = (ctypes.c_char * max(nbytes, 16)).from_address(p)
+    return torch.frombuffer(buf, dtype=dtype, count=n).reshape(shape)
+
+
+def _call(kind, tensors, blob, dtype):
+    L = lib()
+    live = [t for t in tensors if t is not None]
+    for t in live:
+        L.fa_emu_register(_vp(t.data_ptr()), max(16, t.numel() * t.element_size()))
+    arr = (_vp * len(tensors))(*[t.data_ptr() if t is not None else None for t in tensors])
+    buf = ctypes.create_string_buffer(blob, len(blob))
+    try:
+        rc = getattr(L, f"flash_attn_{kind}_checked")(arr, ctypes.cast(buf, _vp), 1 if dtype == torch.float16 else 2, None)
+    finally:
+        for t in live:
+            L.fa_emu_unregister(_vp(t.data_ptr()))
+    if rc:
+        msg = L.fa_emu_last_error().decode() if L.fa_emu_faulted() else L.flash_attn_last_error().decode()
+        L.fa_emu_reset()
+        raise EmuFault(f"flash_attn_{kind}: rc {rc}: {msg}")
+
+
+def fwd(q, k, v, scale, window=(-1, -1), out=None):
+    from byteir_amd import ops
+    b, sq, h, d = q.shape
+    o, lse = out if out is not None else (torch.empty_like(q), torch.empty((b, h, sq), dtype=torch.float32))
+    rng = torch.zeros(2, dtype=torch.int64)
+    _call("fwd", [q, k, v, rng, o, lse, None], ops.pack_flash_args(q, k, v, o, scale, window, 0.0), q.dtype)
+    return o, lse
+
+
+def bwd(do, q, k, v, o, lse, scale, window=(-1, -1), out=None):
+    from byteir_amd import ops
+    b, sq, h, d = q.shape
+    ru = lambda x, m: -(-x // m) * m
+    if out is None:
+        out = (torch.empty_like(q), torch.empty_like(k), torch.empty_like(v),
+               torch.empty((b, h, ru(sq, 128)), dtype=torch.float32), torch.empty((b, ru(sq, 128), h, ru(d, 32)), dtype=torch.float32))
+    dq, dk, dv, dsm, acc = out
+    rng = torch.zeros(2, dtype=torch.int64)
+    _call("bwd", [do, q, k, v, o, lse, rng, dq, dk, dv, dsm, acc], ops.pack_flash_args(q, k, v, o, scale, window, 0.0), q.dtype)
+    return dq, dk, dv
+
+
+def kvcache(q, kcache, vcache, knew, vnew, seqlens_k, scale, window=(-1, -1)):
+    from byteir_amd import ops
+    b, sq, h, d = q.shape
+    o, lse = torch.empty_like(q), torch.empty((b, h, sq), dtype=torch.float32)
+    _call("kvcache", [q, kcache, vcache, knew, vnew, seqlens_k, o, lse],
+          ops.pack_flash_kvcache_args(q, kcache, vcache, knew, vnew, o, scale, window), q.dtype)
+    return o, lse

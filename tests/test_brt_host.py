@@ -320,6 +320,10 @@ def test_product_code_never_touches_the_oracle():
             if name.endswith((".py", ".hip", ".cc", ".h", ".c", ".cpp")):
                 text = open(os.path.join(dirpath, name), errors="replace").read()
                 assert "oracle" not in text.lower(), os.path.join(dirpath, name)
+                # the host execution of the kernels (tests/emu) is test infrastructure too: only the
+                # build script may name it, nothing that runs may load it
+                if name != "build.py":
+                    assert "flash_attn_emu" not in text and "wave_emu" not in text, os.path.join(dirpath, name)
 
 
 def test_missing_kernel_library_fails_loudly(tmp_path, monkeypatch):

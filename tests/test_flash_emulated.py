@@ -1,0 +1,170 @@
+"""The flash-attention kernels executed on the host, lane by lane (no GPU).
+
+tests/emu/wave_emu.h stands in for the HIP runtime header: the .hip sources of
+byteir_amd/csrc/flash_attn are compiled unchanged by a host compiler, a launch runs the grid's
+workgroups one after the other, every lane is a fiber, and the cross-lane operations (MFMA, the
+transposing LDS read, ballot, lane permutes, barriers) are rendezvous points that apply the
+documented register layouts.  What that buys:
+
+* the kernels' logic -- tiling, masks, online softmax, the backward's five products, grouped
+  heads and their partial sums, the key-axis split, the cache append and the decode kernel --
+  is checked against plain float32 attention without a GPU;
+* bounds: tensors that end at (or begin behind) a protected page, buffer loads that apply the
+  hardware's range check and must then land inside a tensor.  Every workgroup of the forward,
+  D, dK/dV, group-sum and dQ launches of the two ragged shapes that once ran in a session which
+  ended in a GPU memory fault (b4 h64/16 s1100 causal d64; b2 h64 sq2100 sk1500 d64) was executed
+  this way, with the guard page at either end: no stray access (about 6 CPU-minutes per
+  shape and placement; the test below repeats a sample of the workgroups).
+
+The emulation says nothing about timing, and nothing about what the compiler makes of the
+sources for the GPU."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import emu_util as E
+
+ATOL = 2e-2
+
+pytestmark = pytest.mark.skipif(not (os.path.exists(E.LIB) or os.path.exists("/opt/rocm/llvm/bin/clang++")),
+                                reason="no host clang to build the emulated library with")
+
+
+def reference(q, k, v, do, scale, window):
+    """float32 attention with autograd -> (o, lse, dq, dk, dv)."""
+    b, sq, h, d = q.shape
+    sk, hk = k.shape[1], k.shape[2]
+    qf, kf, vf = (t.float().detach().requires_grad_(True) for t in (q, k, v))
+    kx, vx = kf.repeat_interleave(h // hk, 2), vf.repeat_interleave(h // hk, 2)
+    s = torch.einsum("bqhd,bkhd->bhqk", qf, kx) * scale
+    i = torch.arange(sq)[:, None] + (sk - sq)
+    j = torch.arange(sk)[None, :]
+    mask = torch.zeros(sq, sk, dtype=torch.bool)
+    if window[1] >= 0:
+        mask |= j > i + window[1]
+    if window[0] >= 0:
+        mask |= j < i - window[0]
+    s = s.masked_fill(mask, float("-inf"))
+    p = torch.nan_to_num(torch.softmax(s, -1))  # rows that see no key: zeros
+    o = torch.einsum("bhqk,bkhd->bqhd", p, vx)
+    if do is None:
+        return o.detach(), torch.logsumexp(s.detach(), -1), None, None, None
+    o.backward(do.float())
+    return o.detach(), torch.logsumexp(s.detach(), -1), qf.grad, kf.grad, vf.grad
+
+
+def randn(shape, dtype, gen):
+    return torch.randn(shape, generator=gen).to(dtype)
+
+
+CASES = [
+    # b, sq, sk, h, h_k, d, window
+    (1, 128, 128, 2, 2, 64, (-1, 0)),
+    (1, 200, 333, 2, 1, 128, (-1, -1)),     # grouped heads, ragged, head_dim 128 (O staged through LDS)
+    (2, 77, 150, 2, 2, 32, (20, 5)),        # sliding window, surplus loader threads at head_dim 32
+    (1, 300, 260, 4, 2, 64, (-1, 0)),       # more queries than keys, causal: rows that see no key
+    (1, 100, 100, 1, 1, 96, (-1, 0)),       # a head_dim without a tuned kernel
+    (1, 200, 300, 8, 2, 64, (-1, 0)),       # backward shares a head group out over workgroups (partials + group sum)
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("case", CASES)
+def test_emulated_forward_and_backward_match_float32_attention(case, dtype):
+    b, sq, sk, h, hk, d, window = case
+    gen = torch.Generator().manual_seed(sq + sk + d)
+    q, k, v, do = randn((b, sq, h, d), dtype, gen), randn((b, sk, hk, d), dtype, gen), randn((b, sk, hk, d), dtype, gen), randn((b, sq, h, d), dtype, gen)
+    scale = 1.0 / np.sqrt(d)
+    o, lse = E.fwd(q, k, v, scale, window)
+    dq, dk, dv = E.bwd(do, q, k, v, o, lse, scale, window)
+    o_ref, lse_ref, dq_ref, dk_ref, dv_ref = reference(q, k, v, do, scale, window)
+    ulp = 2.0 ** -10 if dtype == torch.float16 else 2.0 ** -7
+    for name, got, want in (("o", o, o_ref), ("dq", dq, dq_ref), ("dk", dk, dk_ref), ("dv", dv, dv_ref)):
+        err = (got.float() - want).abs()
+        assert bool(torch.all(err <= ATOL + ulp * want.abs())), (name, case, float(err.max()))
+    seen = torch.isfinite(lse_ref)
+    assert torch.equal(torch.isposinf(lse), ~seen)  # a row without keys: LSE = +inf, O = 0
+    assert float((lse[seen] - lse_ref[seen]).abs().max()) <= 1e-3
+
+
+@pytest.mark.parametrize("case", [
+    # b, sq, sk (cache rows), h, h_k, d, appended rows
+    (2, 1, 300, 4, 2, 128, 1),      # decode kernel, head group in one score tile
+    (3, 1, 1500, 8, 2, 64, 1),      # ... with the keys split over workgroups and the merge kernel
+    (2, 3, 900, 8, 2, 32, 3),
+    (1, 70, 400, 2, 2, 64, 70),     # a prompt chunk: forward kernel with a per-batch key count
+    (1, 1, 600, 2, 2, 80, 1),       # a head_dim without a tuned kernel
+])
+def test_emulated_cache_call_appends_and_attends(case):
+    b, sq, sk, h, hk, d, n_new = case
+    dtype = torch.float16
+    gen = torch.Generator().manual_seed(sk + d)
+    q = randn((b, sq, h, d), dtype, gen)
+    kc, vc = randn((b, sk, hk, d), dtype, gen), randn((b, sk, hk, d), dtype, gen)
+    kn, vn = randn((b, n_new, hk, d), dtype, gen), randn((b, n_new, hk, d), dtype, gen)
+    lens = torch.tensor([sk - n_new - 7 * i for i in range(b)], dtype=torch.int32)
+    kc0, vc0 = kc.clone(), vc.clone()
+    o, lse = E.kvcache(q, kc, vc, kn, vn, lens, 1.0 / np.sqrt(d), (-1, 0))
+    for bi in range(b):
+        at, n = int(lens[bi]), int(lens[bi]) + n_new
+        kk, vv = kc0[bi].clone(), vc0[bi].clone()
+        kk[at:n], vv[at:n] = kn[bi], vn[bi]
+        assert torch.equal(kc[bi], kk) and torch.equal(vc[bi], vv)  # appended in place, nothing else touched
+        o_ref, lse_ref, *_ = reference(q[bi:bi + 1], kk[None, :n], vv[None, :n], None, 1.0 / np.sqrt(d), (-1, 0))
+        assert float((o[bi].float() - o_ref[0]).abs().max()) <= ATOL
+        assert float((lse[bi] - lse_ref[0]).abs().max()) <= 1e-3
+
+
+def test_a_tensor_that_is_too_short_is_reported_with_the_workgroup_and_thread():
+    """Negative controls: K one row short (a buffer load passes the descriptor's range check and
+    then lies outside every tensor) and O one row short (a plain store runs into the protected
+    page)."""
+    from byteir_amd import ops
+    b, sq, sk, h, d = 1, 256, 320, 2, 64
+    gen = torch.Generator().manual_seed(1)
+    mk = lambda rows, at_end=True: E.guarded((b, rows, h, d), torch.float16, at_end).copy_(randn((b, rows, h, d), torch.float16, gen))
+    q, k, v = mk(sq), mk(sk), mk(sk)
+    o, lse, rng = E.guarded((b, sq, h, d), torch.float16), E.guarded((b, h, sq), torch.float32), torch.zeros(2, dtype=torch.int64)
+    blob = ops.pack_flash_args(q, k, v, o, 0.125, (-1, -1), 0.0)
+    E._call("fwd", [q, k, v, rng, o, lse, None], blob, torch.float16)  # as declared: fine
+    k_short = mk(sk - 1)
+    with pytest.raises(E.EmuFault, match=r"outside every tensor.*workgroup \(\d+, 0, 0\) of \(\d+, 1, 1\), thread \d+"):
+        E._call("fwd", [q, k_short, v, rng, o, lse, None], blob, torch.float16)
+    o_short = E.guarded((b, sq - 1, h, d), torch.float16)
+    with pytest.raises(E.EmuFault, match=r"memory access outside every tensor.*workgroup"):
+        E._call("fwd", [q, k, v, rng, o_short, lse, None], blob, torch.float16)
+    E._call("fwd", [q, k, v, rng, o, lse, None], blob, torch.float16)  # and the library still works afterwards
+
+
+@pytest.mark.parametrize("at_end", [True, False])
+@pytest.mark.parametrize("shape", [
+    (4, 1100, 1100, 64, 16, 64, (-1, 0)),
+    (2, 2100, 1500, 64, 64, 64, (-1, -1)),
+])
+def test_a_sample_of_the_workgroups_of_the_two_ragged_shapes_stays_in_bounds(shape, at_end):
+    """Every launch of a forward and a backward call (forward; D, dK/dV, group sum, dQ) with one
+    workgroup in 331 executed (the first of every launch, and ids 330 modulo 331), all tensors
+    guarded.  The results are not looked at: with most workgroups left out the backward
+    reads unwritten intermediates, which cannot change an address."""
+    b, sq, sk, h, hk, d, window = shape
+    gen = torch.Generator().manual_seed(3)
+    dt = torch.bfloat16
+    g = lambda s, t=dt: E.guarded(s, t, at_end)
+    q, k, v, do = (g(s).copy_(randn(s, dt, gen)) for s in ((b, sq, h, d), (b, sk, hk, d), (b, sk, hk, d), (b, sq, h, d)))
+    o, lse = g((b, sq, h, d)).zero_(), g((b, h, sq), torch.float32).fill_(12.0)
+    ru = lambda x, m: -(-x // m) * m
+    out = (g(q.shape), g(k.shape), g(v.shape), g((b, h, ru(sq, 128)), torch.float32).zero_(), g((b, ru(sq, 128), h, ru(d, 32)), torch.float32))
+    L = E.lib()
+    try:
+        for stride in (331,):
+            for phase in (0, stride - 1):
+                E.select(stride, phase)
+                L.fa_emu_reset()
+                E.fwd(q, k, v, 1.0 / np.sqrt(d), window, out=(o, lse))
+                n_fwd = L.fa_emu_blocks_run()
+                E.bwd(do, q, k, v, o, lse, 1.0 / np.sqrt(d), window, out=out)
+                assert n_fwd >= 1 and L.fa_emu_blocks_run() - n_fwd >= 10
+    finally:
+        E.select(1, 0)

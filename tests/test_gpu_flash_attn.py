@@ -307,8 +307,10 @@ def test_random_cases_sweep():
     # Two ragged shapes that were part of a run which ended in a GPU memory fault (together with
     # a 64-rows-per-wave forward variant that is not in the tree).  The cause was not found;
     # the host-side bounds check (tests/test_flash_index_bounds.py) walks every address the
-    # in-tree kernels form for exactly these shapes and finds them all in bounds, but until the
-    # fault is explained they are not run on the GPU: unverified there.
+    # in-tree kernels form for exactly these shapes, and the kernels themselves have been
+    # executed on the host for every workgroup of these shapes under guarded tensors
+    # (tests/test_flash_emulated.py): all in bounds.  Until the fault is explained they are
+    # still not run on the GPU: unverified there.
     pytest.param((4, 1100, 1100, 64, 16, 64, True), marks=pytest.mark.skip(
         reason="ran in a session that ended in an unexplained GPU memory fault; checked on the host only")),
     pytest.param((2, 2100, 1500, 64, 64, 64, False), marks=pytest.mark.skip(
