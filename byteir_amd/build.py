@@ -102,7 +102,9 @@ def build_emu(verbose=False):
     jobs.append((os.path.join(emu, "wave_emu.cc"), os.path.join(obj, "wave_emu.o"), []))
     with concurrent.futures.ThreadPoolExecutor(max_workers=6) as pool:
         list(pool.map(lambda j: _run([clang] + j[2] + flags + ["-c", j[0], "-o", j[1]], False), jobs))
-    _run([clang, "-shared", "-fPIC", "-o", os.path.join(emu, "libflash_attn_emu.so")] + [j[1] for j in jobs], verbose)
+    # -Bsymbolic: the library's own calls stay inside it even when libflash_attn.so, which exports
+    # the same names, is already loaded in the process with RTLD_GLOBAL
+    _run([clang, "-shared", "-fPIC", "-Wl,-Bsymbolic", "-o", os.path.join(emu, "libflash_attn_emu.so")] + [j[1] for j in jobs], verbose)
 
 
 TARGETS = {"kernels": build_kernels, "flash": build_flash, "brt": build_brt, "index_check": build_index_check,
