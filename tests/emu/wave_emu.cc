@@ -56,6 +56,8 @@ bool g_abort = false;      // a lane gave up: the scheduler unwinds the launch
 std::string g_error;
 bool g_faulted = false;
 long long g_sel_stride = 1, g_sel_phase = 0, g_blocks_run = 0;
+int g_burst = 1;            // > 1: random wave order, up to this many passes in a row for the picked wave
+uint64_t g_rng = 1;
 std::vector<long long> g_sel_list;
 
 std::map<uintptr_t, size_t> g_ranges;           // registered [begin, begin + bytes)
@@ -127,22 +129,42 @@ bool run_block() {
     makecontext(&f.ctx, fiber_entry, 0);
     ++b.waves[t / kWave].n_alive;
   }
+  // One pass over a wave resumes each of its lanes once (a lane runs until it blocks at a
+  // cross-lane operation or a barrier, or ends).  Order of the waves: round robin, one pass each
+  // (the default), or -- to look for missing barriers -- a wave picked at random that is given up
+  // to `g_burst` passes in a row, so that it runs as far ahead of the others as the kernel's
+  // synchronisation lets it.
+  const unsigned n_waves = (unsigned)b.waves.size();
+  unsigned w = 0;
+  unsigned idle_waves = 0;  // consecutive waves that made no progress
   while (b.n_alive > 0) {
-    const uint64_t before = b.progress;
-    for (unsigned t = 0; t < n; ++t) {
-      Fiber &f = b.fibers[t];
-      if (f.done) continue;
-      b.cur = (int)t;
-      g_thread_idx = dim3(t % g_block_dim.x, (t / g_block_dim.x) % g_block_dim.y, t / (g_block_dim.x * g_block_dim.y));
-      g_in_fiber = true;
-      swapcontext(&b.main, &f.ctx);
-      g_in_fiber = false;
-      if (g_abort) return false;
+    if (g_burst > 1) {
+      g_rng = g_rng * 6364136223846793005ull + 1442695040888963407ull;
+      w = (unsigned)((g_rng >> 33) % n_waves);
     }
-    if (b.progress == before) {
+    const int passes = g_burst > 1 ? 1 + (int)((g_rng >> 20) % (uint64_t)g_burst) : 1;
+    bool moved = false;
+    for (int pass = 0; pass < passes; ++pass) {
+      const uint64_t before = b.progress;
+      for (unsigned t = w * kWave; t < std::min(n, (w + 1) * kWave); ++t) {
+        Fiber &f = b.fibers[t];
+        if (f.done) continue;
+        b.cur = (int)t;
+        g_thread_idx = dim3(t % g_block_dim.x, (t / g_block_dim.x) % g_block_dim.y, t / (g_block_dim.x * g_block_dim.y));
+        g_in_fiber = true;
+        swapcontext(&b.main, &f.ctx);
+        g_in_fiber = false;
+        if (g_abort) return false;
+      }
+      if (b.progress == before) break;  // the wave waits for the others
+      moved = true;
+    }
+    idle_waves = moved ? 0 : idle_waves + 1;
+    if (idle_waves > 64 * n_waves) {  // every wave has been tried many times over (random picks included)
       g_error = "deadlock: the lanes of a workgroup wait at different cross-lane operations or barriers" + where();
       return false;
     }
+    if (g_burst <= 1) w = (w + 1) % n_waves;
   }
   return true;
 }
@@ -450,6 +472,9 @@ void fa_emu_select(long long stride, long long phase) {
   fa_emu::g_sel_phase = phase;
 }
 void fa_emu_select_list(const long long *ids, int n) { fa_emu::g_sel_list.assign(ids, ids + n); }
+// burst <= 1: waves round robin; burst > 1: a wave picked at random (seeded) runs up to `burst`
+// passes in a row before the next pick
+void fa_emu_schedule(int burst, unsigned long long seed) { fa_emu::g_burst = burst; fa_emu::g_rng = seed * 2 + 1; }
 const char *fa_emu_last_error(void) { return fa_emu::last_error(); }
 int fa_emu_faulted(void) { return fa_emu::g_faulted ? 1 : 0; }
 void fa_emu_reset(void) { fa_emu::g_faulted = false; fa_emu::g_error.clear(); fa_emu::g_blocks_run = 0; fa_emu::g_last_error = 0; }

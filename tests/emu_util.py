@@ -41,6 +41,7 @@ def lib():
         L.fa_emu_unregister.argtypes = [_vp]
         L.fa_emu_select.argtypes = [ctypes.c_longlong, ctypes.c_longlong]
         L.fa_emu_blocks_run.restype = ctypes.c_longlong
+        L.fa_emu_schedule.argtypes = [ctypes.c_int, ctypes.c_ulonglong]
         _L = L
     return _L
 
@@ -48,6 +49,13 @@ def lib():
 def select(stride=1, phase=0):
     """Run only the workgroups of every launch whose linear id is `phase` modulo `stride`."""
     lib().fa_emu_select(stride, phase)
+
+
+def schedule(burst=1, seed=0):
+    """burst <= 1: the waves of a workgroup advance round robin.  burst > 1: a wave picked at random
+    runs up to `burst` steps in a row before the next pick, i.e. as far ahead of the others as
+    the kernel's own barriers allow."""
+    lib().fa_emu_schedule(burst, seed)
 
 
 def guarded(shape, dtype, at_end=True):

@@ -117,6 +117,37 @@ def test_emulated_cache_call_appends_and_attends(case):
         assert float((lse[bi] - lse_ref[0]).abs().max()) <= 1e-3
 
 
+@pytest.mark.parametrize("case", [
+    (1, 300, 700, 2, 2, 64, (-1, 0), torch.bfloat16),
+    (1, 300, 700, 2, 1, 128, (-1, -1), torch.float16),
+    (1, 300, 500, 2, 2, 96, (-1, 0), torch.bfloat16),
+])
+def test_results_do_not_depend_on_how_far_the_waves_run_apart(case):
+    """A missing barrier shows as a result that depends on the order in which the waves of a
+    workgroup advance.  The emulator's default is round robin; here a randomly picked wave runs
+    up to 7 or 400 steps in a row, which lets it get as far ahead as the kernels' barriers
+    permit (several tiles of the LDS ring, if they permitted it).  Forward and backward must be
+    bit-identical to the round-robin run.  (With the tile barrier of the forward kernel taken
+    out, the same comparison fails with differences of 0.4-0.6 in O: the check does bite.)"""
+    b, sq, sk, h, hk, d, window, dtype = case
+    gen = torch.Generator().manual_seed(5)
+    q, k, v, do = (randn(s, dtype, gen) for s in ((b, sq, h, d), (b, sk, hk, d), (b, sk, hk, d), (b, sq, h, d)))
+    scale = 1.0 / np.sqrt(d)
+    bits = lambda t: t.view(torch.int16) if t.dtype != torch.float32 else t.view(torch.int32)
+    try:
+        E.schedule(1, 0)
+        o0, lse0 = E.fwd(q, k, v, scale, window)
+        g0 = E.bwd(do, q, k, v, o0, lse0, scale, window)
+        for burst, seed in ((7, 3), (400, 2)):
+            E.schedule(burst, seed)
+            o1, lse1 = E.fwd(q, k, v, scale, window)
+            g1 = E.bwd(do, q, k, v, o1, lse1, scale, window)
+            for a, c in zip((o0, lse0, *g0), (o1, lse1, *g1)):
+                assert torch.equal(bits(a), bits(c)), (case, burst)
+    finally:
+        E.schedule(1, 0)
+
+
 def test_a_tensor_that_is_too_short_is_reported_with_the_workgroup_and_thread():
     """Negative controls: K one row short (a buffer load passes the descriptor's range check and
     then lies outside every tensor) and O one row short (a plain store runs into the protected
