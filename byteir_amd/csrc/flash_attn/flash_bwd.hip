@@ -463,6 +463,7 @@ __global__ void __launch_bounds__(256, (D <= 64 && KB == 1) ? 2 : 1) dkdv_kernel
         *reinterpret_cast<vec4 *>(&Kt[so]) = a;
         *reinterpret_cast<vec4 *>(&Vt[so]) = b;
       }
+    FA_WAVE_SYNC();  // the wave's two tiles are complete; they are read back across lanes
     const int oc = lane % CPRO, orow = lane / CPRO;
 #pragma unroll
     for (int it = 0; it < 32 / RPI; ++it) {
