@@ -98,13 +98,18 @@ def build_emu(verbose=False):
     os.makedirs(obj, exist_ok=True)
     flags = ["-std=c++17", "-O2", "-fPIC", "-DFA_EMULATE", f"-I{os.path.join(emu, 'include')}", f"-I{emu}",
              f"-I{os.path.join(CSRC, 'flash_attn')}", f"-I{os.path.join(ROOT, 'include')}", "-Wno-unknown-attributes"]
-    jobs = [(src, os.path.join(obj, os.path.basename(src) + ".o"), ["-x", "c++"]) for src in _glob("flash_attn", (".hip",))]
-    jobs.append((os.path.join(emu, "wave_emu.cc"), os.path.join(obj, "wave_emu.o"), []))
-    with concurrent.futures.ThreadPoolExecutor(max_workers=6) as pool:
-        list(pool.map(lambda j: _run([clang] + j[2] + flags + ["-c", j[0], "-o", j[1]], False), jobs))
-    # -Bsymbolic: the library's own calls stay inside it even when libflash_attn.so, which exports
-    # the same names, is already loaded in the process with RTLD_GLOBAL
-    _run([clang, "-shared", "-fPIC", "-Wl,-Bsymbolic", "-o", os.path.join(emu, "libflash_attn_emu.so")] + [j[1] for j in jobs], verbose)
+    flags += [f"-I{os.path.join(CSRC, 'kernels')}", "-ffp-contract=off"]
+    attn = [(src, os.path.join(obj, os.path.basename(src) + ".o"), ["-x", "c++"]) for src in _glob("flash_attn", (".hip",))]
+    # the reductions, the softmax and the input generator; device.hip is the HIP runtime plumbing and stays out
+    kern = [(os.path.join(CSRC, "kernels", n + ".hip"), os.path.join(obj, n + ".hip.o"), ["-x", "c++"]) for n in ("reduce", "softmax", "fill")]
+    rt = [(os.path.join(emu, "wave_emu.cc"), os.path.join(obj, "wave_emu.o"), [])]
+    with concurrent.futures.ThreadPoolExecutor(max_workers=8) as pool:
+        list(pool.map(lambda j: _run([clang] + j[2] + flags + ["-c", j[0], "-o", j[1]], False), attn + kern + rt))
+    # -Bsymbolic: a library's own calls stay inside it even when the GPU library, which exports the
+    # same names, is already loaded in the process with RTLD_GLOBAL
+    _run([clang, "-shared", "-fPIC", "-Wl,-Bsymbolic", "-o", os.path.join(emu, "libflash_attn_emu.so")] + [j[1] for j in attn + rt], verbose)
+    _run([clang, "-shared", "-fPIC", "-Wl,-Bsymbolic", "-Wl,--no-undefined", "-o", os.path.join(emu, "libbrt_rocm_kernels_emu.so")]
+         + [j[1] for j in kern + rt], verbose)
 
 
 TARGETS = {"kernels": build_kernels, "flash": build_flash, "brt": build_brt, "index_check": build_index_check,

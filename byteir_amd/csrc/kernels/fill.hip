@@ -17,6 +17,7 @@
 #include <cstdint>
 
 #include "brt_rocm_kernels.h"
+#include "launch.h"
 #include "brt_rocm_bench.h"
 
 namespace {
@@ -65,9 +66,9 @@ extern "C" int brt_rocm_fill(int dtype, int dist, uint64_t seed, void *ptr, size
   if (blocks > 256 * 64) blocks = 256 * 64;
   const dim3 grid((unsigned)blocks), block(256);
   switch (dtype) {
-  case BRT_ROCM_F32: fill_kernel<float><<<grid, block, 0, stream>>>(static_cast<float *>(ptr), n, dist, seed, a, b); break;
-  case BRT_ROCM_F16: fill_kernel<__half><<<grid, block, 0, stream>>>(static_cast<__half *>(ptr), n, dist, seed, a, b); break;
-  case BRT_ROCM_BF16: fill_kernel<__bf16><<<grid, block, 0, stream>>>(static_cast<__bf16 *>(ptr), n, dist, seed, a, b); break;
+  case BRT_ROCM_F32: BRT_ROCM_LAUNCH((fill_kernel<float>), grid, block, stream, static_cast<float *>(ptr), n, dist, seed, a, b); break;
+  case BRT_ROCM_F16: BRT_ROCM_LAUNCH((fill_kernel<__half>), grid, block, stream, static_cast<__half *>(ptr), n, dist, seed, a, b); break;
+  case BRT_ROCM_BF16: BRT_ROCM_LAUNCH((fill_kernel<__bf16>), grid, block, stream, static_cast<__bf16 *>(ptr), n, dist, seed, a, b); break;
   default: return hipErrorInvalidValue;
   }
   return hipGetLastError();

@@ -27,6 +27,7 @@
 #include <type_traits>
 
 #include "brt_rocm_kernels.h"
+#include "launch.h"
 #include "brt_rocm_bench.h"
 
 namespace {
@@ -419,8 +420,8 @@ hipError_t launch(const Plan &p, const T *in, TO *out, uint64_t A, uint64_t B, u
     if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
     const dim3 grid((unsigned)blocks), block(kBlock);
 #define ROW(G)                                                                                   \
-  if (vec) reduce_row_kernel<T, TO, OP, VF, G, false><<<grid, block, 0, stream>>>(in, out, units, B, p.S, p.seg, len); \
-  else reduce_row_kernel<T, TO, OP, VF, G, true><<<grid, block, 0, stream>>>(in, out, units, B, p.S, p.seg, len)
+  if (vec) BRT_ROCM_LAUNCH((reduce_row_kernel<T, TO, OP, VF, G, false>), grid, block, stream, in, out, units, B, p.S, p.seg, len); \
+  else BRT_ROCM_LAUNCH((reduce_row_kernel<T, TO, OP, VF, G, true>), grid, block, stream, in, out, units, B, p.S, p.seg, len)
     switch (p.g) {
     case 4: ROW(4); break;
     case 16: ROW(16); break;
@@ -439,13 +440,13 @@ hipError_t launch(const Plan &p, const T *in, TO *out, uint64_t A, uint64_t B, u
   if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
   const dim3 grid((unsigned)blocks), block(kBlock);
   if (p.kind == 3 && vec) {
-    if (p.g == 4 * kBlock) reduce_colwide_kernel<T, TO, OP, VF, 4, kColWideU><<<grid, block, 0, stream>>>(in, out, B, C, p.S, p.seg, col_tiles, len);
-    else reduce_colwide_kernel<T, TO, OP, VF, 2, kColWideU><<<grid, block, 0, stream>>>(in, out, B, C, p.S, p.seg, col_tiles, len);
+    if (p.g == 4 * kBlock) BRT_ROCM_LAUNCH((reduce_colwide_kernel<T, TO, OP, VF, 4, kColWideU>), grid, block, stream, in, out, B, C, p.S, p.seg, col_tiles, len);
+    else BRT_ROCM_LAUNCH((reduce_colwide_kernel<T, TO, OP, VF, 2, kColWideU>), grid, block, stream, in, out, B, C, p.S, p.seg, col_tiles, len);
     return hipGetLastError();
   }
 #define COL(TX)                                                                                  \
-  if (vec) reduce_col_kernel<T, TO, OP, VF, TX><<<grid, block, 0, stream>>>(in, out, B, C, p.S, p.seg, col_tiles, len); \
-  else reduce_col_kernel<T, TO, OP, 1, TX><<<grid, block, 0, stream>>>(in, out, B, C, p.S, p.seg, col_tiles, len)
+  if (vec) BRT_ROCM_LAUNCH((reduce_col_kernel<T, TO, OP, VF, TX>), grid, block, stream, in, out, B, C, p.S, p.seg, col_tiles, len); \
+  else BRT_ROCM_LAUNCH((reduce_col_kernel<T, TO, OP, 1, TX>), grid, block, stream, in, out, B, C, p.S, p.seg, col_tiles, len)
   switch (tx) {
   case 8: COL(8); break;
   case 32: COL(32); break;
@@ -530,8 +531,8 @@ extern "C" int brt_rocm_reduce_ex(int op, int dtype, const void *input, void *ou
     }
     const uint64_t n = (uint64_t)A * C, blocks = (n + kBlock - 1) / kBlock;
     if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
-    if (dtype == BRT_ROCM_F32) reduce_fill_kernel<float><<<dim3((unsigned)blocks), dim3(kBlock), 0, stream>>>(static_cast<float *>(output), n, value);
-    else reduce_fill_kernel<__half><<<dim3((unsigned)blocks), dim3(kBlock), 0, stream>>>(static_cast<__half *>(output), n, value);
+    if (dtype == BRT_ROCM_F32) BRT_ROCM_LAUNCH((reduce_fill_kernel<float>), dim3((unsigned)blocks), dim3(kBlock), stream, static_cast<float *>(output), n, value);
+    else BRT_ROCM_LAUNCH((reduce_fill_kernel<__half>), dim3((unsigned)blocks), dim3(kBlock), stream, static_cast<__half *>(output), n, value);
     const hipError_t e = hipGetLastError();
     if (e == hipSuccess && first_pass_done) return hipEventRecord(first_pass_done, stream);
     return e;

@@ -26,6 +26,7 @@
 #include <cstdint>
 
 #include "brt_rocm_kernels.h"
+#include "launch.h"
 
 namespace {
 
@@ -589,7 +590,7 @@ hipError_t run_inner(const T *in, T *out, uint64_t A, uint64_t B, uint64_t C, vo
   }
   if (col_tiles > 0xffffffffull || A * col_tiles * S > 0x7fffffffull) return hipErrorInvalidValue;
   const dim3 grid((unsigned)(A * col_tiles * S)), block(kBlock);
-#define INNER(V, X, M) softmax_inner_kernel<T, V, X, M><<<grid, block, 0, stream>>>(in, out, B, C, (uint32_t)col_tiles, (uint32_t)S, seg_rows, part)
+#define INNER(V, X, M) BRT_ROCM_LAUNCH((softmax_inner_kernel<T, V, X, M>), grid, block, stream, in, out, B, C, (uint32_t)col_tiles, (uint32_t)S, seg_rows, part)
 #define INNER_TX(V, M) do { if (tx == 256) INNER(V, 256, M); else if (tx == 64) INNER(V, 64, M); else INNER(V, 16, M); } while (0)
   hipError_t e = hipSuccess;
   if (S == 1) {
@@ -622,8 +623,8 @@ hipError_t run(const T *in, T *out, uint64_t rows, uint64_t cols, hipStream_t st
     if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
     const dim3 grid((unsigned)blocks), block(kBlock);
     const uint32_t nv = (uint32_t)nvec;
-    if (nvec <= 64) softmax_wave_kernel<T, 1><<<grid, block, 0, stream>>>(in, out, rows, nv);
-    else if (nvec <= 128) softmax_wave_kernel<T, 2><<<grid, block, 0, stream>>>(in, out, rows, nv);
+    if (nvec <= 64) BRT_ROCM_LAUNCH((softmax_wave_kernel<T, 1>), grid, block, stream, in, out, rows, nv);
+    else if (nvec <= 128) BRT_ROCM_LAUNCH((softmax_wave_kernel<T, 2>), grid, block, stream, in, out, rows, nv);
     else {
       // longer rows: RW waves per row, two vectors per lane
       const int rw = nvec <= 256 ? 2 : nvec <= 512 ? 4 : 8;
@@ -632,8 +633,8 @@ hipError_t run(const T *in, T *out, uint64_t rows, uint64_t cols, hipStream_t st
       if (sblocks > 0x7fffffffull) return hipErrorInvalidValue;
       const dim3 sgrid((unsigned)sblocks), sblock(kSplitWaves * 64);
 #define SPLIT(RW)                                                                                \
-  if (full) softmax_split_kernel<T, RW, true><<<sgrid, sblock, 0, stream>>>(in, out, rows, nv);  \
-  else softmax_split_kernel<T, RW, false><<<sgrid, sblock, 0, stream>>>(in, out, rows, nv)
+  if (full) BRT_ROCM_LAUNCH((softmax_split_kernel<T, RW, true>), sgrid, sblock, stream, in, out, rows, nv);  \
+  else BRT_ROCM_LAUNCH((softmax_split_kernel<T, RW, false>), sgrid, sblock, stream, in, out, rows, nv)
       if (rw == 2) { SPLIT(2); } else if (rw == 4) { SPLIT(4); } else { SPLIT(8); }
 #undef SPLIT
     }
@@ -648,13 +649,13 @@ hipError_t run(const T *in, T *out, uint64_t rows, uint64_t cols, hipStream_t st
     const uint64_t xr = span * EPV;                      // floats a workgroup must hold
     // registers per thread and threads per workgroup are sized so that several workgroups share
     // a CU while the row is short enough, and one row's loads overlap another's stores
-    if (xr <= 256 * 32) softmax_regs_kernel<T, 256, 32><<<grid, dim3(256), 0, stream>>>(in, out, cols);
-    else if (xr <= 256 * 64) softmax_regs_kernel<T, 256, 64><<<grid, dim3(256), 0, stream>>>(in, out, cols);
-    else if (xr <= 1024 * 32) softmax_regs_kernel<T, 1024, 32><<<grid, dim3(1024), 0, stream>>>(in, out, cols);
-    else softmax_stream_kernel<T, 1024><<<grid, dim3(1024), 0, stream>>>(in, out, cols);
+    if (xr <= 256 * 32) BRT_ROCM_LAUNCH((softmax_regs_kernel<T, 256, 32>), grid, dim3(256), stream, in, out, cols);
+    else if (xr <= 256 * 64) BRT_ROCM_LAUNCH((softmax_regs_kernel<T, 256, 64>), grid, dim3(256), stream, in, out, cols);
+    else if (xr <= 1024 * 32) BRT_ROCM_LAUNCH((softmax_regs_kernel<T, 1024, 32>), grid, dim3(1024), stream, in, out, cols);
+    else BRT_ROCM_LAUNCH((softmax_stream_kernel<T, 1024>), grid, dim3(1024), stream, in, out, cols);
     return hipGetLastError();
   }
-  softmax_block_kernel<T><<<grid, dim3(kBlock), 0, stream>>>(in, out, cols);
+  BRT_ROCM_LAUNCH((softmax_block_kernel<T>), grid, dim3(kBlock), stream, in, out, cols);
   return hipGetLastError();
 }
 

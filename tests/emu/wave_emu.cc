@@ -60,6 +60,7 @@ int g_burst = 1;            // > 1: random wave order, up to this many passes in
 uint64_t g_rng = 1;
 std::vector<long long> g_sel_list;
 
+std::vector<char *> g_stacks;                   // lane stacks, indexed by thread id, reused by every workgroup
 std::map<uintptr_t, size_t> g_ranges;           // registered [begin, begin + bytes)
 struct Guarded { void *map; size_t map_bytes; };
 std::map<uintptr_t, Guarded> g_guarded;         // user pointer -> mapping
@@ -120,8 +121,13 @@ bool run_block() {
   for (unsigned t = 0; t < n; ++t) {
     Fiber &f = b.fibers[t];
     f.tid = t;
-    f.stack = static_cast<char *>(mmap(nullptr, kStackBytes, PROT_READ | PROT_WRITE, MAP_PRIVATE | MAP_ANONYMOUS | MAP_NORESERVE, -1, 0));
-    if (f.stack == MAP_FAILED) { f.stack = nullptr; g_error = "no memory for a lane's stack"; return false; }
+    if (t < g_stacks.size()) {
+      f.stack = g_stacks[t];  // stacks are kept from one workgroup to the next
+    } else {
+      f.stack = static_cast<char *>(mmap(nullptr, kStackBytes, PROT_READ | PROT_WRITE, MAP_PRIVATE | MAP_ANONYMOUS | MAP_NORESERVE, -1, 0));
+      if (f.stack == MAP_FAILED) { f.stack = nullptr; g_error = "no memory for a lane's stack"; return false; }
+      g_stacks.push_back(f.stack);
+    }
     getcontext(&f.ctx);
     f.ctx.uc_stack.ss_sp = f.stack;
     f.ctx.uc_stack.ss_size = kStackBytes;
@@ -170,10 +176,7 @@ bool run_block() {
 }
 
 void free_stacks() {
-  if (!g_blk) return;
-  for (Fiber &f : g_blk->fibers)
-    if (f.stack) munmap(f.stack, kStackBytes);
-  g_blk->fibers.clear();
+  if (g_blk) g_blk->fibers.clear();  // the stacks themselves stay in g_stacks for the next workgroup
 }
 
 bool selected(long long id) {

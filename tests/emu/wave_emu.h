@@ -119,10 +119,39 @@ struct alignas(16) float4 { float x, y, z, w; };
 struct alignas(8) int2 { int x, y; };
 struct alignas(16) int4 { int x, y, z, w; };
 
+// ---- device math helpers ------------------------------------------------------------------------
+inline float __uint_as_float(unsigned u) { float f; std::memcpy(&f, &u, 4); return f; }
+inline unsigned __float_as_uint(float f) { unsigned u; std::memcpy(&u, &f, 4); return u; }
+// single roundings, never contracted (the host build is compiled with -ffp-contract=off)
+inline float __fmul_rn(float a, float b) { return a * b; }
+inline float __fadd_rn(float a, float b) { return a + b; }
+inline float __fmaf_rn(float a, float b, float c) { return std::fma(a, b, c); }
+
+// ---- hip_fp16.h: the half type as the kernels use it ---------------------------------------------
+struct __half {
+  _Float16 v;
+  __half() = default;
+  __half(_Float16 x) : v(x) {}
+  operator _Float16() const { return v; }
+};
+struct alignas(4) __half2 { __half x, y; };
+inline float __half2float(__half h) { return (float)h.v; }
+inline __half __float2half_rn(float f) { return __half((_Float16)f); }
+inline __half __float2half(float f) { return __half((_Float16)f); }
+inline float2 __half22float2(__half2 h) { return float2{(float)h.x.v, (float)h.y.v}; }
+
 // ---- the HIP runtime calls the launchers make --------------------------------------------------
 typedef int hipError_t;
 typedef void *hipStream_t;
-constexpr hipError_t hipSuccess = 0, hipErrorInvalidValue = 1, hipErrorOutOfMemory = 2, hipErrorLaunchFailure = 719;
+typedef void *hipEvent_t;
+constexpr hipError_t hipSuccess = 0, hipErrorInvalidValue = 1, hipErrorOutOfMemory = 2, hipErrorInvalidDevice = 101,
+                     hipErrorInvalidSymbol = 13, hipErrorLaunchFailure = 719;
+enum hipMemcpyKind { hipMemcpyHostToHost, hipMemcpyHostToDevice, hipMemcpyDeviceToHost, hipMemcpyDeviceToDevice, hipMemcpyDefault };
+inline hipError_t hipMemcpyAsync(void *dst, const void *src, size_t bytes, hipMemcpyKind, hipStream_t) { std::memmove(dst, src, bytes); return hipSuccess; }
+inline hipError_t hipMemsetAsync(void *dst, int value, size_t bytes, hipStream_t) { std::memset(dst, value, bytes); return hipSuccess; }
+inline hipError_t hipGetDevice(int *dev) { *dev = 0; return hipSuccess; }
+inline hipError_t hipEventRecord(hipEvent_t, hipStream_t) { return hipSuccess; }
+inline hipError_t hipGetSymbolAddress(void **p, const void *symbol) { *p = const_cast<void *>(symbol); return hipSuccess; }
 extern hipError_t g_last_error;
 inline hipError_t hipGetLastError() { const hipError_t e = g_last_error; g_last_error = hipSuccess; return e; }
 inline const char *hipGetErrorString(hipError_t e) {
@@ -146,6 +175,27 @@ using fa_emu::hipStream_t;
 using fa_emu::hipSuccess;
 using fa_emu::hipErrorInvalidValue;
 using fa_emu::hipGetLastError;
+using fa_emu::hipEvent_t;
+using fa_emu::hipErrorInvalidDevice;
+using fa_emu::hipErrorInvalidSymbol;
+using fa_emu::hipGetDevice;
+using fa_emu::hipMemcpyKind;
+using fa_emu::hipMemcpyDeviceToDevice;
+using fa_emu::hipMemcpyAsync;
+using fa_emu::hipMemsetAsync;
+using fa_emu::__uint_as_float;
+using fa_emu::__float_as_uint;
+using fa_emu::__fmul_rn;
+using fa_emu::__fadd_rn;
+using fa_emu::__fmaf_rn;
+using fa_emu::hipEventRecord;
+using fa_emu::hipGetSymbolAddress;
+using fa_emu::__half;
+using fa_emu::__half2;
+using fa_emu::__half2float;
+using fa_emu::__float2half_rn;
+using fa_emu::__float2half;
+using fa_emu::__half22float2;
 using fa_emu::hipGetErrorString;
 using fa_emu::hipMallocAsync;
 using fa_emu::hipFreeAsync;
@@ -181,6 +231,9 @@ using std::min;
 #define __builtin_amdgcn_fdot2(...) ::fa_emu::fdot2(__VA_ARGS__)
 #define __builtin_amdgcn_fdot2_f32_bf16(...) ::fa_emu::fdot2(__VA_ARGS__)
 
+#define HIP_SYMBOL(x) (&(x))
+#define __align__(n) __attribute__((aligned(n)))
+#define BRT_ROCM_LAUNCH(kernel, grid, block, stream, ...) FA_LAUNCH(kernel, grid, block, stream, __VA_ARGS__)
 #define FA_LAUNCH(kernel, grid, block, stream, ...) \
   ((void)(stream), ::fa_emu::g_last_error = ::fa_emu::launch((grid), (block), [&]() { kernel(__VA_ARGS__); }) ? ::fa_emu::hipErrorLaunchFailure : ::fa_emu::g_last_error)
 #define FA_WAVE_SYNC() ::fa_emu::wave_sync()

@@ -118,3 +118,92 @@ def kvcache(q, kcache, vcache, knew, vnew, seqlens_k, scale, window=(-1, -1)):
     _call("kvcache", [q, kcache, vcache, knew, vnew, seqlens_k, o, lse],
           ops.pack_flash_kvcache_args(q, kcache, vcache, knew, vnew, o, scale, window), q.dtype)
     return o, lse
+
+
+# ---- the reductions, the softmax and the input generator on the host ------------------------
+KLIB = os.path.join(ROOT, "tests", "emu", "libbrt_rocm_kernels_emu.so")
+_K = None
+
+
+def klib():
+    """tests/emu/libbrt_rocm_kernels_emu.so: reduce.hip, softmax.hip and fill.hip compiled for the
+    host (the C ABI of include/brt_rocm_kernels.h for those three, on host memory)."""
+    global _K
+    if _K is None:
+        if not os.path.exists(KLIB):
+            subprocess.check_call([sys.executable, "-m", "byteir_amd.build", "emu"], cwd=ROOT)
+        K = ctypes.CDLL(KLIB)
+        sz, i32 = ctypes.c_size_t, ctypes.c_int
+        K.brt_rocm_reduce_workspace_bytes.argtypes = [i32, sz, sz, sz]
+        K.brt_rocm_reduce_workspace_bytes.restype = sz
+        K.brt_rocm_reduce.argtypes = [i32, i32, _vp, _vp, sz, sz, sz, _vp, sz, _vp]
+        K.brt_rocm_reduce_static.argtypes = [i32, i32, _vp, _vp, sz, sz, sz, _vp]
+        K.brt_rocm_softmax.argtypes = [i32, _vp, _vp, sz, sz, _vp]
+        K.brt_rocm_softmax_axis.argtypes = [i32, _vp, _vp, sz, sz, sz, _vp]
+        K.brt_rocm_fill.argtypes = [i32, i32, ctypes.c_uint64, _vp, sz, ctypes.c_float, ctypes.c_float, _vp]
+        K.fa_emu_last_error.restype = ctypes.c_char_p
+        K.fa_emu_alloc.restype = _vp
+        K.fa_emu_alloc.argtypes = [sz, i32]
+        K.fa_emu_register.argtypes = [_vp, sz]
+        K.fa_emu_unregister.argtypes = [_vp]
+        _K = K
+    return _K
+
+
+_CODE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
+
+
+def kguarded(shape, dtype, at_end=True, offset_elems=0):
+    """Like guarded(), from the kernels library's own table; `offset_elems` shifts the tensor's
+    start off the 16-byte grid (at_end: the end stays against the protected page)."""
+    K = klib()
+    n = int(np.prod(shape))
+    es = torch.empty(0, dtype=dtype).element_size()
+    nbytes = (n + offset_elems) * es
+    p = K.fa_emu_alloc(max(nbytes, 16), 1 if at_end else 0)
+    if not p:
+        raise MemoryError("fa_emu_alloc")
+    if at_end:  # fa_emu_alloc rounds the size up to 16 bytes: push the tensor against the page's end
+        p += (-nbytes) % 16 if nbytes >= 16 else 0
+    buf = (ctypes.c_char * max(nbytes, 16)).from_address(p)
+    return torch.frombuffer(buf, dtype=dtype, count=n, offset=offset_elems * es).reshape(shape)
+
+
+def _kcheck(rc, what):
+    K = klib()
+    if rc:
+        msg = K.fa_emu_last_error().decode()
+        K.fa_emu_reset()
+        raise EmuFault(f"{what}: rc {rc}: {msg}")
+
+
+def reduce(op, x, A, B, C, out=None, static=False):
+    """brt_rocm_reduce (or brt_rocm_reduce_static) of x viewed as [A, B, C] over B -> [A * C]."""
+    K = klib()
+    code = _CODE[x.dtype]
+    out = out if out is not None else torch.empty(A * C, dtype=x.dtype)
+    if static:
+        rc = K.brt_rocm_reduce_static(op, code, x.data_ptr(), out.data_ptr(), A, B, C, None)
+    else:
+        nws = K.brt_rocm_reduce_workspace_bytes(code, A, B, C)
+        ws = kguarded((max(nws, 16),), torch.uint8) if nws else None
+        rc = K.brt_rocm_reduce(op, code, x.data_ptr(), out.data_ptr(), A, B, C, ws.data_ptr() if ws is not None else None, nws, None)
+    _kcheck(rc, "brt_rocm_reduce")
+    return out
+
+
+def softmax(x, out=None, axis_abc=None):
+    K = klib()
+    out = out if out is not None else torch.empty_like(x)
+    if axis_abc is None:
+        rows, cols = x.shape
+        rc = K.brt_rocm_softmax(_CODE[x.dtype], x.data_ptr(), out.data_ptr(), rows, cols, None)
+    else:
+        rc = K.brt_rocm_softmax_axis(_CODE[x.dtype], x.data_ptr(), out.data_ptr(), *axis_abc, None)
+    _kcheck(rc, "brt_rocm_softmax")
+    return out
+
+
+def fill(t, dist, seed, a=0.0, b=1.0):
+    _kcheck(klib().brt_rocm_fill(_CODE[t.dtype], dist, seed, t.data_ptr(), t.numel(), a, b, None), "brt_rocm_fill")
+    return t
