@@ -292,6 +292,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="counter-collection mode: one copy kernel of known size, then two C2 steps, two cache-decode calls and two softmax calls")
+    ap.add_argument("--mfma-probe", action="store_true",
+                    help="counter-collection mode: only the MFMA rate probe, 40 launches per operand set (fp16 / bf16, zeros / N(0,1))")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build is single-GPU (one process, one MI355X); run with --gpus 1")
@@ -334,6 +336,27 @@ def main():
         lambda: ops.reduce_abc(_lib.REDUCE_MAX, nxt(), out_row, R, Cc, 1, workspace=ws_row),
         lambda: ops.reduce_abc(_lib.REDUCE_SUM, nxt(), out_row, R, Cc, 1, workspace=ws_row),
     ]
+
+    if args.mfma_probe:
+        # for `rocprofv3 --pmc GRBM_GUI_ACTIVE --kernel-trace`: busy cycles over duration = the clock the
+        # chip held during each launch
+        del xs
+        blocks, iters = torch.cuda.get_device_properties(0).multi_processor_count, 8000
+        opnd = torch.empty(blocks * 512 * 256, dtype=torch.uint8, device="cuda")
+        sink = torch.empty(blocks * 512, dtype=torch.float32, device="cuda")
+        flop = blocks * 8 * iters * 16 * 32768
+        rates = {}
+        for name, code, dt in (("f16", 1, torch.float16), ("bf16", 2, torch.bfloat16)):
+            for what in ("zeros", "normal"):
+                if what == "zeros":
+                    opnd.zero_()
+                else:
+                    ops.fill(opnd.view(dt), _lib.FILL_NORMAL, SEED["c4q"], 0.0, 1.0)
+                probe = lambda: _lib.check(K.brt_rocm_mfma_rate_probe(code, opnd.data_ptr(), opnd.numel(), sink.data_ptr(), sink.numel() * 4, blocks, iters, sp))
+                r = time_regions(ev, [probe], 10, 10)
+                rates[f"{name}_{what}"] = round(flop / (r["ms"] * 1e-3) / 1e12, 1)
+        print(json.dumps({"mfma_probe": True, "TFLOPs": rates, "flop_per_launch": flop, "launches_per_operand_set": 40}))
+        return
 
     if args.pmc_probe:
         dst = torch.empty_like(xs[0])
