@@ -85,31 +85,39 @@ def build_test_kernels(verbose=False):
 
 
 def build_emu(verbose=False):
-    """The flash-attention sources compiled for the host (tests/emu/wave_emu.h stands in for the
-    HIP runtime header and runs every lane as a fiber): tests/emu/libflash_attn_emu.so, the
-    library's C ABI on host memory, for the tests that need no GPU.  Needs a host clang (vector
-    extensions, _Float16, __bf16); skipped when there is none."""
+    """The three libraries once more, for the host: the .hip sources compiled unchanged by a host
+    clang against tests/emu/wave_emu.h (which stands in for the HIP runtime header and runs every
+    lane as a fiber), a host stand-in for the device layer, and the runtime linked against them
+    -- tests/emu/lib/{libbrt_rocm_kernels,libflash_attn,libbrt}.so, the same C ABIs on host
+    memory, for the tests that need no GPU.  Needs a host clang (vector extensions, _Float16,
+    __bf16); skipped when there is none.  Nothing in the package loads these."""
     clang = os.path.join(os.environ.get("ROCM_PATH", "/opt/rocm"), "llvm", "bin", "clang++")
     emu = os.path.join(ROOT, "tests", "emu")
     if not os.path.exists(clang) or not os.path.isdir(emu):
         return
     import concurrent.futures
-    obj = os.path.join(emu, "obj")
+    obj, out = os.path.join(emu, "obj"), os.path.join(emu, "lib")
     os.makedirs(obj, exist_ok=True)
+    os.makedirs(out, exist_ok=True)
     flags = ["-std=c++17", "-O2", "-fPIC", "-DFA_EMULATE", f"-I{os.path.join(emu, 'include')}", f"-I{emu}",
-             f"-I{os.path.join(CSRC, 'flash_attn')}", f"-I{os.path.join(ROOT, 'include')}", "-Wno-unknown-attributes"]
-    flags += [f"-I{os.path.join(CSRC, 'kernels')}", "-ffp-contract=off"]
+             f"-I{os.path.join(CSRC, 'flash_attn')}", f"-I{os.path.join(CSRC, 'kernels')}", f"-I{os.path.join(ROOT, 'include')}",
+             "-Wno-unknown-attributes", "-ffp-contract=off"]
     attn = [(src, os.path.join(obj, os.path.basename(src) + ".o"), ["-x", "c++"]) for src in _glob("flash_attn", (".hip",))]
-    # the reductions, the softmax and the input generator; device.hip is the HIP runtime plumbing and stays out
+    # the reductions, the softmax and the input generator; device.hip is the HIP runtime plumbing:
+    # tests/emu/device_emu.cc takes its place
     kern = [(os.path.join(CSRC, "kernels", n + ".hip"), os.path.join(obj, n + ".hip.o"), ["-x", "c++"]) for n in ("reduce", "softmax", "fill")]
+    kern.append((os.path.join(emu, "device_emu.cc"), os.path.join(obj, "device_emu.o"), []))
     rt = [(os.path.join(emu, "wave_emu.cc"), os.path.join(obj, "wave_emu.o"), [])]
     with concurrent.futures.ThreadPoolExecutor(max_workers=8) as pool:
         list(pool.map(lambda j: _run([clang] + j[2] + flags + ["-c", j[0], "-o", j[1]], False), attn + kern + rt))
-    # -Bsymbolic: a library's own calls stay inside it even when the GPU library, which exports the
-    # same names, is already loaded in the process with RTLD_GLOBAL
-    _run([clang, "-shared", "-fPIC", "-Wl,-Bsymbolic", "-o", os.path.join(emu, "libflash_attn_emu.so")] + [j[1] for j in attn + rt], verbose)
-    _run([clang, "-shared", "-fPIC", "-Wl,-Bsymbolic", "-Wl,--no-undefined", "-o", os.path.join(emu, "libbrt_rocm_kernels_emu.so")]
+    # -Bsymbolic: a library's own calls stay inside it whatever else the process has loaded
+    _run([clang, "-shared", "-fPIC", "-Wl,-Bsymbolic", "-o", os.path.join(out, "libflash_attn.so")] + [j[1] for j in attn + rt], verbose)
+    _run([clang, "-shared", "-fPIC", "-Wl,-Bsymbolic", "-Wl,--no-undefined", "-o", os.path.join(out, "libbrt_rocm_kernels.so")]
          + [j[1] for j in kern + rt], verbose)
+    srcs = _glob("brt", (".cc",))
+    if srcs:
+        _run(["g++"] + CXX_FLAGS + [f"-I{os.path.join(CSRC, 'brt')}", "-o", os.path.join(out, "libbrt.so")] + srcs
+             + [f"-L{out}", "-lbrt_rocm_kernels", "-ldl", "-Wl,-rpath,$ORIGIN"], verbose)
 
 
 TARGETS = {"kernels": build_kernels, "flash": build_flash, "brt": build_brt, "index_check": build_index_check,

@@ -62,6 +62,7 @@ std::vector<long long> g_sel_list;
 
 std::vector<char *> g_stacks;                   // lane stacks, indexed by thread id, reused by every workgroup
 std::map<uintptr_t, size_t> g_ranges;           // registered [begin, begin + bytes)
+int g_caller_ranges = 0;                        // how many of them the caller registered (the rest is library scratch)
 struct Guarded { void *map; size_t map_bytes; };
 std::map<uintptr_t, Guarded> g_guarded;         // user pointer -> mapping
 
@@ -420,8 +421,10 @@ unsigned shfl_xor_u32(unsigned v, int mask, int width) {
 // ---- memory ------------------------------------------------------------------------------------
 void register_range(const void *p, size_t bytes) { g_ranges[reinterpret_cast<uintptr_t>(p)] = bytes; }
 void unregister_range(const void *p) { g_ranges.erase(reinterpret_cast<uintptr_t>(p)); }
+// The table is only consulted when the caller has entered its tensors; scratch that the library
+// itself takes (hipMallocAsync) is in it too, but on its own says nothing about the caller's memory.
 bool range_ok(const void *p, size_t bytes) {
-  if (g_ranges.empty()) return true;
+  if (g_caller_ranges == 0) return true;
   const uintptr_t a = reinterpret_cast<uintptr_t>(p);
   auto it = g_ranges.upper_bound(a);
   if (it == g_ranges.begin()) return false;
@@ -466,8 +469,8 @@ hipError_t hipFreeAsync(void *p, hipStream_t) {
 extern "C" {
 void *fa_emu_alloc(size_t bytes, int at_end) { return fa_emu::guarded_alloc(bytes, at_end != 0); }
 void fa_emu_free(void *p) { fa_emu::guarded_free(p); }
-void fa_emu_register(const void *p, size_t bytes) { fa_emu::register_range(p, bytes); }
-void fa_emu_unregister(const void *p) { fa_emu::unregister_range(p); }
+void fa_emu_register(const void *p, size_t bytes) { fa_emu::register_range(p, bytes); ++fa_emu::g_caller_ranges; }
+void fa_emu_unregister(const void *p) { fa_emu::unregister_range(p); if (fa_emu::g_caller_ranges > 0) --fa_emu::g_caller_ranges; }
 // run only the workgroups whose linear id (x fastest) is phase modulo stride; (1, 0): all
 void fa_emu_select(long long stride, long long phase) {
   fa_emu::g_sel_list.clear();

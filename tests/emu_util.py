@@ -1,6 +1,6 @@
-"""The flash-attention library executed on the host (tests/emu/libflash_attn_emu.so: the HIP
-sources compiled against tests/emu/wave_emu.h, every lane a fiber): the same C ABI as
-libflash_attn.so, on CPU tensors.  Tensors are registered with the emulator for the duration of
+"""The flash-attention library executed on the host (tests/emu/lib/libflash_attn.so: the HIP
+sources compiled against tests/emu/wave_emu.h, every lane a fiber): the same C ABI as the GPU
+library of that name, on CPU tensors.  Tensors are registered with the emulator for the duration of
 a call, so that buffer loads that pass their descriptor's range check are also checked against
 the tensors' extents; `guarded` tensors end at (or start behind) a protected page, which turns
 any stray access of a plain load or store into a reported fault."""
@@ -13,7 +13,8 @@ import numpy as np
 import torch
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-LIB = os.path.join(ROOT, "tests", "emu", "libflash_attn_emu.so")
+EMU_LIB_DIR = os.path.join(ROOT, "tests", "emu", "lib")
+LIB = os.path.join(EMU_LIB_DIR, "libflash_attn.so")
 _vp = ctypes.c_void_p
 _L = None
 
@@ -121,13 +122,14 @@ def kvcache(q, kcache, vcache, knew, vnew, seqlens_k, scale, window=(-1, -1)):
 
 
 # ---- the reductions, the softmax and the input generator on the host ------------------------
-KLIB = os.path.join(ROOT, "tests", "emu", "libbrt_rocm_kernels_emu.so")
+KLIB = os.path.join(EMU_LIB_DIR, "libbrt_rocm_kernels.so")
 _K = None
 
 
 def klib():
-    """tests/emu/libbrt_rocm_kernels_emu.so: reduce.hip, softmax.hip and fill.hip compiled for the
-    host (the C ABI of include/brt_rocm_kernels.h for those three, on host memory)."""
+    """tests/emu/lib/libbrt_rocm_kernels.so: reduce.hip, softmax.hip and fill.hip compiled for the
+    host plus a host stand-in for the device layer (the C ABI of include/brt_rocm_kernels.h on
+    host memory)."""
     global _K
     if _K is None:
         if not os.path.exists(KLIB):
