@@ -1,10 +1,10 @@
 #!/usr/bin/env python3
 """Benchmark of the op-kernel hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2] [--no-extras] [--no-cpu] [--pmc-probe]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2] [--no-extras] [--no-cpu] [--pmc-probe | --mfma-probe]
 
-Prints ONE JSON line.  The headline workload (`config.workload`) is the second of the benchmark
-configurations the repository's BASELINE.json lists: ReduceMaxOp_f32_f32 and ReduceSumOp_f32_f32
+Prints ONE JSON line.  The headline workload (`config.workload`) is the second of the five
+benchmark configurations of this path: ReduceMaxOp_f32_f32 and ReduceSumOp_f32_f32
 over axis 0 (column / two-pass split case) and over axis 1 of one [16384, 8192] float tensor; a
 "step" is those four op-kernel launches, `value` is the algorithmic bytes of a step divided by the
 step time, inputs resident in HBM.  The other listed configurations (row sum, fused softmax,
