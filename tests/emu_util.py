@@ -90,16 +90,21 @@ def _call(kind, tensors, blob, dtype):
         raise EmuFault(f"flash_attn_{kind}: rc {rc}: {msg}")
 
 
-def fwd(q, k, v, scale, window=(-1, -1), out=None):
+def _rng(rng_state):
+    """{seed, offset} as the two 64-bit words the calls read."""
+    to_i64 = lambda x: int(x) - (1 << 64) if int(x) >= (1 << 63) else int(x)
+    return torch.tensor([to_i64(rng_state[0]), to_i64(rng_state[1])] if rng_state else [0, 0], dtype=torch.int64)
+
+
+def fwd(q, k, v, scale, window=(-1, -1), out=None, p_dropout=0.0, rng_state=None):
     from byteir_amd import ops
     b, sq, h, d = q.shape
     o, lse = out if out is not None else (torch.empty_like(q), torch.empty((b, h, sq), dtype=torch.float32))
-    rng = torch.zeros(2, dtype=torch.int64)
-    _call("fwd", [q, k, v, rng, o, lse, None], ops.pack_flash_args(q, k, v, o, scale, window, 0.0), q.dtype)
+    _call("fwd", [q, k, v, _rng(rng_state), o, lse, None], ops.pack_flash_args(q, k, v, o, scale, window, p_dropout), q.dtype)
     return o, lse
 
 
-def bwd(do, q, k, v, o, lse, scale, window=(-1, -1), out=None):
+def bwd(do, q, k, v, o, lse, scale, window=(-1, -1), out=None, p_dropout=0.0, rng_state=None):
     from byteir_amd import ops
     b, sq, h, d = q.shape
     ru = lambda x, m: -(-x // m) * m
@@ -107,8 +112,7 @@ def bwd(do, q, k, v, o, lse, scale, window=(-1, -1), out=None):
         out = (torch.empty_like(q), torch.empty_like(k), torch.empty_like(v),
                torch.empty((b, h, ru(sq, 128)), dtype=torch.float32), torch.empty((b, ru(sq, 128), h, ru(d, 32)), dtype=torch.float32))
     dq, dk, dv, dsm, acc = out
-    rng = torch.zeros(2, dtype=torch.int64)
-    _call("bwd", [do, q, k, v, o, lse, rng, dq, dk, dv, dsm, acc], ops.pack_flash_args(q, k, v, o, scale, window, 0.0), q.dtype)
+    _call("bwd", [do, q, k, v, o, lse, _rng(rng_state), dq, dk, dv, dsm, acc], ops.pack_flash_args(q, k, v, o, scale, window, p_dropout), q.dtype)
     return dq, dk, dv
 
 

@@ -191,6 +191,39 @@ def test_results_do_not_depend_on_how_far_the_waves_run_apart(case):
         E.schedule(1, 0)
 
 
+@pytest.mark.parametrize("code", ["f16", "bf16"])
+@pytest.mark.parametrize("case", [
+    # b, sq, sk, h, h_k, d, window, p_dropout
+    (2, 128, 128, 2, 2, 64, (-1, 0), 0.1),
+    (1, 200, 333, 2, 2, 128, (-1, -1), 0.5),
+    (1, 130, 260, 4, 2, 96, (40, 30), 0.2),    # grouped heads: dropout streams are per query head
+])
+def test_emulated_dropout_is_the_reference_function_of_seed_offset_and_position(case, code):
+    """Dropout (Philox4x32-7 on (seed, offset, batch, head, 16 x 32 block), keep when the byte is
+    at most floor(255 p_keep)) against the oracle's thread-by-thread restatement: forward and
+    backward with the same rng_state."""
+    import oracle
+    b, sq, sk, h, hk, d, window, p_drop = case
+    ocode = oracle.F16 if code == "f16" else oracle.BF16
+    rng = np.random.default_rng(sum(case[:6]))
+    mk = lambda shape: oracle.from_f32(rng.standard_normal(shape).astype(np.float32), ocode)
+    q, k, v, do = mk((b, sq, h, d)), mk((b, sk, hk, d)), mk((b, sk, hk, d)), mk((b, sq, h, d))
+    to_t = lambda a: torch.from_numpy(a.view(np.int16).copy()).view(torch.bfloat16) if a.dtype == np.uint16 else torch.from_numpy(a.copy())
+    to_np = lambda t: t.view(torch.int16).numpy().view(np.uint16) if t.dtype == torch.bfloat16 else t.numpy()
+    state = (0x9E3779B97F4A7C15, 0x1_0000_0003)
+    scale = 1.0 / np.sqrt(d)
+    tq, tk, tv, tdo = to_t(q), to_t(k), to_t(v), to_t(do)
+    o, lse = E.fwd(tq, tk, tv, scale, window, p_dropout=p_drop, rng_state=state)
+    _, lse_ref, o32 = oracle.flash_fwd(q, k, v, scale, window, round_p=False, p_dropout=p_drop, rng_state=state)
+    assert np.abs(o.float().numpy() - o32).max() <= ATOL
+    seen = ~np.isposinf(lse_ref)
+    assert np.abs(lse.numpy()[seen] - lse_ref[seen]).max() <= 4e-3
+    dq, dk, dv = E.bwd(tdo, tq, tk, tv, o, lse, scale, window, p_dropout=p_drop, rng_state=state)
+    rq, rk, rv, _ = oracle.flash_bwd(do, q, k, v, to_np(o), lse.numpy(), scale, window, round_p=False, p_dropout=p_drop, rng_state=state)
+    for name, got, want in (("dq", dq, rq), ("dk", dk, rk), ("dv", dv, rv)):
+        assert np.abs(got.float().numpy() - oracle.to_f32(want)).max() <= ATOL, name
+
+
 def test_a_tensor_that_is_too_short_is_reported_with_the_workgroup_and_thread():
     """Negative controls: K one row short (a buffer load passes the descriptor's range check and
     then lies outside every tensor) and O one row short (a plain store runs into the protected
