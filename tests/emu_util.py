@@ -74,16 +74,17 @@ def guarded(shape, dtype, at_end=True):
 
 def _call(kind, tensors, blob, dtype):
     L = lib()
-    live = [t for t in tensors if t is not None]
-    for t in live:
-        L.fa_emu_register(_vp(t.data_ptr()), max(16, t.numel() * t.element_size()))
+    # the storage behind each tensor (a strided view addresses more than numel elements of it)
+    live = {t.untyped_storage().data_ptr(): t.untyped_storage().nbytes() for t in tensors if t is not None}
+    for p, n in live.items():
+        L.fa_emu_register(_vp(p), max(16, n))
     arr = (_vp * len(tensors))(*[t.data_ptr() if t is not None else None for t in tensors])
     buf = ctypes.create_string_buffer(blob, len(blob))
     try:
         rc = getattr(L, f"flash_attn_{kind}_checked")(arr, ctypes.cast(buf, _vp), 1 if dtype == torch.float16 else 2, None)
     finally:
-        for t in live:
-            L.fa_emu_unregister(_vp(t.data_ptr()))
+        for p in live:
+            L.fa_emu_unregister(_vp(p))
     if rc:
         msg = L.fa_emu_last_error().decode() if L.fa_emu_faulted() else L.flash_attn_last_error().decode()
         L.fa_emu_reset()
@@ -109,7 +110,9 @@ def bwd(do, q, k, v, o, lse, scale, window=(-1, -1), out=None, p_dropout=0.0, rn
     b, sq, h, d = q.shape
     ru = lambda x, m: -(-x // m) * m
     if out is None:
-        out = (torch.empty_like(q), torch.empty_like(k), torch.empty_like(v),
+        # dq, dk, dv are addressed with the strides of q, k, v (flash_api.cu:377-389)
+        like = lambda t: torch.empty_strided(t.shape, t.stride(), dtype=t.dtype)
+        out = (like(q), like(k), like(v),
                torch.empty((b, h, ru(sq, 128)), dtype=torch.float32), torch.empty((b, ru(sq, 128), h, ru(d, 32)), dtype=torch.float32))
     dq, dk, dv, dsm, acc = out
     _call("bwd", [do, q, k, v, o, lse, _rng(rng_state), dq, dk, dv, dsm, acc], ops.pack_flash_args(q, k, v, o, scale, window, p_dropout), q.dtype)

@@ -191,6 +191,40 @@ def test_results_do_not_depend_on_how_far_the_waves_run_apart(case):
         E.schedule(1, 0)
 
 
+@pytest.mark.parametrize("layout,case", [
+    ("packed_qkv", (2, 192, 192, 4, 4, 64, (-1, 0))),      # q, k, v are slices of one [b, s, 3, h, d] tensor
+    ("packed_qkv", (1, 130, 130, 2, 2, 96, (-1, -1))),
+    ("bhsd", (2, 160, 224, 4, 4, 128, (-1, 0))),           # [b, h, s, d] storage viewed as [b, s, h, d]
+    ("bhsd", (1, 100, 300, 3, 3, 32, (20, 5))),
+])
+def test_emulated_calls_follow_the_strides_of_their_tensors(layout, case):
+    """The blob carries batch, row and head strides: tensors that are views of larger ones."""
+    b, sq, sk, h, hk, d, window = case
+    dtype = torch.float16
+    gen = torch.Generator().manual_seed(sq + d)
+    q, k, v, do = randn((b, sq, h, d), dtype, gen), randn((b, sk, hk, d), dtype, gen), randn((b, sk, hk, d), dtype, gen), randn((b, sq, h, d), dtype, gen)
+    if layout == "packed_qkv":
+        pk = torch.empty((b, sq, 3, h, d), dtype=dtype)
+        pk[:, :, 0], pk[:, :, 1], pk[:, :, 2] = q, k, v
+        sq_, sk_, sv_ = pk[:, :, 0], pk[:, :, 1], pk[:, :, 2]
+        o_buf = torch.full((b, sq, 2, h, d), 7.0, dtype=dtype)
+        o_view = o_buf[:, :, 1]
+    else:
+        tr = lambda x: x.permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3)
+        sq_, sk_, sv_ = tr(q), tr(k), tr(v)
+        o_buf = torch.full((b, h, sq, d), 7.0, dtype=dtype)
+        o_view = o_buf.permute(0, 2, 1, 3)
+    scale = 1.0 / np.sqrt(d)
+    o, lse = E.fwd(sq_, sk_, sv_, scale, window, out=(o_view, torch.empty((b, h, sq), dtype=torch.float32)))
+    do_s = torch.empty_strided(o.shape, o.stride(), dtype=dtype).copy_(do)  # dO is addressed with the strides of O
+    dq, dk, dv = E.bwd(do_s, sq_, sk_, sv_, o, lse, scale, window)
+    o_ref, lse_ref, dq_ref, dk_ref, dv_ref = reference(q, k, v, do, scale, window)
+    for name, got, want in (("o", o, o_ref), ("dq", dq, dq_ref), ("dk", dk, dk_ref), ("dv", dv, dv_ref)):
+        assert float((got.float() - want).abs().max()) <= ATOL, (name, case)
+    if layout == "packed_qkv":
+        assert bool((o_buf[:, :, 0] == 7.0).all())  # the neighbouring slice of the output's storage is untouched
+
+
 @pytest.mark.parametrize("code", ["f16", "bf16"])
 @pytest.mark.parametrize("case", [
     # b, sq, sk, h, h_k, d, window, p_dropout
