@@ -33,6 +33,12 @@ def lib():
             f = getattr(L, f"flash_attn_{n}_checked")
             f.argtypes = [ctypes.POINTER(_vp), _vp, ctypes.c_int, _vp]
             f.restype = ctypes.c_int
+        for n in ("fwd", "bwd", "kvcache"):
+            getattr(L, f"flash_attn_{n}_ws").argtypes = [ctypes.POINTER(_vp), _vp, ctypes.c_int, _vp, ctypes.c_size_t, _vp]
+            getattr(L, f"flash_attn_{n}_workspace_bytes").restype = ctypes.c_size_t
+        L.flash_attn_fwd_workspace_bytes.argtypes = [_vp, ctypes.c_int]
+        L.flash_attn_kvcache_workspace_bytes.argtypes = [_vp, ctypes.c_int]
+        L.flash_attn_bwd_workspace_bytes.argtypes = [_vp, ctypes.c_int, ctypes.c_size_t]
         L.fa_emu_last_error.restype = ctypes.c_char_p
         L.flash_attn_last_error.restype = ctypes.c_char_p
         L.fa_emu_alloc.restype = _vp
@@ -72,16 +78,30 @@ def guarded(shape, dtype, at_end=True):
     return torch.frombuffer(buf, dtype=dtype, count=n).reshape(shape)
 
 
-def _call(kind, tensors, blob, dtype):
+def workspace_bytes(kind, blob, dtype, dq_accum_bytes=0):
+    """flash_attn_{fwd,bwd,kvcache}_workspace_bytes for an extra_args blob."""
+    L = lib()
+    buf = ctypes.create_string_buffer(blob, len(blob))
+    code = 1 if dtype == torch.float16 else 2
+    if kind == "bwd":
+        return L.flash_attn_bwd_workspace_bytes(ctypes.cast(buf, _vp), code, dq_accum_bytes)
+    return getattr(L, f"flash_attn_{kind}_workspace_bytes")(ctypes.cast(buf, _vp), code)
+
+
+def _call(kind, tensors, blob, dtype, workspace=None):
     L = lib()
     # the storage behind each tensor (a strided view addresses more than numel elements of it)
-    live = {t.untyped_storage().data_ptr(): t.untyped_storage().nbytes() for t in tensors if t is not None}
+    live = {t.untyped_storage().data_ptr(): t.untyped_storage().nbytes() for t in list(tensors) + [workspace] if t is not None}
     for p, n in live.items():
         L.fa_emu_register(_vp(p), max(16, n))
     arr = (_vp * len(tensors))(*[t.data_ptr() if t is not None else None for t in tensors])
     buf = ctypes.create_string_buffer(blob, len(blob))
     try:
-        rc = getattr(L, f"flash_attn_{kind}_checked")(arr, ctypes.cast(buf, _vp), 1 if dtype == torch.float16 else 2, None)
+        code = 1 if dtype == torch.float16 else 2
+        if workspace is not None:  # the caller's scratch (flash_attn_<kind>_ws)
+            rc = getattr(L, f"flash_attn_{kind}_ws")(arr, ctypes.cast(buf, _vp), code, workspace.data_ptr(), workspace.numel() * workspace.element_size(), None)
+        else:
+            rc = getattr(L, f"flash_attn_{kind}_checked")(arr, ctypes.cast(buf, _vp), code, None)
     finally:
         for p in live:
             L.fa_emu_unregister(_vp(p))

@@ -191,6 +191,40 @@ def test_results_do_not_depend_on_how_far_the_waves_run_apart(case):
         E.schedule(1, 0)
 
 
+def test_scratch_in_the_callers_workspace_gives_the_same_bits():
+    """The key-axis split of the forward (few query blocks, many keys) and the partial dK / dV of
+    a shared-out head group, with the scratch in a guarded, poisoned workspace of exactly the
+    size the *_workspace_bytes query names, against the calls that take their own scratch;
+    the backward also without any dq_accum to borrow from."""
+    from byteir_amd import ops
+    bits = lambda t: t.view(torch.int16 if t.element_size() == 2 else torch.int32)
+    dtype = torch.bfloat16
+    gen = torch.Generator().manual_seed(4)
+    q, k, v = randn((1, 64, 2, 64), dtype, gen), randn((1, 1100, 2, 64), dtype, gen), randn((1, 1100, 2, 64), dtype, gen)
+    o, lse, rng = torch.empty_like(q), torch.empty((1, 2, 64), dtype=torch.float32), torch.zeros(2, dtype=torch.int64)
+    blob = ops.pack_flash_args(q, k, v, o, 0.125, (-1, 0), 0.0)
+    need = E.workspace_bytes("fwd", blob, dtype)
+    assert need > 0
+    ws = E.guarded((need,), torch.uint8).fill_(0xFF)
+    o0, l0 = E.fwd(q, k, v, 0.125, (-1, 0))
+    E._call("fwd", [q, k, v, rng, o, lse, None], blob, dtype, workspace=ws)
+    assert torch.equal(bits(o0), bits(o)) and torch.equal(l0, lse)
+    # backward, eight query heads on two key/value heads: the group is shared out over workgroups
+    b, s_, h, hk, d = 1, 300, 8, 2, 64
+    q, k, v, do = randn((b, s_, h, d), dtype, gen), randn((b, s_, hk, d), dtype, gen), randn((b, s_, hk, d), dtype, gen), randn((b, s_, h, d), dtype, gen)
+    o, lse = E.fwd(q, k, v, 0.125, (-1, 0))
+    g0 = E.bwd(do, q, k, v, o, lse, 0.125, (-1, 0))  # partials in dq_accum
+    blob = ops.pack_flash_args(q, k, v, o, 0.125, (-1, 0), 0.0)
+    need = E.workspace_bytes("bwd", blob, dtype, 0)
+    assert need > 0 and E.workspace_bytes("bwd", blob, dtype, 1 << 30) == 0
+    like = lambda t: torch.empty_strided(t.shape, t.stride(), dtype=t.dtype)
+    for ws in (E.guarded((need,), torch.uint8).fill_(0xFF), None):  # the caller's workspace; the library's own allocation
+        dq, dk, dv, dsm = like(q), like(k), like(v), torch.empty((b, h, 384), dtype=torch.float32)
+        E._call("bwd", [do, q, k, v, o, lse, rng, dq, dk, dv, dsm, None], blob, dtype, workspace=ws)
+        for a, c in zip(g0, (dq, dk, dv)):
+            assert torch.equal(bits(a), bits(c))
+
+
 @pytest.mark.parametrize("layout,case", [
     ("packed_qkv", (2, 192, 192, 4, 4, 64, (-1, 0))),      # q, k, v are slices of one [b, s, 3, h, d] tensor
     ("packed_qkv", (1, 130, 130, 2, 2, 96, (-1, -1))),
