@@ -70,6 +70,8 @@ def guarded(shape, dtype, at_end=True):
     byte is the first behind one.  Lives until the process ends."""
     L = lib()
     n = int(np.prod(shape))
+    if n == 0:
+        return torch.empty(shape, dtype=dtype)  # no bytes: nothing to guard (its data pointer is null)
     nbytes = n * torch.empty(0, dtype=dtype).element_size()
     p = L.fa_emu_alloc(max(nbytes, 16), 1 if at_end else 0)
     if not p:

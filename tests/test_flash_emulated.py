@@ -191,6 +191,29 @@ def test_results_do_not_depend_on_how_far_the_waves_run_apart(case):
         E.schedule(1, 0)
 
 
+@pytest.mark.parametrize("d", [64, 80, 128])
+def test_emulated_calls_without_keys_or_without_queries(d):
+    """seqlen_k = 0: O = 0, LSE = +inf, dQ = 0 (flash_fwd_kernel.h:70-104); seqlen_q = 0: nothing
+    to write forward, dK = dV = 0.  Guarded tensors: the empty side has no bytes to touch."""
+    b, h, dtype = 2, 4, torch.float16
+    gen = torch.Generator().manual_seed(d)
+    G = lambda s, t=dtype: E.guarded(s, t)
+    for sq in (3, 200):
+        q, do = G((b, sq, h, d)).copy_(randn((b, sq, h, d), dtype, gen)), G((b, sq, h, d)).copy_(randn((b, sq, h, d), dtype, gen))
+        k, v = G((b, 0, h, d)), G((b, 0, h, d))
+        o, lse = E.fwd(q, k, v, 0.3, (-1, -1), out=(G(q.shape).fill_(7.0), G((b, h, sq), torch.float32)))
+        assert bool((o == 0).all()) and bool(torch.isposinf(lse).all())
+        dq, dk, dv = E.bwd(do, q, k, v, o, lse, 0.3, (-1, -1))
+        assert bool((dq == 0).all()) and dk.numel() == 0 and dv.numel() == 0
+    sk = 150
+    q, do = G((b, 0, h, d)), G((b, 0, h, d))
+    k, v = G((b, sk, h, d)).copy_(randn((b, sk, h, d), dtype, gen)), G((b, sk, h, d)).copy_(randn((b, sk, h, d), dtype, gen))
+    o, lse = E.fwd(q, k, v, 0.3, (-1, 0), out=(G(q.shape), G((b, h, 0), torch.float32)))
+    out = (G(q.shape), G(k.shape).fill_(7.0), G(v.shape).fill_(7.0), G((b, h, 0), torch.float32), G((b, 0, h, d), torch.float32))
+    dq, dk, dv = E.bwd(do, q, k, v, o, lse, 0.3, (-1, 0), out=out)
+    assert dq.numel() == 0 and bool((dk == 0).all()) and bool((dv == 0).all())
+
+
 def test_scratch_in_the_callers_workspace_gives_the_same_bits():
     """The key-axis split of the forward (few query blocks, many keys) and the partial dK / dV of
     a shared-out head group, with the scratch in a guarded, poisoned workspace of exactly the
