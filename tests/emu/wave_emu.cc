@@ -308,12 +308,12 @@ void tr_fn(const void *const *in, void *const *out, int n, void *) {
   }
 }
 
-void ballot_fn(const void *const *in, void *const *out, int n, void *) {
+// (ballot and readfirstlane clear the slots before they meet, so a lane that has exited has a null
+// slot: its bit stays clear, and the first live lane is the first non-null one)
+void ballot_fn(const void *const *in, void *const *out, int, void *) {
   uint64_t m = 0;
-  // slots are lane ids only when the wave is whole; with exited lanes their bits stay clear
   for (int l = 0; l < kWave; ++l)
-    if (in[l] && l < kWave) m |= (uint64_t)(*static_cast<const bool *>(in[l]) ? 1 : 0) << l;
-  (void)n;
+    if (in[l] && *static_cast<const bool *>(in[l])) m |= uint64_t(1) << l;
   for (int l = 0; l < kWave; ++l)
     if (out[l]) *static_cast<uint64_t *>(out[l]) = m;
 }

@@ -16,6 +16,9 @@
 // What it is not: a timing model, or a model of anything the hardware does that the ISA
 // documents leave open (it rounds an MFMA once from a double accumulation).
 //
+// One launch at a time, from one thread: the scheduler's state is global.  A stray access is
+// caught by a SIGSEGV handler that leaves the faulting lane through setcontext (Linux).
+//
 // All lanes of a wave must reach the same cross-lane operations in the same order (true for
 // these kernels: their divergent branches contain none); a mismatch or a deadlock is detected
 // and reported, not silently mis-executed.
